@@ -1,0 +1,320 @@
+"""The cache manager: pages for keys and values, a block table per request and
+group, and numbered slots for per-request state of fixed size.
+
+A step is a transaction, as in the reference (miniserve/kv/manager.py:119-192,
+kv/paged.py:59-104): ``prepare_step`` reserves the missing pages tentatively and
+computes the slot of every new token, ``commit_step`` makes them part of the
+tables and advances the committed lengths, ``abort_step`` gives exactly the
+step's new pages back.  Beyond the reference: groups of calls with different
+needs have pools, allocators and tables of their own; a group with a window gives
+pages back as soon as no later position can read them; every live request holds a
+numbered state slot.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Mapping, Sequence
+
+from ..parts.base import KVCacheView, StateView
+from .allocator import OutOfPagesError, PageAllocator
+from .layout import CacheLayout
+from .table import BlockTable
+
+
+class CacheError(RuntimeError):
+    pass
+
+
+@dataclass(frozen=True)
+class CapacitySnapshot:
+    """What the scheduler may know: numbers only (reference: miniserve/kv/base.py:14-36)."""
+
+    block_size: int
+    total_blocks: tuple[int, ...]      # per group
+    free_blocks: tuple[int, ...]       # per group
+    free_slots: int
+    total_slots: int
+    held_blocks: Mapping[str, tuple[int, ...]] = field(default_factory=dict)   # per live request, per group
+
+    def pages_for(self, before: int, after: int) -> int:
+        """New pages that growing a request from ``before`` to ``after`` tokens takes in every group."""
+
+        return -(-after // self.block_size) - -(-before // self.block_size)
+
+    @property
+    def min_free_blocks(self) -> int:
+        return min(self.free_blocks) if self.free_blocks else 1 << 60
+
+
+@dataclass(frozen=True)
+class StepItem:
+    request_id: str
+    start: int        # first new position = tokens already committed
+    end: int          # length after the step
+
+
+@dataclass
+class SequenceStepMeta:
+    """One request's share of a prepared step."""
+
+    request_id: str
+    state_slot: int
+    before: int
+    after: int
+    block_tables: list[tuple[int, ...]]     # per group, committed + tentative pages
+    slot_mappings: list[tuple[int, ...]]    # per group, one slot per new token
+    new_pages: list[list[int]]              # per group
+
+
+@dataclass
+class StepReservation:
+    step_id: int
+    sequences: list[SequenceStepMeta] = field(default_factory=list)
+    closed: bool = False
+
+
+@dataclass
+class _Live:
+    request_id: str
+    state_slot: int
+    committed: int = 0
+    tables: list[BlockTable] = field(default_factory=list)
+    pending: bool = False
+
+
+class CacheManager:
+    def __init__(
+        self,
+        layout: CacheLayout,
+        *,
+        block_size: int,
+        num_blocks: int | Sequence[int],
+        max_num_seqs: int,
+        max_model_len: int,
+    ) -> None:
+        if block_size <= 0 or max_num_seqs <= 0 or max_model_len <= 0:
+            raise ValueError("block_size, max_num_seqs and max_model_len must be positive.")
+        self.layout = layout
+        self.block_size = block_size
+        counts = [num_blocks] * len(layout.groups) if isinstance(num_blocks, int) else list(num_blocks)
+        if len(counts) != len(layout.groups):
+            raise ValueError("num_blocks must give one count per cache group.")
+        self.num_blocks = tuple(counts)
+        self.max_num_seqs = max_num_seqs
+        self.max_model_len = max_model_len
+        self.allocators = [PageAllocator(count) for count in counts]
+        self._free_slots = list(range(max_num_seqs - 1, -1, -1))   # pop() gives the lowest
+        self._live: dict[str, _Live] = {}
+        self._next_step_id = 0
+        self._open: StepReservation | None = None
+        # storage, attached by allocate_storage()
+        self.key_pools: list = []
+        self.value_pools: list = []
+        self.state_tensors: list = []
+
+    # ---- storage --------------------------------------------------------------------
+    def allocate_storage(self, dtype, device) -> None:
+        """Pools ``[calls, pages, kv_heads, block_size, head_dim]`` per group, allocated
+        once and never initialised (a page's content is read only below the
+        committed length; reference: miniserve/kv/paged.py:39-41), and zeroed
+        state tensors ``[slots, *shape]``."""
+
+        import torch
+
+        self.key_pools, self.value_pools, self.state_tensors = [], [], []
+        for group, count in zip(self.layout.groups, self.num_blocks):
+            shape = (len(group.calls), count, group.need.num_kv_heads, self.block_size, group.need.head_dim)
+            self.key_pools.append(torch.empty(shape, dtype=dtype, device=device))
+            self.value_pools.append(torch.empty(shape, dtype=dtype, device=device))
+        for need in self.layout.states:
+            self.state_tensors.append(torch.zeros((self.max_num_seqs, *need.shape), dtype=need.dtype, device=device))
+
+    def call_views(self) -> list:
+        """The cache of every call of the run order: ``KVCacheView``, ``StateView`` or None."""
+
+        views = []
+        for placement in self.layout.placements:
+            if placement.kind == "kv":
+                views.append(
+                    KVCacheView(
+                        group=placement.group,
+                        key=self.key_pools[placement.group][placement.index],
+                        value=self.value_pools[placement.group][placement.index],
+                        block_size=self.block_size,
+                        write=placement.write,
+                    )
+                )
+            elif placement.kind == "state":
+                views.append(StateView(self.state_tensors[placement.index]))
+            else:
+                views.append(None)
+        return views
+
+    # ---- admission and release --------------------------------------------------------
+    def admit(self, request_id: str) -> int:
+        """Give ``request_id`` a state slot and empty tables; returns the slot."""
+
+        if request_id in self._live:
+            raise CacheError(f"request {request_id!r} is already live.")
+        if not self._free_slots:
+            raise CacheError("NO_FREE_SLOT: every state slot is taken.")
+        slot = self._free_slots.pop()
+        self._live[request_id] = _Live(
+            request_id, slot, tables=[BlockTable(self.block_size) for _ in self.layout.groups]
+        )
+        for tensor in self.state_tensors:
+            tensor[slot].zero_()
+        return slot
+
+    def release(self, request_id: str) -> None:
+        """Give back everything the request holds: its pages of every group and its slot."""
+
+        live = self._live.get(request_id)
+        if live is None:
+            raise CacheError(f"request {request_id!r} is not live.")
+        if live.pending:
+            raise CacheError(f"request {request_id!r} is part of an open step.")
+        for allocator, table in zip(self.allocators, live.tables):
+            pages = table.live_pages()
+            if pages:
+                allocator.release(pages)
+        self._free_slots.append(live.state_slot)
+        self._free_slots.sort(reverse=True)
+        del self._live[request_id]
+
+    def is_live(self, request_id: str) -> bool:
+        return request_id in self._live
+
+    def live_requests(self) -> tuple[str, ...]:
+        return tuple(self._live)
+
+    def committed_tokens(self, request_id: str) -> int:
+        return self._live[request_id].committed
+
+    def state_slot(self, request_id: str) -> int:
+        return self._live[request_id].state_slot
+
+    def block_table(self, request_id: str, group: int = 0) -> tuple[int, ...]:
+        return self._live[request_id].tables[group].snapshot()
+
+    # ---- the step transaction ---------------------------------------------------------
+    def prepare_step(self, items: Sequence[StepItem]) -> StepReservation:
+        if self._open is not None:
+            raise CacheError("a step is already open; commit or abort it first.")
+        seen: set[str] = set()
+        for item in items:
+            live = self._live.get(item.request_id)
+            if live is None:
+                raise CacheError(f"request {item.request_id!r} is not live.")
+            if item.request_id in seen:
+                raise CacheError(f"request {item.request_id!r} appears twice in one step.")
+            seen.add(item.request_id)
+            if item.start != live.committed:
+                raise CacheError(
+                    f"request {item.request_id!r}: the step starts at {item.start}, {live.committed} tokens are committed."
+                )
+            if item.end <= item.start or item.end > self.max_model_len:
+                raise CacheError(f"request {item.request_id!r}: the step ends at {item.end} (limit {self.max_model_len}).")
+        reservation = StepReservation(self._next_step_id)
+        self._next_step_id += 1
+        taken: list[tuple[int, list[int]]] = []
+        try:
+            for item in items:
+                live = self._live[item.request_id]
+                meta = SequenceStepMeta(item.request_id, live.state_slot, item.start, item.end, [], [], [])
+                for index, (allocator, table) in enumerate(zip(self.allocators, live.tables)):
+                    missing = table.required_blocks(item.end) - len(table.physical_block_ids)
+                    new_pages = allocator.allocate(max(missing, 0))
+                    taken.append((index, new_pages))
+                    tentative = table.physical_block_ids + new_pages
+                    slots = []
+                    for position in range(item.start, item.end):
+                        logical, offset = divmod(position, self.block_size)
+                        slots.append(tentative[logical] * self.block_size + offset)
+                    meta.block_tables.append(tuple(tentative))
+                    meta.slot_mappings.append(tuple(slots))
+                    meta.new_pages.append(new_pages)
+                reservation.sequences.append(meta)
+        except OutOfPagesError:
+            for index, pages in taken:
+                if pages:
+                    self.allocators[index].release(pages)
+            raise
+        for item in items:
+            self._live[item.request_id].pending = True
+        self._open = reservation
+        return reservation
+
+    def commit_step(self, reservation: StepReservation) -> None:
+        self._close(reservation)
+        for meta in reservation.sequences:
+            live = self._live[meta.request_id]
+            for group, table, pages in zip(self.layout.groups, live.tables, meta.new_pages):
+                table.append_blocks(pages)
+            live.committed = meta.after
+            live.pending = False
+            self._give_back_passed_pages(live)
+
+    def abort_step(self, reservation: StepReservation) -> None:
+        self._close(reservation)
+        for meta in reservation.sequences:
+            for allocator, pages in zip(self.allocators, meta.new_pages):
+                if pages:
+                    allocator.release(pages)
+            self._live[meta.request_id].pending = False
+
+    def _close(self, reservation: StepReservation) -> None:
+        if reservation.closed or self._open is not reservation:
+            raise CacheError("this step is not the open one (a step id can be used once).")
+        reservation.closed = True
+        self._open = None
+
+    def _give_back_passed_pages(self, live: _Live) -> None:
+        """With ``n`` tokens committed the next query stands at ``n`` or later and
+        reads keys ``>= n - window + 1``; pages wholly below that go back."""
+
+        for group, allocator, table in zip(self.layout.groups, self.allocators, live.tables):
+            if group.window is None:
+                continue
+            pages = table.give_back_before(live.committed - group.window + 1)
+            if pages:
+                allocator.release(pages)
+
+    # ---- accounting -------------------------------------------------------------------
+    def capacity(self) -> CapacitySnapshot:
+        return CapacitySnapshot(
+            block_size=self.block_size,
+            total_blocks=self.num_blocks,
+            free_blocks=tuple(allocator.free_count() for allocator in self.allocators),
+            free_slots=len(self._free_slots),
+            total_slots=self.max_num_seqs,
+            held_blocks={
+                request_id: tuple(len(table.live_pages()) for table in live.tables)
+                for request_id, live in self._live.items()
+            },
+        )
+
+    def assert_invariants(self) -> None:
+        """No page is lost or held twice: per group, the pages of all tables, the
+        open step's tentative pages and the free list are disjoint and add up."""
+
+        for index, allocator in enumerate(self.allocators):
+            allocator.assert_invariants()
+            held: list[int] = []
+            for live in self._live.values():
+                held.extend(live.tables[index].live_pages())
+            if self._open is not None:
+                for meta in self._open.sequences:
+                    held.extend(meta.new_pages[index])
+            if len(held) != len(set(held)):
+                raise AssertionError(f"group {index}: a page is held twice.")
+            if set(held) & set(allocator.free_ids()):
+                raise AssertionError(f"group {index}: a held page is on the free list.")
+            if len(held) + allocator.free_count() != allocator.num_pages:
+                raise AssertionError(f"group {index}: pages are lost ({len(held)} held, {allocator.free_count()} free).")
+        slots = [live.state_slot for live in self._live.values()]
+        if len(slots) != len(set(slots)) or set(slots) & set(self._free_slots):
+            raise AssertionError("a state slot is held twice.")
+        if len(slots) + len(self._free_slots) != self.max_num_seqs:
+            raise AssertionError("state slots are lost.")

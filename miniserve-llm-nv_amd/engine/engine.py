@@ -1,0 +1,223 @@
+"""The engine: requests in, tokens out.  ``add_request`` admits, ``step`` runs one
+scheduled batch through the step function and samples, ``generate`` loops until
+every request has finished (reference: miniserve/engine/core.py:193-265 submit,
+:278-439 the step, :568-591 the synchronous loop).
+"""
+
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass
+from typing import Callable, Sequence
+
+from ..sampling import Sampler
+from .batch import StepEntry
+from .plan import ExecutionPlan
+from .request import Request, SamplingParams
+from .scheduler import Scheduler
+from .sequence import TERMINAL, RequestStatus, SequenceState
+
+
+@dataclass(frozen=True)
+class StepOutput:
+    """A token that a step produced for a request, and whether the request ended with it."""
+
+    request_id: str
+    token_id: int
+    finished: bool
+    finish_reason: str | None
+
+
+@dataclass(frozen=True)
+class GenerationResult:
+    request_id: str
+    prompt_token_ids: tuple[int, ...]
+    token_ids: tuple[int, ...]
+    finish_reason: str | None
+    num_preemptions: int = 0
+
+
+class Engine:
+    """``runner`` offers ``step(entries) -> logits``, ``admit``, ``release``,
+    ``cache.capacity()``, ``spec``, ``max_model_len``, ``block_size`` and
+    ``engine_config`` (the ``ModelRunner``; tests may pass a stand-in)."""
+
+    def __init__(self, runner, *, sampler=None, clock_ns: Callable[[], int] = time.monotonic_ns) -> None:
+        self.runner = runner
+        config = runner.engine_config
+        max_positions = runner.spec.max_positions
+        self.max_model_len = runner.max_model_len
+        self.max_num_batched_tokens = config.resolved_max_num_batched_tokens(max_positions)
+        self.enable_chunked_prefill = config.enable_chunked_prefill
+        self.max_pending_requests = config.max_pending_requests
+        self.vocab_size = runner.spec.vocab_size
+        self.scheduler = Scheduler(
+            max_num_seqs=config.max_num_seqs,
+            max_num_batched_tokens=self.max_num_batched_tokens,
+            enable_chunked_prefill=config.enable_chunked_prefill,
+            prefill_chunk_size=config.prefill_chunk_size,
+        )
+        self.sampler = sampler if sampler is not None else Sampler()
+        self._clock_ns = clock_ns
+        self._sequences: dict[str, SequenceState] = {}
+        self._results: dict[str, GenerationResult] = {}
+        self.last_plan: ExecutionPlan | None = None
+        self.counters = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0, "empty_plans": 0}
+
+    # ---- admission --------------------------------------------------------------------
+    def add_request(
+        self,
+        request_id: str,
+        prompt_token_ids: Sequence[int],
+        sampling_params: SamplingParams | None = None,
+        *,
+        arrival_ns: int | None = None,
+    ) -> None:
+        """Checks of the reference's ``submit`` (core.py:193-236), before any state exists."""
+
+        params = sampling_params if sampling_params is not None else SamplingParams()
+        request = Request(
+            request_id,
+            tuple(prompt_token_ids),
+            params,
+            self._clock_ns() if arrival_ns is None else arrival_ns,
+        )
+        if request_id in self._sequences or request_id in self._results:
+            raise ValueError(f"Duplicate request_id: {request_id}")
+        active = sum(1 for state in self._sequences.values() if state.status not in TERMINAL)
+        if active >= self.max_pending_requests:
+            raise RuntimeError("QUEUE_FULL: max_pending_requests reached.")
+        total = len(request.prompt_token_ids) + params.max_new_tokens
+        if total > self.max_model_len:
+            raise ValueError(
+                f"CONTEXT_LENGTH_EXCEEDED: prompt {len(request.prompt_token_ids)} + max_new_tokens "
+                f"{params.max_new_tokens} exceeds max_model_len {self.max_model_len}."
+            )
+        capacity = self.runner.cache.capacity()
+        if capacity.pages_for(0, total) > min(capacity.total_blocks, default=1 << 60):
+            raise ValueError("CONTEXT_CAPACITY_EXCEEDED: the request alone needs more pages than the pool holds.")
+        if any(token >= self.vocab_size for token in request.prompt_token_ids):
+            raise ValueError("prompt token id is outside the vocabulary.")
+        if params.top_k > self.vocab_size:
+            raise ValueError("top_k must not exceed the vocabulary size.")
+        if any(token >= self.vocab_size for token in params.stop_token_ids):
+            raise ValueError("stop token id is outside the vocabulary.")
+        if not self.enable_chunked_prefill and total - 1 > self.max_num_batched_tokens:
+            # without portions, a preempted request must be able to run all its tokens in one step
+            raise ValueError(
+                "CHUNKED_PREFILL_DISABLED: the request does not fit max_num_batched_tokens in one step; "
+                "enable chunked prefill."
+            )
+        self._sequences[request_id] = SequenceState.from_request(request)
+
+    def cancel(self, request_id: str) -> None:
+        state = self._sequences[request_id]
+        state.cancel()
+        self._finalize(state)
+
+    def has_unfinished(self) -> bool:
+        return bool(self._sequences)
+
+    # ---- one step ---------------------------------------------------------------------
+    def step(self) -> list[StepOutput]:
+        views = [state.snapshot() for state in self._sequences.values()]
+        plan = self.scheduler.schedule(views, self.runner.cache.capacity())
+        self.last_plan = plan
+        for request_id in plan.preempted:
+            self.runner.release(request_id)
+            self._sequences[request_id].preempt()
+            self.counters["preemptions"] += 1
+        if plan.empty:
+            self.counters["empty_plans"] += 1
+            return []
+
+        entries: list[StepEntry] = []
+        sampled: list[SequenceState] = []
+        for item in plan.decode_items:
+            entries.append(StepEntry(item.request_id, (item.input_token_id,), (0,)))
+            sampled.append(self._sequences[item.request_id])
+        for item in plan.prefill_items:
+            state = self._sequences[item.request_id]
+            if state.status is RequestStatus.WAITING:
+                self.runner.admit(item.request_id)
+                state.begin_prefill()
+            tokens = state.all_tokens[item.token_start : item.token_end]
+            final = item.token_end == state.prefill_target
+            entries.append(StepEntry(item.request_id, tuple(tokens), (len(tokens) - 1,) if final else ()))
+            if final:
+                sampled.append(state)
+
+        try:
+            logits = self.runner.step(entries)
+            staged = ()
+            if sampled:
+                staged = self.sampler.stage(logits, [(s.request_id, s.sampling_params) for s in sampled])
+        except Exception as exc:
+            # the step left no trace in the cache; its requests fail (reference: core.py:396-406)
+            for entry in entries:
+                state = self._sequences[entry.request_id]
+                state.fail(f"{type(exc).__name__}: {exc}")
+                self._finalize(state)
+            raise
+        self.sampler.commit(staged)
+
+        self.counters["steps"] += 1
+        self.counters["decode_tokens"] += len(plan.decode_items)
+        self.counters["prefill_tokens"] += plan.scheduled_tokens - len(plan.decode_items)
+        for item in plan.decode_items:
+            self._sequences[item.request_id].mark_decode_input_computed()
+        for item in plan.prefill_items:
+            self._sequences[item.request_id].commit_prefill(item.token_end)
+        outputs: list[StepOutput] = []
+        for state, sample in zip(sampled, staged):
+            state.append_sampled_token(sample.token_id)
+            reason = state.should_finish()
+            if reason is not None:
+                state.finish(reason)
+                self._finalize(state)
+            outputs.append(StepOutput(state.request_id, sample.token_id, reason is not None, reason))
+        return outputs
+
+    def _finalize(self, state: SequenceState) -> None:
+        """A request that ended gives back its pages, its state slot and its random stream."""
+
+        if self.runner.cache.is_live(state.request_id):
+            self.runner.release(state.request_id)
+        self.sampler.release(state.request_id)
+        self._results[state.request_id] = GenerationResult(
+            state.request_id,
+            state.prompt_token_ids,
+            tuple(state.generated_token_ids),
+            state.finish_reason,
+            state.num_preemptions,
+        )
+        del self._sequences[state.request_id]
+
+    def pop_result(self, request_id: str) -> GenerationResult:
+        return self._results.pop(request_id)
+
+    # ---- the synchronous loop ---------------------------------------------------------
+    def generate(
+        self,
+        prompts: Sequence[Sequence[int]],
+        sampling_params: SamplingParams | Sequence[SamplingParams] | None = None,
+    ) -> list[list[int]]:
+        """Token ids in, generated token ids out, one list per prompt."""
+
+        if isinstance(sampling_params, SamplingParams) or sampling_params is None:
+            params = [sampling_params or SamplingParams()] * len(prompts)
+        else:
+            params = list(sampling_params)
+            if len(params) != len(prompts):
+                raise ValueError("one SamplingParams per prompt is needed.")
+        base = len(self._results) + len(self._sequences)
+        request_ids = [f"generate-{base + index}" for index in range(len(prompts))]
+        for index, (request_id, prompt, p) in enumerate(zip(request_ids, prompts, params)):
+            self.add_request(request_id, prompt, p, arrival_ns=index)
+        idle = 0
+        while any(request_id in self._sequences for request_id in request_ids):
+            produced = self.step()
+            idle = 0 if (produced or not self.last_plan.empty) else idle + 1
+            if idle > 2:
+                raise RuntimeError("the scheduler made no progress: no request fits the cache.")
+        return [list(self.pop_result(request_id).token_ids) for request_id in request_ids]

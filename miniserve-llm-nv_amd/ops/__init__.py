@@ -1,0 +1,297 @@
+"""Python face of the HIP kernels: one function per kernel, each checking on the
+host that the operands have the shapes, types and layout that the kernel and its
+grid assume, before anything is launched.  Tensors are torch tensors on the GPU;
+torch is the allocator and gives the stream.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .library import KernelError, call, library_path, load
+
+__all__ = [
+    "KernelError",
+    "attention",
+    "embedding_gather",
+    "library_path",
+    "linear",
+    "load",
+    "qk_norm_rope_append",
+    "residual_add",
+    "rmsnorm",
+    "sample_rows",
+    "silu_mul",
+]
+
+_DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODES[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16 storage, not {dtype}.") from None
+
+
+def _check(tensor: torch.Tensor, name: str, *, dtype: torch.dtype | None = None, shape: tuple | None = None) -> None:
+    if not isinstance(tensor, torch.Tensor):
+        raise KernelError(f"{name} must be a tensor.")
+    if not tensor.is_cuda:
+        raise KernelError(f"{name} must live on the GPU (got {tensor.device}); there is no CPU path.")
+    if not tensor.is_contiguous():
+        raise KernelError(f"{name} must be contiguous.")
+    if dtype is not None and tensor.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, not {tensor.dtype}.")
+    if shape is not None and tuple(tensor.shape) != tuple(shape):
+        raise KernelError(f"{name} must have shape {tuple(shape)}, not {tuple(tensor.shape)}.")
+
+
+def _ptr(tensor: torch.Tensor | None) -> int | None:
+    return None if tensor is None else tensor.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def embedding_gather(token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """``out[t] = table[token_ids[t]]`` as float32 ``[N, hidden]`` (the residual stream)."""
+
+    _check(token_ids, "token_ids", dtype=torch.int32)
+    _check(table, "table")
+    if token_ids.ndim != 1 or table.ndim != 2 or token_ids.numel() == 0:
+        raise KernelError("embedding_gather takes token_ids [N>0] and table [vocab, hidden].")
+    vocab, hidden = table.shape
+    out = torch.empty((token_ids.numel(), hidden), dtype=torch.float32, device=table.device)
+    call("ms_embedding_gather", _ptr(token_ids), _ptr(table), _ptr(out), token_ids.numel(), hidden, vocab,
+         _code(table.dtype), _stream())
+    return out
+
+
+def rmsnorm(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    eps: float,
+    *,
+    delta: torch.Tensor | None = None,
+    rows: torch.Tensor | None = None,
+    write_back: bool = False,
+) -> torch.Tensor:
+    """RMSNorm over the last dimension of ``x [n, dim]``.
+
+    ``x`` is float32 (the residual stream) or of the weight's type.  With
+    ``delta`` the norm is taken of ``x + delta``; ``write_back`` stores that sum
+    into ``x``.  With ``rows`` (int32) output row ``r`` reads input row
+    ``rows[r]``.  The output has the weight's type."""
+
+    _check(weight, "weight")
+    _check(x, "x")
+    if x.ndim != 2 or weight.ndim != 1 or x.shape[1] != weight.numel():
+        raise KernelError(f"rmsnorm: x {tuple(x.shape)} does not match weight {tuple(weight.shape)}.")
+    if x.dtype != torch.float32 and x.dtype != weight.dtype:
+        raise KernelError("rmsnorm: x must be float32 or of the weight's type.")
+    n_in, dim = x.shape
+    if delta is not None:
+        _check(delta, "delta", dtype=weight.dtype, shape=(n_in, dim))
+    if rows is not None:
+        _check(rows, "rows", dtype=torch.int32)
+        if rows.ndim != 1:
+            raise KernelError("rmsnorm: rows must be one-dimensional.")
+    n_out = n_in if rows is None else rows.numel()
+    if n_out == 0:
+        raise KernelError("rmsnorm: no rows.")
+    out = torch.empty((n_out, dim), dtype=weight.dtype, device=x.device)
+    call("ms_rmsnorm", _ptr(x), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), n_out, dim, float(eps),
+         int(x.dtype == torch.float32), int(write_back), _code(weight.dtype), _stream())
+    return out
+
+
+def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
+    """``h += delta`` with ``h`` float32."""
+
+    _check(h, "h", dtype=torch.float32)
+    _check(delta, "delta", shape=tuple(h.shape))
+    if h.ndim != 2 or h.numel() == 0:
+        raise KernelError("residual_add takes h [n>0, dim>0].")
+    call("ms_residual_add", _ptr(h), _ptr(delta), h.shape[0], h.shape[1], _code(delta.dtype), _stream())
+
+
+def qk_norm_rope_append(
+    packed: torch.Tensor,
+    *,
+    num_q_heads: int,
+    num_kv_heads: int,
+    head_dim: int,
+    q_weight: torch.Tensor | None,
+    k_weight: torch.Tensor | None,
+    eps: float,
+    inv_freq: torch.Tensor | None,
+    positions: torch.Tensor | None,
+    slot_mapping: torch.Tensor | None = None,
+    key_pool: torch.Tensor | None = None,
+    value_pool: torch.Tensor | None = None,
+) -> torch.Tensor | None:
+    """Per-head norm of q and k, rotation, and the cache write, in one kernel.
+
+    ``packed [N, (num_q_heads + 2*num_kv_heads) * head_dim]`` holds q heads, then
+    k heads, then v heads.  Returns q ``[N, num_q_heads, head_dim]`` (None when
+    there are no q heads); k and v go to ``pool[page, kv_head, offset]`` with
+    ``slot = page * block_size + offset`` from ``slot_mapping`` (int32)."""
+
+    _check(packed, "packed")
+    heads = num_q_heads + 2 * num_kv_heads
+    if packed.ndim != 2 or packed.shape[1] != heads * head_dim or packed.shape[0] == 0:
+        raise KernelError(
+            f"qk_norm_rope_append: packed {tuple(packed.shape)} is not [N, {heads} * {head_dim}]."
+        )
+    n = packed.shape[0]
+    dtype = packed.dtype
+    for name, weight in (("q_weight", q_weight), ("k_weight", k_weight)):
+        if weight is not None:
+            _check(weight, name, dtype=dtype, shape=(head_dim,))
+    if inv_freq is not None:
+        _check(inv_freq, "inv_freq", dtype=torch.float32, shape=(head_dim // 2,))
+        if positions is None:
+            raise KernelError("qk_norm_rope_append: rotation needs positions.")
+    if positions is not None:
+        _check(positions, "positions", dtype=torch.int32, shape=(n,))
+    block_size = 0
+    if num_kv_heads > 0:
+        if slot_mapping is None or key_pool is None or value_pool is None:
+            raise KernelError("qk_norm_rope_append: a cache write needs slot_mapping and both pools.")
+        _check(slot_mapping, "slot_mapping", dtype=torch.int32, shape=(n,))
+        _check(key_pool, "key_pool", dtype=dtype)
+        _check(value_pool, "value_pool", dtype=dtype, shape=tuple(key_pool.shape))
+        if key_pool.ndim != 4 or key_pool.shape[1] != num_kv_heads or key_pool.shape[3] != head_dim:
+            raise KernelError(
+                f"qk_norm_rope_append: pool {tuple(key_pool.shape)} is not "
+                f"[pages, {num_kv_heads}, block_size, {head_dim}]."
+            )
+        block_size = key_pool.shape[2]
+    q_out = None
+    if num_q_heads > 0:
+        q_out = torch.empty((n, num_q_heads, head_dim), dtype=dtype, device=packed.device)
+    call("ms_qk_norm_rope_append", _ptr(packed), _ptr(q_weight), _ptr(k_weight), _ptr(inv_freq), _ptr(positions),
+         _ptr(slot_mapping), _ptr(q_out), _ptr(key_pool), _ptr(value_pool), n, num_q_heads, num_kv_heads,
+         head_dim, block_size, float(eps), _code(dtype), _stream())
+    return q_out
+
+
+def attention(
+    q: torch.Tensor,
+    key_pool: torch.Tensor,
+    value_pool: torch.Tensor,
+    *,
+    block_table: torch.Tensor,
+    seq_of_token: torch.Tensor,
+    positions: torch.Tensor,
+    scale: float,
+    window: int | None = None,
+) -> torch.Tensor:
+    """Causal attention of ``q [N, heads, head_dim]`` over the paged cache.
+
+    Token ``t`` belongs to sequence ``seq_of_token[t]``, stands at absolute
+    position ``positions[t]`` and sees the keys ``lo..positions[t]`` of that
+    sequence through ``block_table [S, max_blocks]`` (int32), ``lo`` being 0 or
+    ``positions[t] - window + 1``.  The caller guarantees that every page the
+    table names for those keys lies inside the pool."""
+
+    _check(q, "q")
+    if q.ndim != 3 or q.shape[0] == 0:
+        raise KernelError("attention: q must be [N>0, heads, head_dim].")
+    n, heads, head_dim = q.shape
+    _check(key_pool, "key_pool", dtype=q.dtype)
+    _check(value_pool, "value_pool", dtype=q.dtype, shape=tuple(key_pool.shape))
+    if key_pool.ndim != 4 or key_pool.shape[3] != head_dim:
+        raise KernelError(f"attention: pool {tuple(key_pool.shape)} is not [pages, kv_heads, block_size, {head_dim}].")
+    _, kv_heads, block_size, _ = key_pool.shape
+    if heads % kv_heads != 0:
+        raise KernelError(f"attention: {heads} query heads are not a multiple of {kv_heads} kv heads.")
+    _check(block_table, "block_table", dtype=torch.int32)
+    if block_table.ndim != 2 or block_table.shape[1] == 0:
+        raise KernelError("attention: block_table must be [S, max_blocks>0].")
+    _check(seq_of_token, "seq_of_token", dtype=torch.int32, shape=(n,))
+    _check(positions, "positions", dtype=torch.int32, shape=(n,))
+    window = 0 if window is None else int(window)
+    if window < 0:
+        raise KernelError("attention: window must be positive or None.")
+    out = torch.empty_like(q)
+    call("ms_attention_generic", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(seq_of_token),
+         _ptr(positions), _ptr(out), n, heads, kv_heads, head_dim, block_size, block_table.shape[1], float(scale),
+         window, _code(q.dtype), _stream())
+    return out
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, *, accumulate_into: torch.Tensor | None = None) -> torch.Tensor:
+    """``x [M, K] @ weight [N, K]^T``.
+
+    float32: this library's FMA kernel (true 32-bit; row results do not depend on
+    M); ``accumulate_into`` (float32 ``[M, N]``) receives ``+=``.  bfloat16: the
+    library matrix product (hipBLASLt through torch) with 32-bit accumulation."""
+
+    _check(x, "x")
+    _check(weight, "weight", dtype=x.dtype)
+    if x.ndim != 2 or weight.ndim != 2 or x.shape[1] != weight.shape[1] or x.shape[0] == 0:
+        raise KernelError(f"linear: x {tuple(x.shape)} does not match weight {tuple(weight.shape)}.")
+    m, k = x.shape
+    n = weight.shape[0]
+    if x.dtype == torch.float32:
+        if accumulate_into is not None:
+            _check(accumulate_into, "accumulate_into", dtype=torch.float32, shape=(m, n))
+            out = accumulate_into
+        else:
+            out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+        call("ms_gemm_f32", _ptr(x), _ptr(weight), _ptr(out), m, n, k, int(accumulate_into is not None), _stream())
+        return out
+    _code(x.dtype)
+    out = torch.mm(x, weight.t())
+    if accumulate_into is not None:
+        residual_add(accumulate_into, out)
+        return accumulate_into
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` of ``gate_up [N, 2*I]`` (gate columns first) -> ``[N, I]``."""
+
+    _check(gate_up, "gate_up")
+    if gate_up.ndim != 2 or gate_up.shape[1] % 2 != 0 or gate_up.numel() == 0:
+        raise KernelError("silu_mul takes gate_up [N>0, 2*I].")
+    rows, width = gate_up.shape
+    out = torch.empty((rows, width // 2), dtype=gate_up.dtype, device=gate_up.device)
+    call("ms_silu_mul", _ptr(gate_up), _ptr(out), rows, width // 2, _code(gate_up.dtype), _stream())
+    return out
+
+
+def sample_rows(
+    logits: torch.Tensor,
+    *,
+    temperature: torch.Tensor | None = None,
+    top_k: torch.Tensor | None = None,
+    top_p: torch.Tensor | None = None,
+    uniform: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """One token per row of float32 ``logits [R, V]`` -> int32 ``[R]``.
+
+    ``temperature`` None or 0 in a row: argmax.  Otherwise temperature, top-k
+    (0 = off), top-p (1 = off), then the inverse CDF at ``uniform[r]`` in token
+    order.  A row with a non-finite logit gives -1."""
+
+    _check(logits, "logits", dtype=torch.float32)
+    if logits.ndim != 2 or logits.numel() == 0:
+        raise KernelError("sample_rows takes logits [R>0, V>0].")
+    rows, vocab = logits.shape
+    if temperature is not None:
+        _check(temperature, "temperature", dtype=torch.float32, shape=(rows,))
+        if uniform is None:
+            raise KernelError("sample_rows: sampling needs uniform numbers.")
+        _check(uniform, "uniform", dtype=torch.float32, shape=(rows,))
+        if top_k is not None:
+            _check(top_k, "top_k", dtype=torch.int32, shape=(rows,))
+        if top_p is not None:
+            _check(top_p, "top_p", dtype=torch.float32, shape=(rows,))
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    call("ms_sample_rows", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(out),
+         rows, vocab, _stream())
+    return out

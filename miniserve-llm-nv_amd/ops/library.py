@@ -1,0 +1,94 @@
+"""Loads the HIP library through ctypes and declares every entry point.
+
+There is no fallback: when the library cannot be found or built, or an entry
+point reports an error, the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import sys
+import threading
+from ctypes import c_char_p, c_float, c_int, c_void_p
+
+from . import build as _build
+
+
+class KernelError(RuntimeError):
+    """An entry point of the HIP library refused its arguments or its launch."""
+
+
+_P, _I, _F = c_void_p, c_int, c_float
+
+# name -> argument types (the trailing stream argument included).
+_SIGNATURES: dict[str, list] = {
+    "ms_embedding_gather": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "ms_rmsnorm": [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _I, _P],
+    "ms_residual_add": [_P, _P, _I, _I, _I, _P],
+    "ms_qk_norm_rope_append": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
+    "ms_attention_generic": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "ms_gemm_f32": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "ms_silu_mul": [_P, _P, _I, _I, _I, _P],
+    "ms_sample_rows": [_P, _P, _P, _P, _P, _P, _I, _I, _P],
+}
+
+_lock = threading.Lock()
+_library: ctypes.CDLL | None = None
+_library_path: str | None = None
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    lib.ms_last_error.restype = c_char_p
+    lib.ms_last_error.argtypes = []
+    lib.ms_target_arch.restype = c_char_p
+    lib.ms_target_arch.argtypes = []
+    for name, argtypes in _SIGNATURES.items():
+        try:
+            function = getattr(lib, name)
+        except AttributeError:
+            raise KernelError(
+                f"{_library_path} lacks the entry point {name}; rebuild it "
+                "(python -c 'import __graft_entry__ as g; g.build()')."
+            ) from None
+        function.restype = c_int
+        function.argtypes = argtypes
+
+
+def load() -> ctypes.CDLL:
+    """The loaded library.  What is built is loaded; only when nothing is built
+    is it compiled, once, with progress lines on stderr."""
+
+    global _library, _library_path
+    if _library is not None:
+        return _library
+    with _lock:
+        if _library is not None:
+            return _library
+        path = _build.find_built_library()
+        if path is None:
+            path = _build.build(force=True)
+        elif _build.is_stale(path):
+            print(
+                f"[miniserve_amd] warning: {path} is older than its sources; rebuild it.",
+                file=sys.stderr,
+                flush=True,
+            )
+        _library_path = str(path)
+        try:
+            lib = ctypes.CDLL(_library_path)
+        except OSError as exc:
+            raise KernelError(f"cannot load {_library_path}: {exc}") from exc
+        _declare(lib)
+        _library = lib
+    return _library
+
+
+def library_path() -> str | None:
+    return _library_path
+
+
+def call(name: str, *args) -> None:
+    lib = load()
+    status = getattr(lib, name)(*args)
+    if status != 0:
+        raise KernelError(lib.ms_last_error().decode("utf-8", "replace"))

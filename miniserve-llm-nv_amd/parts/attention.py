@@ -1,0 +1,156 @@
+"""Grouped-query attention over the paged cache, with optional per-head norms of
+q and k and an optional position encoding (reference: miniserve/model/qwen3.py:56-323).
+
+Order of operations (qwen3.py:174-250): project q, k, v; norm q and k per head;
+rotate q and k; write k and v to the cache; attend causally over the cache
+(this step's tokens included); project the heads back.
+"""
+
+from __future__ import annotations
+
+from typing import Mapping
+
+import torch
+
+from .. import ops
+from ..config.model_spec import PartSpec
+from .base import KVCacheNeed, KVCacheView, Part, StepContext, WeightSpec, build_part, register_part, require_params
+from .norm import RMSNorm
+from .rotary import RotaryHalf
+
+
+class Attention(Part):
+    def __init__(self, spec: PartSpec, dtype: torch.dtype) -> None:
+        params = require_params(spec, "hidden_size", "num_heads", "num_kv_heads", "head_dim")
+        self.hidden_size = int(params["hidden_size"])
+        self.num_heads = int(params["num_heads"])
+        self.num_kv_heads = int(params["num_kv_heads"])
+        self.head_dim = int(params["head_dim"])
+        if self.num_heads <= 0 or self.num_kv_heads <= 0 or self.num_heads % self.num_kv_heads:
+            raise ValueError("attention needs num_heads to be a positive multiple of num_kv_heads.")
+        scale = params.get("scale")
+        self.scale = float(self.head_dim**-0.5 if scale is None else scale)
+        window = params.get("window")
+        if window is not None and (not isinstance(window, int) or window <= 0):
+            raise ValueError("attention window must be a positive integer or None.")
+        self.window = window
+        self.dtype = dtype
+        self.prefix = spec.prefix
+        self.q_norm = build_part("norm", params["q_norm"], dtype) if params.get("q_norm") else None
+        self.k_norm = build_part("norm", params["k_norm"], dtype) if params.get("k_norm") else None
+        self.position = build_part("position", params["position"], dtype) if params.get("position") else None
+        self.w_qkv: torch.Tensor | None = None
+        self.w_q: torch.Tensor | None = None
+        self.w_o: torch.Tensor | None = None
+        # The fused kernel covers RMSNorm (or no norm) with one eps and the
+        # half-split rotary (or none); anything else is composed from the parts.
+        norms = [n for n in (self.q_norm, self.k_norm) if n is not None]
+        self._fused = (
+            all(isinstance(n, RMSNorm) and n.dim == self.head_dim for n in norms)
+            and len({n.eps for n in norms}) <= 1
+            and (self.position is None or (isinstance(self.position, RotaryHalf) and self.position.dim == self.head_dim))
+            and self.head_dim % 2 == 0
+        )
+
+    # -- description ----------------------------------------------------------------
+    def sub_parts(self) -> list[Part]:
+        return [p for p in (self.q_norm, self.k_norm, self.position) if p is not None]
+
+    def weight_specs(self) -> list[WeightSpec]:
+        q_width = self.num_heads * self.head_dim
+        kv_width = self.num_kv_heads * self.head_dim
+        return [
+            WeightSpec(self.prefix + "q_proj.weight", (q_width, self.hidden_size)),
+            WeightSpec(self.prefix + "k_proj.weight", (kv_width, self.hidden_size)),
+            WeightSpec(self.prefix + "v_proj.weight", (kv_width, self.hidden_size)),
+            WeightSpec(self.prefix + "o_proj.weight", (self.hidden_size, q_width)),
+        ]
+
+    def cache_need(self) -> KVCacheNeed:
+        return KVCacheNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """q, k and v rows are stacked into one matrix, q rows first, then k, then
+        v, so one product gives the packed ``[N, (Hq + 2 Hkv) * D]`` row."""
+
+        q = tensors[self.prefix + "q_proj.weight"]
+        self.w_qkv = torch.cat(
+            [q, tensors[self.prefix + "k_proj.weight"], tensors[self.prefix + "v_proj.weight"]], dim=0
+        ).contiguous()
+        self.w_q = self.w_qkv[: q.shape[0]]
+        self.w_o = tensors[self.prefix + "o_proj.weight"]
+
+    # -- execution ------------------------------------------------------------------
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: KVCacheView) -> torch.Tensor:
+        if not isinstance(cache, KVCacheView):
+            raise TypeError("attention needs a paged key/value cache.")
+        group = ctx.groups[cache.group]
+        n = x.shape[0]
+        kv_heads = self.num_kv_heads if cache.write else 0
+        packed = ops.linear(x, self.w_qkv if cache.write else self.w_q)
+        if self._fused:
+            q = ops.qk_norm_rope_append(
+                packed,
+                num_q_heads=self.num_heads,
+                num_kv_heads=kv_heads,
+                head_dim=self.head_dim,
+                q_weight=None if self.q_norm is None else self.q_norm.weight,
+                k_weight=None if self.k_norm is None else self.k_norm.weight,
+                eps=next((p.eps for p in (self.q_norm, self.k_norm) if p is not None), 1.0),
+                inv_freq=None if self.position is None else self.position.inv_freq(x.device),
+                positions=ctx.positions,
+                slot_mapping=group.slot_mapping if cache.write else None,
+                key_pool=cache.key if cache.write else None,
+                value_pool=cache.value if cache.write else None,
+            )
+        else:
+            q = self._prepare_unfused(packed, ctx, cache, group, kv_heads)
+        attended = ops.attention(
+            q,
+            cache.key,
+            cache.value,
+            block_table=group.block_table,
+            seq_of_token=ctx.seq_of_token,
+            positions=ctx.positions,
+            scale=self.scale,
+            window=self.window,
+        )
+        return ops.linear(attended.reshape(n, self.num_heads * self.head_dim), self.w_o)
+
+    def _prepare_unfused(self, packed, ctx, cache, group, kv_heads) -> torch.Tensor:
+        """Norms and position encoding through their own parts, then the cache write."""
+
+        n = packed.shape[0]
+        q_width = self.num_heads * self.head_dim
+        kv_width = kv_heads * self.head_dim
+        q = packed[:, :q_width].reshape(n, self.num_heads, self.head_dim).contiguous()
+        if self.q_norm is not None:
+            q = self.q_norm.forward(q)
+        if self.position is not None:
+            q = self.position.apply(q, ctx.positions)
+        if kv_heads == 0:
+            return q
+        k = packed[:, q_width : q_width + kv_width].reshape(n, kv_heads, self.head_dim).contiguous()
+        if self.k_norm is not None:
+            k = self.k_norm.forward(k)
+        if self.position is not None:
+            k = self.position.apply(k, ctx.positions)
+        kv = torch.cat([k.reshape(n, kv_width), packed[:, q_width + kv_width :]], dim=1).contiguous()
+        ops.qk_norm_rope_append(
+            kv,
+            num_q_heads=0,
+            num_kv_heads=kv_heads,
+            head_dim=self.head_dim,
+            q_weight=None,
+            k_weight=None,
+            eps=1.0,
+            inv_freq=None,
+            positions=None,
+            slot_mapping=group.slot_mapping,
+            key_pool=cache.key,
+            value_pool=cache.value,
+        )
+        return q
+
+
+register_part("mixer", "attention", Attention)

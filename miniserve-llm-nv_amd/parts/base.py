@@ -1,0 +1,208 @@
+"""Interfaces of the parts a layer is built from, and their registries.
+
+A part is constructed from its ``PartSpec`` alone (its sizes and constants), says
+which tensors it wants (``weight_specs``), receives them (``load_weights``) and
+runs on a flat batch of tokens.  No part knows which model it is in.
+
+Categories and what each must offer:
+
+``norm``              ``forward(x) -> y`` and ``add_forward(residual, delta, *,
+                      rows=None, write_back=True) -> y``: the norm of
+                      ``residual + delta``; the sum is stored into the 32-bit
+                      ``residual`` when ``write_back``.
+``position``          ``apply(x [N, heads, dim], positions [N]) -> x'``; no weights.
+``mixer``             ``cache_need() -> KVCacheNeed | StateNeed | None`` and
+                      ``forward(x [N, H], ctx: StepContext, cache) -> [N, H]``,
+                      ``cache`` being a ``KVCacheView``, a ``StateView`` or None.
+``feed_forward``      ``forward(x [N, H], ctx) -> [N, H]``.
+``block``             the arrangement of one layer's parts around the residual
+                      stream: ``forward(residual, delta, ctx, cache) ->
+                      (residual, delta)``; the sum ``residual + delta`` is what
+                      the next block (or the final norm) starts from.
+``embedding``         ``forward(token_ids [N]) -> float32 [N, H]``.
+``head``              ``forward(x [R, H]) -> float32 logits [R, V]``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Mapping
+
+import torch
+
+from ..config.model_spec import PartSpec
+
+CATEGORIES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")
+
+
+# ---- what a part says about its tensors ------------------------------------------
+
+@dataclass(frozen=True)
+class WeightSpec:
+    """One checkpoint tensor that a part wants.
+
+    ``init`` picks the random-weights distribution: ``"matrix"`` ~ N(0, 0.02),
+    ``"norm"`` ~ 1 + N(0, 0.1), ``"zeros"``.  ``keep`` says how the tensor is
+    held: ``"compute"`` in the engine's dtype (bfloat16 or float32),
+    ``"float32"`` always in 32-bit, ``"int32"`` an integer table.
+    ``optional`` tensors may be absent; ``same_as`` names a tensor that an
+    optional one must equal bit for bit when it is present (a tied head)."""
+
+    name: str
+    shape: tuple[int, ...]
+    init: str = "matrix"
+    keep: str = "compute"
+    optional: bool = False
+    same_as: str | None = None
+
+
+# ---- what a mixer says about its cache -------------------------------------------
+
+@dataclass(frozen=True)
+class KVCacheNeed:
+    """Keys and values in pages.  ``window`` None: all keys are kept; an int: only
+    the last ``window`` keys of a position are ever read, older pages go back."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size: one tensor of ``shape`` per live request."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class KVCacheView:
+    """One call's slice of its group's pools: ``[pages, kv_heads, block_size, head_dim]``."""
+
+    group: int
+    key: torch.Tensor
+    value: torch.Tensor
+    block_size: int
+    write: bool = True     # False: this call reads another call's cache
+
+
+@dataclass
+class StateView:
+    """One call's state for every slot: ``[max_num_seqs, *shape]``."""
+
+    tensor: torch.Tensor
+
+
+# ---- the batch of one step, as parts see it ---------------------------------------
+
+@dataclass
+class GroupStepView:
+    """Cache metadata of one group for this step."""
+
+    block_table: torch.Tensor    # int32 [S, max_blocks]
+    slot_mapping: torch.Tensor   # int32 [N]: page * block_size + offset of each new token
+
+
+@dataclass
+class StepContext:
+    """A flat ragged batch: ``N`` tokens of ``S`` sequences, each sequence's tokens
+    contiguous and at consecutive absolute positions."""
+
+    num_tokens: int
+    num_seqs: int
+    token_ids: torch.Tensor       # int32 [N]
+    positions: torch.Tensor       # int32 [N], absolute
+    seq_of_token: torch.Tensor    # int32 [N]
+    query_start: torch.Tensor     # int32 [S + 1]
+    context_lens: torch.Tensor    # int32 [S], length after this step
+    state_slots: torch.Tensor     # int32 [S]
+    groups: list[GroupStepView]
+    # host copies, for launch decisions
+    query_lens: list[int] = field(default_factory=list)
+    context_lens_host: list[int] = field(default_factory=list)
+    query_start_host: list[int] = field(default_factory=list)
+    state_slots_host: list[int] = field(default_factory=list)
+    first_positions_host: list[int] = field(default_factory=list)
+
+    @property
+    def max_query_len(self) -> int:
+        return max(self.query_lens)
+
+    @property
+    def max_context_len(self) -> int:
+        return max(self.context_lens_host)
+
+
+# ---- registries -------------------------------------------------------------------
+
+_REGISTRIES: dict[str, dict[str, Callable[..., Any]]] = {category: {} for category in CATEGORIES}
+
+
+def register_part(category: str, kind: str, factory: Callable[..., Any]) -> None:
+    """Register ``factory(spec: PartSpec, dtype: torch.dtype) -> part`` under ``kind``."""
+
+    if category not in _REGISTRIES:
+        raise ValueError(f"unknown part category {category!r}; one of {CATEGORIES}.")
+    _REGISTRIES[category][kind] = factory
+
+
+def unregister_part(category: str, kind: str) -> None:
+    _REGISTRIES[category].pop(kind, None)
+
+
+def build_part(category: str, spec: PartSpec, dtype: torch.dtype) -> Any:
+    try:
+        factory = _REGISTRIES[category][spec.kind]
+    except KeyError:
+        known = ", ".join(sorted(_REGISTRIES.get(category, {}))) or "none"
+        raise KeyError(f"no {category} part of kind {spec.kind!r} is registered (known: {known}).") from None
+    return factory(spec, dtype)
+
+
+def registered_parts(category: str) -> tuple[str, ...]:
+    return tuple(sorted(_REGISTRIES[category]))
+
+
+def require_params(spec: PartSpec, *names: str) -> Mapping[str, Any]:
+    missing = [name for name in names if name not in spec.params]
+    if missing:
+        raise ValueError(f"part {spec.kind!r} lacks parameters {missing}.")
+    return spec.params
+
+
+class Part:
+    """Base of all parts: no weights, nothing to load."""
+
+    def weight_specs(self) -> list[WeightSpec]:
+        return []
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        return None
+
+    def sub_parts(self) -> list["Part"]:
+        return []
+
+
+def collect_weight_specs(part: Part) -> list[WeightSpec]:
+    specs = list(part.weight_specs())
+    for child in part.sub_parts():
+        specs.extend(collect_weight_specs(child))
+    return specs
+
+
+def load_part_weights(part: Part, tensors: Mapping[str, torch.Tensor]) -> None:
+    part.load_weights(tensors)
+    for child in part.sub_parts():
+        load_part_weights(child, tensors)
+
+
+def build_block(layer, dtype: torch.dtype) -> Any:
+    """A block factory takes the whole ``LayerSpec`` (``layer.block`` is its kind)."""
+
+    try:
+        factory = _REGISTRIES["block"][layer.block]
+    except KeyError:
+        known = ", ".join(sorted(_REGISTRIES["block"])) or "none"
+        raise KeyError(f"no block arrangement {layer.block!r} is registered (known: {known}).") from None
+    return factory(layer, dtype)

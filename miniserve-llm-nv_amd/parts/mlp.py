@@ -1,0 +1,50 @@
+"""Gated feed-forward: ``down(act(gate(x)) * up(x))``, no biases, every token the
+same weights (reference: miniserve/model/layers.py:71-87)."""
+
+from __future__ import annotations
+
+from typing import Mapping
+
+import torch
+
+from .. import ops
+from ..config.model_spec import PartSpec
+from .base import Part, StepContext, WeightSpec, register_part, require_params
+
+_ACTIVATIONS = {"silu": ops.silu_mul}
+
+
+class GatedMLP(Part):
+    def __init__(self, spec: PartSpec, dtype: torch.dtype) -> None:
+        params = require_params(spec, "hidden_size", "intermediate_size", "activation")
+        self.hidden_size = int(params["hidden_size"])
+        self.intermediate_size = int(params["intermediate_size"])
+        activation = params["activation"]
+        if activation not in _ACTIVATIONS:
+            raise ValueError(f"gated_mlp knows the activations {sorted(_ACTIVATIONS)}, not {activation!r}.")
+        self._gated_activation = _ACTIVATIONS[activation]
+        self.dtype = dtype
+        self.prefix = spec.prefix
+        self.w_gate_up: torch.Tensor | None = None
+        self.w_down: torch.Tensor | None = None
+
+    def weight_specs(self) -> list[WeightSpec]:
+        return [
+            WeightSpec(self.prefix + "gate_proj.weight", (self.intermediate_size, self.hidden_size)),
+            WeightSpec(self.prefix + "up_proj.weight", (self.intermediate_size, self.hidden_size)),
+            WeightSpec(self.prefix + "down_proj.weight", (self.hidden_size, self.intermediate_size)),
+        ]
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """Gate rows, then up rows, in one matrix: one product gives ``[N, 2 I]``."""
+
+        self.w_gate_up = torch.cat(
+            [tensors[self.prefix + "gate_proj.weight"], tensors[self.prefix + "up_proj.weight"]], dim=0
+        ).contiguous()
+        self.w_down = tensors[self.prefix + "down_proj.weight"]
+
+    def forward(self, x: torch.Tensor, ctx: StepContext | None = None) -> torch.Tensor:
+        return ops.linear(self._gated_activation(ops.linear(x, self.w_gate_up)), self.w_down)
+
+
+register_part("feed_forward", "gated_mlp", GatedMLP)

@@ -1,0 +1,121 @@
+"""Choosing the next token: greedy, or temperature -> top-k -> top-p -> one draw,
+with one random stream per request (reference: miniserve/model/sampling.py:61-242).
+
+The choice itself is made on the device by ``ops.sample_rows``; the host keeps
+the per-request generators and draws ONE uniform number per sampled token from
+them.  As in the reference, a draw is *staged*: the generator advances only when
+the step that produced the logits is committed.
+"""
+
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import Sequence
+
+import torch
+
+from ..engine.request import SamplingParams
+
+_BELOW_ONE = 1.0 - 2.0**-24      # largest float32 below 1
+
+
+@dataclass(frozen=True)
+class StagedSample:
+    request_id: str
+    token_id: int
+    generator_state: torch.Tensor | None      # None: greedy, no randomness used
+
+
+class NonFiniteLogitsError(ValueError):
+    pass
+
+
+class Sampler:
+    def __init__(self) -> None:
+        self._generators: dict[str, torch.Generator] = {}
+
+    # ---- random streams ---------------------------------------------------------------
+    @staticmethod
+    def _new_generator(params: SamplingParams) -> torch.Generator:
+        generator = torch.Generator(device="cpu")
+        seed = params.seed if params.seed is not None else int.from_bytes(os.urandom(8), "little") & (2**63 - 1)
+        generator.manual_seed(seed)
+        return generator
+
+    @staticmethod
+    def draw_uniform(generator: torch.Generator) -> float:
+        """One number in [0, 1) that float32 represents below 1."""
+
+        value = float(torch.rand((), generator=generator, dtype=torch.float64))
+        return min(value, _BELOW_ONE)
+
+    # ---- sampling ---------------------------------------------------------------------
+    def stage(
+        self, logits: torch.Tensor, requests: Sequence[tuple[str, SamplingParams]]
+    ) -> tuple[StagedSample, ...]:
+        """One token per row of float32 ``logits [R, V]`` (on the GPU) for the R
+        requests, without advancing any generator."""
+
+        from .. import ops
+
+        if logits.ndim != 2 or logits.shape[0] != len(requests) or logits.shape[1] == 0:
+            raise ValueError("logits must have shape [requests, vocab].")
+        if not logits.is_floating_point():
+            raise TypeError("logits must use a floating-point dtype.")
+        vocab = logits.shape[1]
+        states: list[torch.Tensor | None] = []
+        uniforms: list[float] = []
+        for request_id, params in requests:
+            if params.top_k > vocab:
+                raise ValueError("top_k must not exceed the vocabulary size.")
+            if params.temperature == 0:
+                states.append(None)
+                uniforms.append(0.0)
+                continue
+            known = self._generators.get(request_id)
+            scratch = torch.Generator(device="cpu")
+            scratch.set_state((known or self._new_generator(params)).get_state())
+            uniforms.append(self.draw_uniform(scratch))
+            states.append(scratch.get_state())
+        logits = logits.float().contiguous()
+        if all(state is None for state in states):
+            tokens = ops.sample_rows(logits)
+        else:
+            device = logits.device
+            tokens = ops.sample_rows(
+                logits,
+                temperature=torch.tensor([p.temperature for _, p in requests], dtype=torch.float32, device=device),
+                top_k=torch.tensor([p.top_k for _, p in requests], dtype=torch.int32, device=device),
+                top_p=torch.tensor([p.top_p for _, p in requests], dtype=torch.float32, device=device),
+                uniform=torch.tensor(uniforms, dtype=torch.float32, device=device),
+            )
+        token_ids = tokens.tolist()
+        if any(token < 0 for token in token_ids):
+            raise NonFiniteLogitsError("logits must contain only finite values.")
+        return tuple(
+            StagedSample(request_id, int(token), state)
+            for (request_id, _), token, state in zip(requests, token_ids, states)
+        )
+
+    def commit(self, samples: Sequence[StagedSample]) -> None:
+        for sample in samples:
+            if sample.generator_state is None:
+                continue
+            generator = self._generators.get(sample.request_id)
+            if generator is None:
+                generator = torch.Generator(device="cpu")
+                self._generators[sample.request_id] = generator
+            generator.set_state(sample.generator_state)
+
+    def sample(self, logits: torch.Tensor, requests: Sequence[tuple[str, SamplingParams]]) -> list[int]:
+        staged = self.stage(logits, requests)
+        self.commit(staged)
+        return [sample.token_id for sample in staged]
+
+    def release(self, request_id: str) -> None:
+        self._generators.pop(request_id, None)
+
+    @property
+    def active_request_ids(self) -> tuple[str, ...]:
+        return tuple(sorted(self._generators))

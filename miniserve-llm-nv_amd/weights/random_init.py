@@ -1,0 +1,85 @@
+"""Random-weights mode: a model folder (``config.json`` + ``model.safetensors``)
+from a configuration and a seed.  The reference has no such mode (its model is
+filled from safetensors only, miniserve/api/bootstrap.py:113-115).
+
+Matrices and embeddings ~ N(0, 0.02), norm weights ~ 1 + N(0, 0.1), drawn in
+float32 from one CPU generator in the model's fixed tensor order, so a seed
+names one model everywhere.
+"""
+
+from __future__ import annotations
+
+import json
+from pathlib import Path
+from typing import Sequence
+
+import torch
+
+from ..parts.base import WeightSpec
+
+MATRIX_STD = 0.02
+NORM_STD = 0.1
+STORE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def draw_tensor(spec: WeightSpec, generator: torch.Generator, device: torch.device | str = "cpu") -> torch.Tensor:
+    if spec.keep == "int32":
+        return torch.zeros(spec.shape, dtype=torch.int32, device=device)
+    if spec.init == "matrix":
+        return torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device) * MATRIX_STD
+    if spec.init == "norm":
+        return 1.0 + torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device) * NORM_STD
+    if spec.init == "zeros":
+        return torch.zeros(spec.shape, dtype=torch.float32, device=device)
+    raise ValueError(f"{spec.name}: unknown init rule {spec.init!r}.")
+
+
+def random_tensors(specs: Sequence[WeightSpec], seed: int) -> dict[str, torch.Tensor]:
+    """Float32 CPU tensors for every non-tied spec, in spec order."""
+
+    generator = torch.Generator(device="cpu").manual_seed(seed)
+    return {spec.name: draw_tensor(spec, generator) for spec in specs if spec.same_as is None}
+
+
+def write_random_model(config, folder: str | Path, *, seed: int, store_dtype: str = "float32") -> Path:
+    """Write ``config.json`` and ``model.safetensors`` for ``config`` (any
+    registered architecture's configuration object) into ``folder``."""
+
+    from safetensors.torch import save_file
+
+    from ..parts.model import DecoderModel
+
+    if store_dtype not in STORE_DTYPES:
+        raise ValueError(f"store_dtype must be one of {sorted(STORE_DTYPES)}.")
+    folder = Path(folder)
+    folder.mkdir(parents=True, exist_ok=True)
+    specs = DecoderModel(config.model_spec(), "float32").weight_specs()
+    tensors = {}
+    for name, tensor in random_tensors(specs, seed).items():
+        if tensor.is_floating_point():
+            tensor = tensor.to(STORE_DTYPES[store_dtype])
+        tensors[name] = tensor.contiguous()
+    data = config.to_dict()
+    data["torch_dtype"] = store_dtype
+    (folder / "config.json").write_text(json.dumps(data, indent=2) + "\n", encoding="utf-8")
+    save_file(tensors, str(folder / "model.safetensors"))
+    return folder
+
+
+def random_device_tensors(
+    specs: Sequence[WeightSpec], *, seed: int, dtype: torch.dtype, device: torch.device | str
+) -> dict[str, torch.Tensor]:
+    """The same distributions drawn tensor by tensor on the device, for models too
+    large to pass through a file or host memory (benchmarks).  The values differ
+    from :func:`random_tensors` with the same seed."""
+
+    generator = torch.Generator(device=device).manual_seed(seed)
+    tensors = {}
+    for spec in specs:
+        if spec.same_as is not None:
+            continue
+        tensor = draw_tensor(spec, generator, device)
+        if tensor.is_floating_point() and spec.keep == "compute":
+            tensor = tensor.to(dtype)
+        tensors[spec.name] = tensor
+    return tensors
