@@ -29,10 +29,10 @@ extern "C" int ms_silu_mul(const void* gate_up, void* out, int rows, int inter, 
   int64_t blocks = (total + threads - 1) / threads;
   if (blocks > 65536) blocks = 65536;
   if (dtype == MS_F32) {
-    silu_mul_kernel<float><<<dim3(blocks), threads, 0, stream>>>(static_cast<const float*>(gate_up),
+    hipLaunchKernelGGL((silu_mul_kernel<float>), dim3(blocks), dim3(threads), 0, stream, static_cast<const float*>(gate_up),
                                                                  static_cast<float*>(out), rows, inter);
   } else if (dtype == MS_BF16) {
-    silu_mul_kernel<ms::bf16><<<dim3(blocks), threads, 0, stream>>>(static_cast<const ms::bf16*>(gate_up),
+    hipLaunchKernelGGL((silu_mul_kernel<ms::bf16>), dim3(blocks), dim3(threads), 0, stream, static_cast<const ms::bf16*>(gate_up),
                                                                     static_cast<ms::bf16*>(out), rows, inter);
   } else {
     return ms_fail("silu_mul: unknown dtype code %d", dtype);
@@ -61,10 +61,10 @@ extern "C" int ms_residual_add(void* h, const void* delta, int rows, int dim, in
   int64_t blocks = (total + threads - 1) / threads;
   if (blocks > 65536) blocks = 65536;
   if (dtype == MS_F32) {
-    residual_add_kernel<float><<<dim3(blocks), threads, 0, stream>>>(static_cast<float*>(h),
+    hipLaunchKernelGGL((residual_add_kernel<float>), dim3(blocks), dim3(threads), 0, stream, static_cast<float*>(h),
                                                                      static_cast<const float*>(delta), total);
   } else if (dtype == MS_BF16) {
-    residual_add_kernel<ms::bf16><<<dim3(blocks), threads, 0, stream>>>(
+    hipLaunchKernelGGL((residual_add_kernel<ms::bf16>), dim3(blocks), dim3(threads), 0, stream, 
         static_cast<float*>(h), static_cast<const ms::bf16*>(delta), total);
   } else {
     return ms_fail("residual_add: unknown dtype code %d", dtype);

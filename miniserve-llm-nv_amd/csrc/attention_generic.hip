@@ -128,13 +128,13 @@ extern "C" int ms_attention_generic(const void* q, const void* key_pool, const v
   MS_REQUIRE(num_q_heads <= 65535, "attention_generic: too many heads");
   const dim3 grid(num_tokens, num_q_heads);
   if (dtype == MS_F32) {
-    attention_generic_kernel<float><<<grid, ms::kWave, 0, stream>>>(
+    hipLaunchKernelGGL((attention_generic_kernel<float>), dim3(grid), dim3(ms::kWave), 0, stream, 
         static_cast<const float*>(q), static_cast<const float*>(key_pool), static_cast<const float*>(value_pool),
         static_cast<const int32_t*>(block_table), static_cast<const int32_t*>(seq_of_token),
         static_cast<const int32_t*>(positions), static_cast<float*>(out), num_q_heads, num_kv_heads, head_dim,
         block_size, max_blocks, scale, window);
   } else if (dtype == MS_BF16) {
-    attention_generic_kernel<ms::bf16><<<grid, ms::kWave, 0, stream>>>(
+    hipLaunchKernelGGL((attention_generic_kernel<ms::bf16>), dim3(grid), dim3(ms::kWave), 0, stream, 
         static_cast<const ms::bf16*>(q), static_cast<const ms::bf16*>(key_pool),
         static_cast<const ms::bf16*>(value_pool), static_cast<const int32_t*>(block_table),
         static_cast<const int32_t*>(seq_of_token), static_cast<const int32_t*>(positions),

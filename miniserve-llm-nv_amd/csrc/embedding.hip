@@ -21,10 +21,10 @@ extern "C" int ms_embedding_gather(const void* token_ids, const void* table, voi
   const int threads = hidden >= 256 ? 256 : 64;
   const dim3 grid(num_tokens);
   if (dtype == MS_F32) {
-    embedding_gather_kernel<float><<<grid, threads, 0, stream>>>(
+    hipLaunchKernelGGL((embedding_gather_kernel<float>), dim3(grid), dim3(threads), 0, stream, 
         static_cast<const int32_t*>(token_ids), static_cast<const float*>(table), static_cast<float*>(out), hidden);
   } else if (dtype == MS_BF16) {
-    embedding_gather_kernel<ms::bf16><<<grid, threads, 0, stream>>>(
+    hipLaunchKernelGGL((embedding_gather_kernel<ms::bf16>), dim3(grid), dim3(threads), 0, stream, 
         static_cast<const int32_t*>(token_ids), static_cast<const ms::bf16*>(table), static_cast<float*>(out),
         hidden);
   } else {

@@ -76,7 +76,7 @@ extern "C" int ms_gemm_f32(const void* a, const void* w, void* c, int m, int n, 
   MS_REQUIRE(m > 0 && n > 0 && k > 0, "gemm_f32: empty shape %d x %d x %d", m, n, k);
   const dim3 grid((n + kTileN - 1) / kTileN, (m + kTileM - 1) / kTileM);
   MS_REQUIRE(grid.y <= 65535, "gemm_f32: %d rows exceed the grid limit", m);
-  gemm_f32_kernel<<<grid, 256, 0, stream>>>(static_cast<const float*>(a), static_cast<const float*>(w),
+  hipLaunchKernelGGL(gemm_f32_kernel, dim3(grid), dim3(256), 0, stream, static_cast<const float*>(a), static_cast<const float*>(w),
                                             static_cast<float*>(c), m, n, k, accumulate);
   MS_CHECK_LAUNCH("gemm_f32");
   return 0;

@@ -60,16 +60,16 @@ extern "C" int ms_rmsnorm(void* x, const void* delta, const void* weight, void* 
   const dim3 grid(n_out);
   const int32_t* r = static_cast<const int32_t*>(rows);
   if (dtype == MS_F32) {
-    rmsnorm_kernel<float, float><<<grid, threads, 0, stream>>>(
+    hipLaunchKernelGGL((rmsnorm_kernel<float, float>), dim3(grid), dim3(threads), 0, stream, 
         static_cast<float*>(x), static_cast<const float*>(delta), static_cast<const float*>(weight),
         static_cast<float*>(out), r, dim, eps, write_back);
   } else if (dtype == MS_BF16) {
     if (x_is_f32) {
-      rmsnorm_kernel<float, ms::bf16><<<grid, threads, 0, stream>>>(
+      hipLaunchKernelGGL((rmsnorm_kernel<float, ms::bf16>), dim3(grid), dim3(threads), 0, stream, 
           static_cast<float*>(x), static_cast<const ms::bf16*>(delta), static_cast<const ms::bf16*>(weight),
           static_cast<ms::bf16*>(out), r, dim, eps, write_back);
     } else {
-      rmsnorm_kernel<ms::bf16, ms::bf16><<<grid, threads, 0, stream>>>(
+      hipLaunchKernelGGL((rmsnorm_kernel<ms::bf16, ms::bf16>), dim3(grid), dim3(threads), 0, stream, 
           static_cast<ms::bf16*>(x), static_cast<const ms::bf16*>(delta), static_cast<const ms::bf16*>(weight),
           static_cast<ms::bf16*>(out), r, dim, eps, write_back);
     }

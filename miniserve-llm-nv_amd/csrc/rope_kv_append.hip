@@ -103,7 +103,7 @@ int launch(const void* packed, const void* q_weight, const void* k_weight, const
            int num_tokens, int num_q_heads, int num_kv_heads, int head_dim, int block_size, float eps,
            hipStream_t stream) {
   const dim3 grid(num_tokens, num_q_heads + 2 * num_kv_heads);
-  qk_norm_rope_append_kernel<T><<<grid, ms::kWave, 0, stream>>>(
+  hipLaunchKernelGGL((qk_norm_rope_append_kernel<T>), dim3(grid), dim3(ms::kWave), 0, stream, 
       static_cast<const T*>(packed), static_cast<const T*>(q_weight), static_cast<const T*>(k_weight),
       static_cast<const float*>(inv_freq), static_cast<const int32_t*>(positions),
       static_cast<const int32_t*>(slot_mapping), static_cast<T*>(q_out), static_cast<T*>(key_pool),

@@ -225,7 +225,7 @@ extern "C" int ms_sample_rows(const void* logits, const void* temperature, const
                               const void* uniform, void* out, int rows, int vocab, hipStream_t stream) {
   MS_REQUIRE(rows > 0 && vocab > 0, "sample_rows: empty shape");
   MS_REQUIRE(!temperature || uniform, "sample_rows: sampling rows need uniform numbers");
-  sample_rows_kernel<<<dim3(rows), kThreads, 0, stream>>>(
+  hipLaunchKernelGGL(sample_rows_kernel, dim3(rows), dim3(kThreads), 0, stream, 
       static_cast<const float*>(logits), static_cast<const float*>(temperature),
       static_cast<const int32_t*>(top_k), static_cast<const float*>(top_p), static_cast<const float*>(uniform),
       static_cast<int32_t*>(out), vocab);

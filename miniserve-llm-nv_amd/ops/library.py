@@ -55,8 +55,9 @@ def _declare(lib: ctypes.CDLL) -> None:
 
 
 def load() -> ctypes.CDLL:
-    """The loaded library.  What is built is loaded; only when nothing is built
-    is it compiled, once, with progress lines on stderr."""
+    """The loaded library.  What is built is loaded; it is compiled, with progress
+    lines on stderr, only when nothing is built or what is built does not match
+    the sources."""
 
     global _library, _library_path
     if _library is not None:
@@ -68,11 +69,10 @@ def load() -> ctypes.CDLL:
         if path is None:
             path = _build.build(force=True)
         elif _build.is_stale(path):
-            print(
-                f"[miniserve_amd] warning: {path} is older than its sources; rebuild it.",
-                file=sys.stderr,
-                flush=True,
-            )
+            # A library that does not match its sources may disagree with the Python
+            # side about argument types; it is never run.
+            print(f"[miniserve_amd] {path} does not match its sources; rebuilding.", file=sys.stderr, flush=True)
+            path = _build.build(force=True)
         _library_path = str(path)
         try:
             lib = ctypes.CDLL(_library_path)
