@@ -1,0 +1,95 @@
+"""A stand-in for the model runner, for testing the engine loop on the CPU: a real
+cache manager (without storage) and "logits" that depend only on a request's
+token prefix, so what a request generates cannot depend on scheduling."""
+
+from __future__ import annotations
+
+import hashlib
+from types import SimpleNamespace
+
+import torch
+
+from miniserve_amd.cache import CacheLayout, CacheManager, StepItem
+from miniserve_amd.config import EngineConfig
+from miniserve_amd.parts import KVCacheNeed
+
+
+def next_token(prefix: tuple[int, ...], vocab: int) -> int:
+    digest = hashlib.sha256(repr(prefix).encode()).digest()
+    return int.from_bytes(digest[:4], "little") % vocab
+
+
+class FakeRunner:
+    def __init__(self, engine_config: EngineConfig, *, vocab_size=97, max_positions=256, fail_on_step=None):
+        self.spec = SimpleNamespace(vocab_size=vocab_size, max_positions=max_positions)
+        self.engine_config = engine_config.validate(max_positions=max_positions)
+        self.max_model_len = engine_config.resolved_max_model_len(max_positions)
+        self.block_size = engine_config.kv_block_size
+        need = SimpleNamespace(call=0, need=KVCacheNeed(1, 8), cache_from=None)
+        self.cache = CacheManager(
+            CacheLayout.from_needs([need]), block_size=self.block_size, num_blocks=engine_config.num_kv_blocks,
+            max_num_seqs=engine_config.max_num_seqs, max_model_len=self.max_model_len,
+        )
+        self.tokens: dict[str, list[int]] = {}
+        self.steps: list[list[tuple[str, int, int]]] = []     # per step: (request, start, end)
+        self.fail_on_step = fail_on_step
+
+    def admit(self, request_id):
+        self.tokens[request_id] = []
+        return self.cache.admit(request_id)
+
+    def release(self, request_id):
+        self.tokens.pop(request_id, None)
+        self.cache.release(request_id)
+
+    def step(self, entries):
+        items = []
+        for entry in entries:
+            start = self.cache.committed_tokens(entry.request_id)
+            assert start == len(self.tokens[entry.request_id]), "the engine skipped or repeated tokens"
+            items.append(StepItem(entry.request_id, start, start + len(entry.token_ids)))
+        reservation = self.cache.prepare_step(items)
+        if self.fail_on_step is not None and len(self.steps) == self.fail_on_step:
+            self.fail_on_step = None
+            self.cache.abort_step(reservation)
+            raise RuntimeError("injected kernel failure")
+        rows = []
+        for entry in entries:
+            base = self.tokens[entry.request_id]
+            for place in entry.want:
+                prefix = tuple(base) + tuple(entry.token_ids[: place + 1])
+                row = torch.zeros(self.spec.vocab_size)
+                row[next_token(prefix, self.spec.vocab_size)] = 1.0
+                rows.append(row)
+            base.extend(entry.token_ids)
+        self.cache.commit_step(reservation)
+        self.cache.assert_invariants()
+        self.steps.append([(i.request_id, i.start, i.end) for i in items])
+        return torch.stack(rows) if rows else None
+
+
+class ArgmaxSampler:
+    """Greedy on the host; the engine's sampler interface."""
+
+    def stage(self, logits, requests):
+        from miniserve_amd.sampling import StagedSample
+
+        return tuple(StagedSample(rid, int(torch.argmax(row)), None) for (rid, _), row in zip(requests, logits))
+
+    def commit(self, samples):
+        pass
+
+    def release(self, request_id):
+        pass
+
+
+def expected_generation(prompt, max_new_tokens, vocab, stop=()):
+    tokens = list(prompt)
+    out = []
+    for _ in range(max_new_tokens):
+        token = next_token(tuple(tokens), vocab)
+        out.append(token)
+        tokens.append(token)
+        if token in stop:
+            break
+    return out

@@ -1,0 +1,358 @@
+"""The scheduler's decisions, the request state machine and the engine loop (no GPU)."""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+from fake_runner import ArgmaxSampler, FakeRunner, expected_generation
+
+from miniserve_amd.cache import CapacitySnapshot
+from miniserve_amd.config import EngineConfig
+from miniserve_amd.engine import (
+    DecodeItem,
+    Engine,
+    ExecutionPlan,
+    PrefillItem,
+    Request,
+    RequestStatus,
+    SamplingParams,
+    Scheduler,
+    SequenceState,
+    SequenceView,
+)
+
+W, P, D = RequestStatus.WAITING, RequestStatus.PREFILLING, RequestStatus.DECODING
+
+
+def view(name, status, *, target=10, cursor=0, generated=0, arrival=0, max_new=8) -> SequenceView:
+    computed = cursor if status is not D else target + generated - 1
+    total = target if status is not D else target + generated
+    return SequenceView(
+        request_id=name, status=status, prefill_target=target, prefill_cursor=cursor if status is not D else target,
+        computed_tokens=computed, total_tokens=total, num_generated=generated, max_new_tokens=max_new,
+        arrival_ns=arrival, next_input_token_id=7 if status is D else None,
+    )
+
+
+def capacity(free, *, total=64, block_size=4, free_slots=4, slots=8, held=None) -> CapacitySnapshot:
+    return CapacitySnapshot(block_size, (total,), (free,), free_slots, slots, held or {})
+
+
+def scheduler(**options) -> Scheduler:
+    base = dict(max_num_seqs=8, max_num_batched_tokens=32)
+    base.update(options)
+    return Scheduler(**base)
+
+
+# ---- the request state machine: the reference's vectors --------------------------------
+
+def request(max_new_tokens=2, stop=()):
+    return Request("r", (10, 20, 30), SamplingParams(max_new_tokens=max_new_tokens, stop_token_ids=stop), 1)
+
+
+def test_prefill_and_decode_preserve_pending_token_invariant():
+    # reference: tests/unit/test_sequence_state.py:54-71
+    state = SequenceState.from_request(request())
+    state.begin_prefill()
+    state.commit_prefill(3)
+    state.append_sampled_token(42)
+    assert state.status is D and state.all_tokens == (10, 20, 30, 42)
+    assert state.computed_tokens == 3 and state.total_tokens == state.computed_tokens + 1
+    assert state.snapshot().next_input_token_id == 42
+    state.mark_decode_input_computed()
+    state.append_sampled_token(43)
+    assert state.should_finish() == "length"
+    state.finish("length")
+    assert state.status is RequestStatus.FINISHED and state.computed_tokens == state.total_tokens - 1
+
+
+def test_stop_token_finishes_without_being_run():
+    # reference: tests/unit/test_sequence_state.py:74-82
+    state = SequenceState.from_request(request(max_new_tokens=4, stop=(99,)))
+    state.begin_prefill()
+    state.commit_prefill(3)
+    state.append_sampled_token(99)
+    assert state.should_finish() == "stop"
+    state.finish("stop")
+    assert state.computed_tokens == 3 and state.total_tokens == 4
+
+
+def test_partial_prefill_does_not_sample_and_illegal_moves_fail():
+    # reference: tests/unit/test_sequence_state.py:84-104
+    state = SequenceState.from_request(request())
+    with pytest.raises(RuntimeError, match="pending sampled token"):
+        state.mark_decode_input_computed()
+    state.begin_prefill()
+    state.commit_prefill(2)
+    assert state.status is P and state.prefill_cursor == state.computed_tokens == 2
+    with pytest.raises(RuntimeError, match="must be computed before sampling"):
+        state.append_sampled_token(1)
+    with pytest.raises(RuntimeError, match="advance within the prompt"):
+        state.commit_prefill(2)
+    state.commit_prefill(3)
+    state.append_sampled_token(42)
+    assert state.status is D
+
+
+def test_preemption_keeps_tokens_and_runs_them_again():
+    state = SequenceState.from_request(request(max_new_tokens=5))
+    state.begin_prefill()
+    state.commit_prefill(3)
+    state.append_sampled_token(42)
+    state.mark_decode_input_computed()
+    state.append_sampled_token(43)
+    state.preempt()
+    snapshot = state.snapshot()
+    assert snapshot.status is W and snapshot.prefill_target == 5 and snapshot.computed_tokens == 0
+    assert snapshot.num_generated == 2 and snapshot.num_preemptions == 1
+    state.begin_prefill()
+    state.commit_prefill(5)
+    state.append_sampled_token(44)
+    assert state.all_tokens == (10, 20, 30, 42, 43, 44) and state.status is D
+
+
+def test_plan_checks():
+    # reference: tests/unit/test_sequence_state.py:107-138
+    ExecutionPlan(0, (PrefillItem("r", 0, 3),), (), 3)
+    with pytest.raises(ValueError, match="does not match"):
+        ExecutionPlan(2, (PrefillItem("r", 0, 2),), (), 1)
+    with pytest.raises(TypeError, match="immutable tuples"):
+        ExecutionPlan(0, [PrefillItem("r", 0, 1)], (), 1)
+    with pytest.raises(ValueError, match="only once"):
+        ExecutionPlan(0, (PrefillItem("r", 0, 1),), (DecodeItem("r", 1, 1),), 2)
+    with pytest.raises(ValueError, match="same step"):
+        ExecutionPlan(0, (PrefillItem("r", 0, 1),), (), 1, preempted=("r",))
+    for invalid in (True, 1.5):
+        with pytest.raises(ValueError):
+            DecodeItem("r", invalid, 0)
+
+
+# ---- decisions -------------------------------------------------------------------------
+
+def test_decode_first_then_prompts_in_arrival_order():
+    views = [
+        view("late-waiting", W, arrival=5, target=6),
+        view("decoding-b", D, arrival=2, generated=1),
+        view("early-waiting", W, arrival=3, target=9),
+        view("decoding-a", D, arrival=1, generated=2),
+    ]
+    plan = scheduler().schedule(views, capacity(40))
+    assert [i.request_id for i in plan.decode_items] == ["decoding-a", "decoding-b"]
+    assert plan.decode_items[0].position == 11 and plan.decode_items[0].input_token_id == 7
+    assert [(i.request_id, i.token_start, i.token_end) for i in plan.prefill_items] == [
+        ("early-waiting", 0, 9), ("late-waiting", 0, 6),
+    ]
+    assert plan.scheduled_tokens == 17 and plan.preempted == ()
+
+
+def test_same_arrival_is_ordered_by_id_and_the_function_is_pure():
+    views = [view("b", W, target=20), view("a", W, target=20)]
+    first = scheduler(max_num_batched_tokens=25).schedule(views, capacity(40))
+    second = scheduler(max_num_batched_tokens=25).schedule(list(reversed(views)), capacity(40))
+    assert first == second
+    assert [i.request_id for i in first.prefill_items] == ["a"]      # whole prompts only: b does not fit
+
+
+def test_token_budget_and_portions():
+    views = [view("a", W, target=50), view("b", W, arrival=1, target=10)]
+    whole = scheduler().schedule(views, capacity(40))
+    assert [(i.request_id, i.token_end) for i in whole.prefill_items] == [("b", 10)]   # a never fits unchunked
+    chunked = scheduler(enable_chunked_prefill=True).schedule(views, capacity(40))
+    assert [(i.request_id, i.token_start, i.token_end) for i in chunked.prefill_items] == [("a", 0, 32)]
+    sized = scheduler(enable_chunked_prefill=True, prefill_chunk_size=7).schedule(views, capacity(40))
+    assert [(i.request_id, i.token_end) for i in sized.prefill_items] == [("a", 7), ("b", 7)]
+    resumed = scheduler(enable_chunked_prefill=True, prefill_chunk_size=7).schedule(
+        [view("a", P, target=50, cursor=49)], capacity(40)
+    )
+    assert [(i.token_start, i.token_end) for i in resumed.prefill_items] == [(49, 50)]   # a portion of one token
+
+
+def test_decoding_cannot_starve_a_prompt_when_portions_are_allowed():
+    # reference: miniserve/engine/scheduler.py:150-164
+    views = [view(f"d{i}", D, arrival=i, generated=1) for i in range(4)] + [view("p", W, arrival=9, target=30)]
+    plan = scheduler(max_num_batched_tokens=4, enable_chunked_prefill=True).schedule(views, capacity(40))
+    assert len(plan.decode_items) == 3 and [(i.request_id, i.token_end) for i in plan.prefill_items] == [("p", 1)]
+    plain = scheduler(max_num_batched_tokens=4).schedule(views, capacity(40))
+    assert len(plain.decode_items) == 4 and plain.prefill_items == ()
+
+
+def test_portion_shrinks_to_the_pages_that_are_free():
+    # 2 free pages of 4 and 1 token of room in the request's last page
+    plan = scheduler(enable_chunked_prefill=True).schedule([view("a", P, target=40, cursor=7)], capacity(2))
+    assert [(i.token_start, i.token_end) for i in plan.prefill_items] == [(7, 16)]
+    none = scheduler(enable_chunked_prefill=True).schedule([view("a", W, target=40)], capacity(0))
+    assert none.empty
+    whole = scheduler().schedule([view("a", W, target=40)], capacity(2))
+    assert whole.empty                                            # whole prompts are not cut
+
+
+def test_waiting_requests_need_a_state_slot():
+    views = [view("a", W, target=4), view("b", W, arrival=1, target=4)]
+    plan = scheduler().schedule(views, capacity(40, free_slots=1))
+    assert [i.request_id for i in plan.prefill_items] == ["a"]
+    capped = scheduler(max_num_seqs=2).schedule([view("x", D, generated=1), view("y", D, arrival=1, generated=1)] + views,
+                                                capacity(40, free_slots=3))
+    assert capped.prefill_items == ()
+
+
+def test_out_of_pages_preempts_the_youngest_running_request():
+    # every request stands at a page edge (computed 12 = 3 pages of 4) and needs a new page; none is free
+    views = [view(n, D, arrival=i, target=10, generated=3) for i, n in enumerate(("old", "mid", "young"))]
+    held = {"old": (3,), "mid": (3,), "young": (3,)}
+    plan = scheduler().schedule(views, capacity(0, held=held))
+    assert plan.preempted == ("young",)
+    assert [i.request_id for i in plan.decode_items] == ["old", "mid"]
+    # with one free page nobody is preempted but the last one in line waits
+    plan = scheduler().schedule(views, capacity(1, held=held))
+    assert plan.preempted == ("young",) and [i.request_id for i in plan.decode_items] == ["old", "mid"]
+    plan = scheduler().schedule(views, capacity(3, held=held))
+    assert plan.preempted == () and len(plan.decode_items) == 3
+
+
+def test_the_oldest_is_never_preempted_and_waiting_requests_preempt_nobody():
+    alone = [view("old", D, target=10, generated=3)]
+    plan = scheduler().schedule(alone, capacity(0, held={"old": (3,)}))
+    assert plan.preempted == () and plan.empty                      # it waits; nothing younger exists
+    views = [view("run", D, arrival=5, target=10, generated=3), view("new", W, arrival=0, target=8)]
+    plan = scheduler().schedule(views, capacity(1, held={"run": (3,)}))
+    assert plan.preempted == () and [i.request_id for i in plan.decode_items] == ["run"]
+    assert plan.prefill_items == ()                                  # no page left for the older waiting request
+
+
+def test_a_prompt_in_progress_may_preempt_a_younger_one_but_not_one_already_scheduled():
+    views = [view("older", P, arrival=0, target=40, cursor=8), view("younger", P, arrival=1, target=40, cursor=8)]
+    held = {"older": (2,), "younger": (2,)}
+    plan = scheduler(enable_chunked_prefill=True, prefill_chunk_size=8).schedule(views, capacity(0, held=held))
+    assert plan.preempted == ("younger",)
+    assert [(i.request_id, i.token_start, i.token_end) for i in plan.prefill_items] == [("older", 8, 16)]
+    views = [view("older", P, arrival=0, target=40, cursor=8), view("younger", D, arrival=1, target=7, generated=1)]
+    plan = scheduler(enable_chunked_prefill=True, prefill_chunk_size=8).schedule(views, capacity(0, held=held))
+    assert plan.preempted == () and [i.request_id for i in plan.decode_items] == ["younger"]
+    assert plan.prefill_items == ()
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_budgets_hold_for_random_views(seed):
+    rng = random.Random(seed)
+    for _ in range(60):
+        views, held = [], {}
+        for index in range(rng.randint(1, 9)):
+            status = rng.choice((W, P, D))
+            target = rng.randint(1, 40)
+            cursor = 0 if status is W else (rng.randint(1, target) - 1 if status is P else target)
+            generated = rng.randint(1, 5) if status is D else 0
+            v = view(f"r{index}", status, target=target, cursor=cursor, generated=generated, arrival=rng.randint(0, 4))
+            views.append(v)
+            if status is not W:
+                held[v.request_id] = (-(-v.computed_tokens // 4),)
+        free = rng.randint(0, 12)
+        budget = rng.randint(1, 24)
+        chunked = rng.random() < 0.5
+        running = sum(1 for v in views if v.status is not W)
+        plan = Scheduler(max_num_seqs=8, max_num_batched_tokens=budget, enable_chunked_prefill=chunked).schedule(
+            views, capacity(free, free_slots=8 - running, held=held)
+        )
+        assert plan.scheduled_tokens <= budget
+        by_id = {v.request_id: v for v in views}
+        pages = sum(held[r][0] for r in plan.preempted) + free
+        for item in plan.decode_items:
+            v = by_id[item.request_id]
+            pages -= -(-(v.computed_tokens + 1) // 4) - -(-v.computed_tokens // 4)
+        for item in plan.prefill_items:
+            v = by_id[item.request_id]
+            assert item.token_start == v.prefill_cursor and item.token_end <= v.prefill_target
+            if not chunked:
+                assert item.token_end == v.prefill_target
+            pages -= -(-item.token_end // 4) - -(-item.token_start // 4)
+        assert pages >= 0
+        oldest_running = min((v for v in views if v.status is not W), key=lambda v: (v.arrival_ns, v.request_id), default=None)
+        if oldest_running is not None:
+            assert oldest_running.request_id not in plan.preempted
+        assert all(by_id[r].status is not W for r in plan.preempted)
+
+
+# ---- the engine loop with a stand-in runner ---------------------------------------------
+
+def make_engine(**options):
+    base = dict(dtype="float32", kv_block_size=4, num_kv_blocks=64, max_num_seqs=4, max_model_len=128)
+    base.update(options)
+    fail = base.pop("fail_on_step", None)
+    runner = FakeRunner(EngineConfig(**base), fail_on_step=fail)
+    return Engine(runner, sampler=ArgmaxSampler()), runner
+
+
+PROMPTS = [[3, 1, 4, 1, 5], list(range(17)), list(range(40, 73)), [9]]
+
+
+def test_generate_is_the_same_whatever_the_scheduling():
+    expected = [expected_generation(p, 12, 97) for p in PROMPTS]
+    params = SamplingParams(max_new_tokens=12)
+    roomy, _ = make_engine()
+    assert roomy.generate(PROMPTS, params) == expected
+    chunked, runner = make_engine(enable_chunked_prefill=True, prefill_chunk_size=7, max_num_batched_tokens=16)
+    assert chunked.generate(PROMPTS, params) == expected
+    assert any(len(step) > 1 for step in runner.steps)                 # portions ran beside decoded tokens
+    # so few pages that requests are preempted and run again: 14 pages of 4 for 4 requests of up to 45 tokens
+    tight, runner = make_engine(num_kv_blocks=14, enable_chunked_prefill=True, max_num_batched_tokens=64)
+    assert tight.generate(PROMPTS, params) == expected
+    assert tight.counters["preemptions"] > 0
+    assert runner.cache.capacity().free_blocks == (14,) and runner.cache.capacity().free_slots == 4
+    runner.cache.assert_invariants()
+
+
+def test_stop_tokens_and_per_request_parameters():
+    engine, _ = make_engine()
+    first = expected_generation(PROMPTS[0], 12, 97)
+    stop = first[3]
+    params = [SamplingParams(max_new_tokens=12, stop_token_ids=(stop,)), SamplingParams(max_new_tokens=2)]
+    out = engine.generate(PROMPTS[:2], params)
+    assert out[0] == first[: first.index(stop) + 1] and out[1] == expected_generation(PROMPTS[1], 2, 97)
+
+
+def test_admission_checks():
+    # reference: miniserve/engine/core.py:193-236
+    engine, _ = make_engine(num_kv_blocks=8)
+    engine.add_request("a", [1, 2, 3])
+    with pytest.raises(ValueError, match="Duplicate"):
+        engine.add_request("a", [1])
+    with pytest.raises(ValueError, match="CONTEXT_LENGTH_EXCEEDED"):
+        engine.add_request("b", [1] * 120, SamplingParams(max_new_tokens=9))
+    with pytest.raises(ValueError, match="CONTEXT_CAPACITY_EXCEEDED"):
+        engine.add_request("c", [1] * 30, SamplingParams(max_new_tokens=8))
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        engine.add_request("d", [97])
+    with pytest.raises(ValueError, match="top_k"):
+        engine.add_request("e", [1], SamplingParams(temperature=1.0, top_k=98))
+    with pytest.raises(ValueError, match="stop token"):
+        engine.add_request("f", [1], SamplingParams(stop_token_ids=(500,)))
+    small, _ = make_engine(max_num_batched_tokens=16)
+    with pytest.raises(ValueError, match="CHUNKED_PREFILL_DISABLED"):
+        small.add_request("g", [1] * 20)
+    full, _ = make_engine(max_pending_requests=1)
+    full.add_request("h", [1])
+    with pytest.raises(RuntimeError, match="QUEUE_FULL"):
+        full.add_request("i", [1])
+
+
+def test_a_failed_step_leaves_no_trace_and_fails_its_requests():
+    engine, runner = make_engine(fail_on_step=1)
+    engine.add_request("a", [1, 2, 3], SamplingParams(max_new_tokens=4), arrival_ns=0)
+    engine.step()
+    with pytest.raises(RuntimeError, match="injected"):
+        engine.step()
+    assert engine.pop_result("a").finish_reason == "error"
+    assert runner.cache.capacity().free_blocks == (64,) and runner.cache.live_requests() == ()
+    engine.add_request("b", [1, 2, 3], SamplingParams(max_new_tokens=4), arrival_ns=1)
+    while engine.has_unfinished():
+        engine.step()
+    assert list(engine.pop_result("b").token_ids) == expected_generation([1, 2, 3], 4, 97)
+
+
+def test_cancel_gives_everything_back():
+    engine, runner = make_engine()
+    engine.add_request("a", list(range(9)), SamplingParams(max_new_tokens=5))
+    engine.step()
+    engine.cancel("a")
+    assert runner.cache.capacity().free_blocks == (64,) and not engine.has_unfinished()
+    assert engine.pop_result("a").finish_reason == "cancelled"
