@@ -1,0 +1,207 @@
+"""Generation through the entry point on the GPU: greedy against the plain
+implementation, sampling with seeds, long decoding, too few pages, the command
+line, and toy parts and architectures that are registered from outside."""
+
+from __future__ import annotations
+
+import json
+import subprocess
+import sys
+
+import plain_qwen3 as plain
+import plain_sampling
+import pytest
+import torch
+from helpers import ROOT, random_tokens, read_config, read_weights
+
+pytestmark = pytest.mark.gpu
+
+DEVICE = "cuda:0"
+# a greedy token may differ from the oracle's only where the two best logits are this close
+# (the reference's near-tie rule: miniserve/benchmark/compare_hf.py:369, margin <= 2 * max error)
+NEAR_TIE = {"float32": 4e-5, "bfloat16": 5e-2}
+
+
+def rounded(weights, dtype):
+    if dtype == "bfloat16":
+        return {k: v.to(torch.bfloat16).float() for k, v in weights.items()}
+    return weights
+
+
+def check_greedy(got, prompt, weights, config, dtype):
+    want, margins = plain.greedy_generate(weights, config, prompt, len(got))
+    for index, (a, b) in enumerate(zip(got, want)):
+        if a != b:
+            assert margins[index] <= NEAR_TIE[dtype], f"token {index} after a prompt of {len(prompt)}: {a} != {b}"
+            return index          # later tokens follow another prefix
+    return len(got)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_tiny_a(dtype, model_folders):
+    """BASELINE configuration Tiny A: prompts of 5, 17 and 33 tokens, 8 greedy tokens each."""
+
+    from miniserve_amd.engine import SamplingParams
+    from miniserve_amd.entrypoint import LLM
+
+    folder, block = model_folders["a"]
+    config, weights = read_config(folder), rounded(read_weights(folder), dtype)
+    prompts = [random_tokens(n, config["vocab_size"], 200 + n) for n in (5, 17, 33)]
+    llm = LLM(str(folder), dtype=dtype, kv_block_size=block, num_kv_blocks=16, max_num_seqs=4)
+    got = llm.generate(prompts, SamplingParams(max_new_tokens=8))
+    assert [len(tokens) for tokens in got] == [8, 8, 8]
+    agreed = [check_greedy(tokens, prompt, weights, config, dtype) for tokens, prompt in zip(got, prompts)]
+    if dtype == "float32":
+        assert agreed == [8, 8, 8]
+    cache = llm.runner.cache
+    assert cache.live_requests() == () and cache.capacity().free_blocks == (16,)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_chunked_prefill_mixed_with_decode_tiny_b(dtype, model_folders):
+    """BASELINE configuration Tiny B: prompts of 1, 9, 24 and 40 tokens, portions of
+    7 mixed with decoding; greedy, then temperature 0.8 from seed 0."""
+
+    from miniserve_amd.engine import SamplingParams
+    from miniserve_amd.entrypoint import LLM
+    from miniserve_amd.sampling import Sampler
+
+    folder, block = model_folders["b"]
+    config, weights = read_config(folder), rounded(read_weights(folder), dtype)
+    prompts = [random_tokens(n, config["vocab_size"], 300 + n) for n in (1, 9, 24, 40)]
+    llm = LLM(str(folder), dtype=dtype, kv_block_size=block, num_kv_blocks=40, max_num_seqs=4,
+              enable_chunked_prefill=True, prefill_chunk_size=7, max_num_batched_tokens=16)
+    got = llm.generate(prompts, SamplingParams(max_new_tokens=10))
+    for tokens, prompt in zip(got, prompts):
+        check_greedy(tokens, prompt, weights, config, dtype)
+    assert llm.engine.counters["prefill_tokens"] == sum(len(p) for p in prompts)
+    whole = LLM(str(folder), dtype=dtype, kv_block_size=block, num_kv_blocks=40, max_num_seqs=4)
+    again = whole.generate(prompts, SamplingParams(max_new_tokens=10))
+    if dtype == "float32":
+        assert again == got               # the way the work is cut does not change a token
+
+    # temperature 0.8, seed 0: every token is the plain sampler's choice for the engine's own
+    # logits at that step... checked through the oracle's logits where the draw is not at an edge
+    params = SamplingParams(temperature=0.8, max_new_tokens=6, seed=0)
+    sampled = llm.generate(prompts, params)
+    assert sampled == llm.generate(prompts, params)                               # a seed fixes the stream
+    assert sampled != llm.generate(prompts, SamplingParams(temperature=0.8, max_new_tokens=6, seed=1))
+    if dtype == "float32":
+        for prompt, tokens in zip(prompts, sampled):
+            stream = torch.Generator().manual_seed(0)
+            sequence = list(prompt)
+            for token in tokens:
+                logits = plain.forward_logits(weights, config, sequence)[-1].float()
+                uniform = Sampler.draw_uniform(stream)
+                probabilities = torch.softmax(logits.double() / 0.8, dim=-1)
+                edges = torch.cumsum(probabilities, dim=-1)
+                if float((edges - uniform).abs().min()) < 1e-4:
+                    break                                                         # a draw on an edge may fall either way
+                assert token == plain_sampling.sample_row(logits, 0.8, 0, 1.0, uniform)
+                sequence.append(token)
+
+
+def test_long_decoding(model_folders):
+    """Hundreds of decoded tokens past several page edges, compared at the end and
+    on the way with the oracle's logits (teacher-forced, so a near tie cannot derail it)."""
+
+    from miniserve_amd.config import EngineConfig
+    from miniserve_amd.engine import ModelRunner, StepEntry
+
+    folder, block = model_folders["a"]
+    config, weights = read_config(folder), read_weights(folder)
+    tokens = random_tokens(400, config["vocab_size"], 77)
+    runner = ModelRunner.from_folder(folder, EngineConfig(dtype="float32", kv_block_size=block, num_kv_blocks=26, decode_graphs=False))
+    expected = plain.forward_logits(weights, config, tokens).float()
+    runner.admit("long")
+    rows = [runner.step([StepEntry("long", tuple(tokens[:3]), (2,))]).cpu()]
+    for position in range(3, 400):
+        rows.append(runner.step([StepEntry("long", (tokens[position],), (0,))]).cpu())
+    got = torch.cat(rows)
+    error = (got - expected[2:]).abs().max(dim=-1).values
+    assert float(error.max()) <= 2e-5, f"first wrong position {2 + int((error > 2e-5).nonzero()[0])}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sharp_attention_over_hundreds_of_tokens(dtype, model_folders, tmp_path):
+    """With random weights attention is nearly uniform and a lost far key would hide.
+    Here the q/k norm weights are scaled so that scores are 16 times larger: weights
+    concentrate on single, often far, keys."""
+
+    from safetensors.torch import save_file
+
+    from miniserve_amd.config import EngineConfig
+    from miniserve_amd.engine import ModelRunner, StepEntry
+
+    folder, block = model_folders["b"]
+    config, weights = read_config(folder), dict(read_weights(folder))
+    for name in weights:
+        if name.endswith("q_norm.weight") or name.endswith("k_norm.weight"):
+            weights[name] = weights[name] * 4.0
+        if name.endswith("v_proj.weight") or name.endswith("o_proj.weight"):
+            weights[name] = weights[name] * 4.0
+    sharp = tmp_path / "sharp"
+    sharp.mkdir()
+    (sharp / "config.json").write_text(json.dumps(config))
+    save_file(weights, str(sharp / "model.safetensors"))
+    tokens = random_tokens(700, config["vocab_size"], 5)
+    oracle = rounded(weights, dtype)
+    expected = plain.forward_logits(oracle, config, tokens).float()
+    uniform = plain.forward_logits(rounded(read_weights(folder), dtype), config, tokens).float()
+    assert float((expected - uniform).abs().max()) > 0.05                         # the scaling matters
+    runner = ModelRunner.from_folder(sharp, EngineConfig(dtype=dtype, kv_block_size=block, num_kv_blocks=100,
+                                                        enable_chunked_prefill=True, decode_graphs=False))
+    runner.admit("s")
+    rows, position = [], 0
+    for size in (300, 2, 255, 100, 11) + (1,) * 32:
+        part = tokens[position : position + size]
+        rows.append(runner.step([StepEntry("s", tuple(part), tuple(range(len(part))))]).cpu())
+        position += size
+    assert position == 700
+    # Scores 16 times larger carry 16 times the absolute rounding.  The yardstick is the
+    # plain implementation itself in the reduced arithmetic (float32; or every intermediate
+    # rounded to bfloat16 where the reference rounds) against its float64 form: the engine
+    # may be off by three times that, no more.
+    if dtype == "float32":
+        reduced = plain.forward_logits(oracle, config, tokens, dtype=torch.float32)
+    else:
+        reduced = plain.forward_logits(oracle, config, tokens, rd=torch.bfloat16)
+    natural = float((reduced - expected).abs().max())
+    tolerance = 3 * natural
+    print(f"sharp {dtype}: rounding of the plain form {natural:.2e}, tolerance {tolerance:.2e}", flush=True)
+    error = (torch.cat(rows) - expected).abs().max(dim=-1).values
+    assert float(error.max()) <= tolerance, f"first wrong position {int((error > tolerance).nonzero()[0])}"
+
+
+def test_too_few_pages_preempt_and_still_give_the_same_tokens(model_folders):
+    from miniserve_amd.engine import SamplingParams
+    from miniserve_amd.entrypoint import LLM
+
+    folder, block = model_folders["a"]
+    config = read_config(folder)
+    prompts = [random_tokens(n, config["vocab_size"], 400 + n) for n in (30, 41, 18, 25)]
+    params = SamplingParams(max_new_tokens=24)
+    roomy = LLM(str(folder), dtype="float32", kv_block_size=block, num_kv_blocks=32, max_num_seqs=4)
+    expected = roomy.generate(prompts, params)
+    tight = LLM(str(folder), dtype="float32", kv_block_size=block, num_kv_blocks=9, max_num_seqs=4,
+                enable_chunked_prefill=True)
+    assert tight.generate(prompts, params) == expected
+    assert tight.engine.counters["preemptions"] > 0
+    assert tight.runner.cache.capacity().free_blocks == (9,)
+    tight.runner.cache.assert_invariants()
+
+
+def test_command_line(model_folders):
+    folder, block = model_folders["a"]
+    config, weights = read_config(folder), read_weights(folder)
+    process = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "miniserve-generate"), "--model", str(folder), "--dtype", "float32",
+         "--kv-block-size", str(block), "--num-kv-blocks", "16", "--prompt-ids", "5,9,200,31", "--prompt-ids", "7",
+         "--max-new-tokens", "5"],
+        capture_output=True, text=True, timeout=300,
+    )
+    assert process.returncode == 0, process.stderr[-2000:]
+    lines = [json.loads(line) for line in process.stdout.strip().splitlines()]
+    assert [line["prompt_token_ids"] for line in lines] == [[5, 9, 200, 31], [7]]
+    for line in lines:
+        assert check_greedy(line["token_ids"], line["prompt_token_ids"], weights, config, "float32") == 5

@@ -1,0 +1,482 @@
+"""Each kernel alone against a plain torch reference, at other sizes than the
+engine's: around the wave (63/64/65) and workgroup edges, head sizes in steps of
+16, widths and vocabularies that are no power of two (the reference tests its op
+at 1, 31, 32, 33, 257, 1024, 1031: tests/cuda_extension/test_vector_add.py:23)."""
+
+from __future__ import annotations
+
+import math
+
+import plain_qwen3 as plain
+import plain_sampling
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEVICE = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def rand(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    generator = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=generator) * scale).to(dtype).to(DEVICE)
+
+
+def tolerance(dtype, f32=2e-5, bf16=4e-3):
+    # the reference's own tolerances: 2e-5 float32 / 4e-3 half for the norm
+    # (miniserve/toolchain/benchmark_rmsnorm.py:73), 2e-4 / 8e-3 for attention
+    return f32 if dtype == torch.float32 else bf16
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from miniserve_amd import ops as module
+
+    module.load()
+    assert module.library_path().endswith("libminiserve_hip.so")
+    return module
+
+
+# ---- embedding --------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [1, 63, 64, 65, 257, 1031])
+def test_embedding_gather(ops, dtype, hidden):
+    table = rand(509, hidden, seed=hidden, dtype=dtype)
+    ids = torch.tensor([0, 508, 3, 3, 77, 256], dtype=torch.int32, device=DEVICE)
+    out = ops.embedding_gather(ids, table)
+    assert out.dtype == torch.float32
+    assert torch.equal(out, table[ids.long()].float())
+
+
+# ---- RMSNorm ----------------------------------------------------------------------------
+
+def rmsnorm_reference(x, weight, eps, storage):
+    """32-bit statistics, round to storage, multiply by the weight (layers.py:30-34)."""
+
+    values = x.double()
+    normed = (values * torch.rsqrt(values.pow(2).mean(-1, keepdim=True) + eps)).to(storage)
+    return (weight.double() * normed.double()).to(storage)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(1, 1024), (7, 1024), (33, 1024), (4, 4096), (3, 1), (5, 63), (5, 65), (2, 96), (9, 5120), (2, 1031)])
+def test_rmsnorm_shapes_of_the_reference_and_edges(ops, dtype, shape):
+    # reference shapes: miniserve/toolchain/benchmark_rmsnorm.py:97, seed 7000 + rows + hidden (:68)
+    rows, dim = shape
+    x = rand(rows, dim, seed=7000 + rows + dim, dtype=dtype)
+    weight = torch.linspace(0.5, 1.5, dim).to(dtype).to(DEVICE)
+    out = ops.rmsnorm(x, weight, 1e-6)
+    expected = rmsnorm_reference(x, weight, 1e-6, dtype)
+    torch.testing.assert_close(out.double(), expected.double(), atol=tolerance(dtype), rtol=tolerance(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_residual_forms(ops, dtype):
+    residual = rand(6, 200, seed=1)
+    delta = rand(6, 200, seed=2, dtype=dtype)
+    weight = (1 + 0.1 * rand(200, seed=3)).to(dtype)
+    total = residual + delta.float()
+    kept = residual.clone()
+    out = ops.rmsnorm(kept, weight, 1e-5, delta=delta, write_back=True)
+    assert torch.equal(kept, total)                                             # h <- h + delta in 32-bit
+    expected = rmsnorm_reference(total, weight, 1e-5, dtype)
+    torch.testing.assert_close(out.double(), expected.double(), atol=tolerance(dtype), rtol=tolerance(dtype))
+    rows = torch.tensor([5, 0, 3], dtype=torch.int32, device=DEVICE)
+    kept = residual.clone()
+    picked = ops.rmsnorm(kept, weight, 1e-5, delta=delta, rows=rows)
+    assert torch.equal(kept, residual)                                          # gathered rows write nothing back
+    assert torch.equal(picked, out[rows.long()])
+    # a row's result does not depend on the batch around it
+    alone = ops.rmsnorm(residual[2:3].clone(), weight, 1e-5, delta=delta[2:3].contiguous(), write_back=True)
+    assert torch.equal(alone[0], out[2])
+
+
+def test_rmsnorm_vector_of_the_reference(ops):
+    # tests/correctness/test_rmsnorm_reference.py:23-32
+    values = torch.tensor([[0.0, 1.0, -1.0, 1e-4, -1e-4, 8.0, -8.0, 2.0]], device=DEVICE)
+    weight = torch.linspace(0.75, 1.25, 8, device=DEVICE)
+    expected = plain.rms_norm(values.cpu().double(), weight.cpu().double(), 1e-6)
+    torch.testing.assert_close(ops.rmsnorm(values, weight, 1e-6).cpu().double(), expected, atol=1e-6, rtol=1e-6)
+
+
+def test_kernels_refuse_what_they_cannot_do(ops):
+    from miniserve_amd.ops import KernelError
+
+    x = rand(4, 64)
+    with pytest.raises(KernelError, match="GPU"):
+        ops.rmsnorm(x.cpu(), torch.ones(64), 1e-6)
+    with pytest.raises(KernelError, match="does not match"):
+        ops.rmsnorm(x, torch.ones(65, device=DEVICE), 1e-6)
+    with pytest.raises(KernelError, match="float32 or bfloat16"):
+        ops.silu_mul(x.half())
+    with pytest.raises(KernelError, match="eps"):
+        ops.rmsnorm(x, torch.ones(64, device=DEVICE), 0.0)
+    with pytest.raises(KernelError, match="contiguous"):
+        ops.silu_mul(x.t())
+    with pytest.raises(KernelError, match="exceeds"):
+        ops.qk_norm_rope_append(rand(1, 1026), num_q_heads=1, num_kv_heads=0, head_dim=1026, q_weight=None,
+                                k_weight=None, eps=1.0, inv_freq=None, positions=None)
+    with pytest.raises(KernelError, match="even"):
+        ops.qk_norm_rope_append(rand(1, 15), num_q_heads=1, num_kv_heads=0, head_dim=15, q_weight=None,
+                                k_weight=None, eps=1.0, inv_freq=None, positions=None)
+
+
+# ---- q/k norm, rotation, cache write ------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,block", [(4, 2, 16, 16), (8, 1, 32, 8), (3, 3, 48, 5), (16, 8, 128, 16), (2, 1, 256, 4), (5, 1, 80, 3)])
+def test_qk_norm_rope_append(ops, dtype, heads, kv_heads, dim, block):
+    from miniserve_amd.parts.rotary import inverse_frequencies
+
+    n, pages, theta, eps = 11, 9, 50000.0, 1e-5
+    packed = rand(n, (heads + 2 * kv_heads) * dim, seed=dim, dtype=dtype)
+    qw = (1 + 0.1 * rand(dim, seed=1)).to(dtype)
+    kw = (1 + 0.1 * rand(dim, seed=2)).to(dtype)
+    positions = torch.tensor([0, 1, 2, 63, 64, 65, 1000, 4095, 7, 7, 30000], dtype=torch.int32, device=DEVICE)
+    slots = torch.randperm(pages * block, generator=torch.Generator().manual_seed(3))[:n].to(torch.int32).to(DEVICE)
+    key_pool = torch.zeros(pages, kv_heads, block, dim, dtype=dtype, device=DEVICE)
+    value_pool = torch.zeros_like(key_pool)
+    q = ops.qk_norm_rope_append(
+        packed, num_q_heads=heads, num_kv_heads=kv_heads, head_dim=dim, q_weight=qw, k_weight=kw, eps=eps,
+        inv_freq=inverse_frequencies(dim, theta).to(DEVICE), positions=positions, slot_mapping=slots,
+        key_pool=key_pool, value_pool=value_pool,
+    )
+    rows = packed.cpu().double().view(n, heads + 2 * kv_heads, dim)
+    cos, sin = plain.rope_angles(positions.cpu().long(), dim, theta)
+
+    def prepare(x, weight):
+        normed = rmsnorm_reference(x, weight.cpu(), eps, dtype).double()
+        return plain.apply_rope(normed.transpose(0, 1), cos, sin).transpose(0, 1)
+
+    expected_q = prepare(rows[:, :heads], qw)
+    expected_k = prepare(rows[:, heads : heads + kv_heads], kw)
+    expected_v = rows[:, heads + kv_heads :]
+    tol = tolerance(dtype, 1e-5, 1.6e-2)         # one bfloat16 rounding of values up to ~4
+    torch.testing.assert_close(q.cpu().double(), expected_q, atol=tol, rtol=tol)
+    page, offset = slots.cpu().long() // block, slots.cpu().long() % block
+    torch.testing.assert_close(key_pool.cpu().double()[page, :, offset], expected_k, atol=tol, rtol=tol)
+    assert torch.equal(value_pool.cpu().double()[page, :, offset], expected_v)
+    touched = torch.zeros(pages, block, dtype=torch.bool)
+    touched[page, offset] = True
+    untouched = lambda pool: pool.cpu().permute(0, 2, 1, 3)[~touched]
+    assert torch.all(untouched(key_pool) == 0) and torch.all(untouched(value_pool) == 0)
+
+
+def test_rotation_and_norm_alone(ops):
+    """Without weights the kernel is the rotation alone; without frequencies the norm alone."""
+
+    from miniserve_amd.parts.rotary import inverse_frequencies
+
+    x = rand(5, 3 * 32, seed=9)
+    positions = torch.tensor([0, 3, 9, 100, 511], dtype=torch.int32, device=DEVICE)
+    only_rope = ops.qk_norm_rope_append(x, num_q_heads=3, num_kv_heads=0, head_dim=32, q_weight=None, k_weight=None,
+                                        eps=1.0, inv_freq=inverse_frequencies(32, 1e4).to(DEVICE), positions=positions)
+    cos, sin = plain.rope_angles(positions.cpu().long(), 32, 1e4)
+    expected = plain.apply_rope(x.cpu().double().view(5, 3, 32).transpose(0, 1), cos, sin).transpose(0, 1)
+    torch.testing.assert_close(only_rope.cpu().double(), expected, atol=1e-5, rtol=1e-5)
+    assert torch.equal(only_rope[0], x.view(5, 3, 32)[0])                       # position 0 is the identity
+    weight = 1 + 0.1 * rand(32, seed=4)
+    only_norm = ops.qk_norm_rope_append(x, num_q_heads=3, num_kv_heads=0, head_dim=32, q_weight=weight, k_weight=None,
+                                        eps=1e-6, inv_freq=None, positions=None)
+    torch.testing.assert_close(only_norm.view(15, 32), ops.rmsnorm(x.view(15, 32), weight, 1e-6), atol=1e-6, rtol=1e-6)
+
+
+# ---- attention over the paged cache -------------------------------------------------------
+
+def paged_case(batch_contexts, heads, kv_heads, dim, block, dtype, *, query_lens=None, seed=0, reverse=True):
+    """Random q and cache for sequences of the given context lengths; each sequence
+    brings ``query_lens[i]`` last positions as queries.  Pages are handed out in
+    reversed order so that physical order differs from logical order, as the
+    reference's own check does (miniserve/toolchain/benchmark_paged_decode.py:26-60)."""
+
+    generator = torch.Generator().manual_seed(seed)
+    query_lens = query_lens or [1] * len(batch_contexts)
+    blocks_each = [-(-c // block) for c in batch_contexts]
+    total = sum(blocks_each) + 2
+    order = list(range(total - 1, -1, -1)) if reverse else list(range(total))
+    key_pool = torch.full((total, kv_heads, block, dim), float("nan"))
+    value_pool = torch.full((total, kv_heads, block, dim), float("nan"))
+    table = torch.zeros(len(batch_contexts), max(blocks_each), dtype=torch.int32)
+    keys, values, queries, seq_of_token, positions = [], [], [], [], []
+    cursor = 0
+    for index, (context, qlen) in enumerate(zip(batch_contexts, query_lens)):
+        k = torch.randn(context, kv_heads, dim, generator=generator).to(dtype).float()
+        v = torch.randn(context, kv_heads, dim, generator=generator).to(dtype).float()
+        q = torch.randn(qlen, heads, dim, generator=generator).to(dtype).float()
+        for logical in range(blocks_each[index]):
+            page = order[cursor]
+            cursor += 1
+            table[index, logical] = page
+            span = slice(logical * block, min((logical + 1) * block, context))
+            key_pool[page, :, : span.stop - span.start] = k[span].transpose(0, 1)
+            value_pool[page, :, : span.stop - span.start] = v[span].transpose(0, 1)
+        keys.append(k)
+        values.append(v)
+        queries.append(q)
+        seq_of_token += [index] * qlen
+        positions += list(range(context - qlen, context))
+    return {
+        "q": torch.cat(queries).to(dtype).to(DEVICE),
+        "key_pool": key_pool.to(dtype).to(DEVICE),
+        "value_pool": value_pool.to(dtype).to(DEVICE),
+        "block_table": table.to(DEVICE),
+        "seq_of_token": torch.tensor(seq_of_token, dtype=torch.int32, device=DEVICE),
+        "positions": torch.tensor(positions, dtype=torch.int32, device=DEVICE),
+        "keys": keys, "values": values, "queries": queries, "query_lens": query_lens,
+    }
+
+
+def attention_reference(case, scale, window=None):
+    outs = []
+    for k, v, q in zip(case["keys"], case["values"], case["queries"]):
+        context, qlen = k.shape[0], q.shape[0]
+        padded = torch.zeros(context, q.shape[1], q.shape[2], dtype=torch.float64)
+        padded[context - qlen :] = q.double()
+        full = plain.causal_attention(padded.transpose(0, 1), k.double().transpose(0, 1), v.double().transpose(0, 1), scale, window)
+        outs.append(full.transpose(0, 1)[context - qlen :])
+    return torch.cat(outs)
+
+
+def run_attention(ops, case, scale, window=None):
+    return ops.attention(case["q"], case["key_pool"], case["value_pool"], block_table=case["block_table"],
+                         seq_of_token=case["seq_of_token"], positions=case["positions"], scale=scale, window=window)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("batch,context", [(1, 1), (1, 17), (2, 33), (4, 65)])
+def test_paged_decode_workloads_of_the_reference(ops, dtype, batch, context):
+    # Hq16 / Hkv8 / bs16 / D128, reversed tables, seed 8800 + 100 B + C; 2e-4 float32, 8e-3 half
+    # (miniserve/toolchain/benchmark_paged_decode.py:26-60, 112-116, 141)
+    case = paged_case([context] * batch, 16, 8, 128, 16, dtype, seed=8800 + 100 * batch + context)
+    out = run_attention(ops, case, 128**-0.5)
+    expected = attention_reference(case, 128**-0.5)
+    tol = tolerance(dtype, 2e-4, 8e-3)
+    torch.testing.assert_close(out.cpu().double(), expected, atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,block", [(4, 2, 16, 16), (8, 1, 32, 8), (6, 3, 48, 5), (5, 5, 80, 7), (2, 1, 256, 32), (12, 4, 64, 16), (3, 1, 112, 1)])
+def test_attention_sizes_chunks_and_decode_rows_in_one_batch(ops, dtype, heads, kv_heads, dim, block):
+    contexts = [1, 63, 64, 65, 130, 257]
+    query_lens = [1, 1, 64, 7, 130, 2]           # decode rows, whole prompts and portions side by side
+    case = paged_case(contexts, heads, kv_heads, dim, block, dtype, query_lens=query_lens, seed=dim + block)
+    out = run_attention(ops, case, dim**-0.5)
+    expected = attention_reference(case, dim**-0.5)
+    tol = tolerance(dtype, 2e-4, 8e-3)
+    torch.testing.assert_close(out.cpu().double(), expected, atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_one_far_key_among_hundreds_stands_out(ops, dtype):
+    """Random keys give near-uniform weights, which would hide a lost page.  Here one
+    key, far back, carries almost all the weight, and its value is unlike all others."""
+
+    for far in (0, 15, 16, 17, 300, 511, 512, 700):
+        case = paged_case([701], 4, 2, 64, 16, dtype, seed=far)
+        k, v = case["keys"][0], case["values"][0]
+        q = case["queries"][0]
+        page, offset = int(case["block_table"][0, far // 16]), far % 16
+        k[far] = 0.0
+        q[0] = 0.0
+        q[0, :, 0] = 8.0
+        k[far, :, 0] = 8.0                                                      # score 64 * scale = 8 above the rest
+        v[far] = 100.0
+        case["q"] = q.to(dtype).to(DEVICE)
+        case["key_pool"][page, :, offset] = k[far].to(dtype).to(DEVICE)
+        case["value_pool"][page, :, offset] = v[far].to(dtype).to(DEVICE)
+        out = run_attention(ops, case, 64**-0.5)
+        expected = attention_reference(case, 64**-0.5)
+        assert float(expected.min()) > 10.0                                     # the far key dominates
+        tol = tolerance(dtype, 2e-4, 8e-3)
+        torch.testing.assert_close(out.cpu().double(), expected, atol=tol * 100, rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 5, 16, 64, 100])
+def test_window_edges(ops, dtype, window):
+    """The key just inside the window carries a large value, the key just outside a
+    huge one: an edge off by one changes the result beyond any tolerance."""
+
+    contexts, query_lens = [131, 70, 9], [3, 70, 1]
+    case = paged_case(contexts, 4, 2, 32, 8, dtype, query_lens=query_lens, seed=window)
+    for index, (context, v) in enumerate(zip(contexts, case["values"])):
+        last = context - 1
+        inside, outside = last - window + 1, last - window
+        for position, value in ((inside, 50.0), (outside, -1000.0)):
+            if position >= 0:
+                v[position] = value
+                page = int(case["block_table"][index, position // 8])
+                case["value_pool"][page, :, position % 8] = value
+    out = run_attention(ops, case, 32**-0.5, window=window)
+    expected = attention_reference(case, 32**-0.5, window=window)
+    tol = tolerance(dtype, 2e-4, 8e-3)
+    torch.testing.assert_close(out.cpu().double(), expected, atol=tol * 50, rtol=tol)
+
+
+def test_attention_is_bit_identical_across_batches_in_float32(ops):
+    case = paged_case([200, 77], 4, 2, 48, 16, torch.float32, query_lens=[200, 1], seed=5)
+    together = run_attention(ops, case, 0.2)
+    alone = dict(case)                       # the same cache, only the last query of each sequence
+    alone["q"] = torch.stack([case["q"][199], case["q"][200]])
+    alone["seq_of_token"] = torch.tensor([0, 1], dtype=torch.int32, device=DEVICE)
+    alone["positions"] = torch.tensor([199, 76], dtype=torch.int32, device=DEVICE)
+    separate = run_attention(ops, alone, 0.2)
+    assert torch.equal(separate[0], together[199]) and torch.equal(separate[1], together[200])
+
+
+# ---- products and activation ---------------------------------------------------------------
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (1, 509, 96), (63, 65, 17), (64, 64, 16), (65, 63, 33), (130, 200, 257), (7, 1031, 64)])
+def test_gemm_f32_is_true_32_bit(ops, m, n, k):
+    x, w = rand(m, k, seed=m), rand(n, k, seed=n + 1)
+    out = ops.linear(x, w)
+    expected = x.cpu().double() @ w.cpu().double().T
+    torch.testing.assert_close(out.cpu().double(), expected, atol=1e-5 * math.sqrt(k), rtol=1e-6)
+    # sequential accumulation over k in float32, exactly
+    if k <= 33:
+        acc = torch.zeros(m, n)
+        xc, wc = x.cpu(), w.cpu()
+        for index in range(k):
+            acc = torch.addcmul(acc, xc[:, index : index + 1], wc[:, index].unsqueeze(0))
+        assert float((out.cpu() - acc).abs().max()) <= 1e-6
+    # a row's result does not depend on the rows around it
+    row = ops.linear(x[m // 2 : m // 2 + 1].contiguous(), w)
+    assert torch.equal(row[0], out[m // 2])
+    target = rand(m, n, seed=5)
+    before = target.clone()
+    ops.linear(x, w, accumulate_into=target)
+    assert torch.equal(target, before + out)
+
+
+def test_linear_bfloat16_and_fused_projection_rows(ops):
+    """One product over stacked q|k|v (or gate|up) rows equals the separate products."""
+
+    x = rand(37, 96, seed=1, dtype=torch.bfloat16)
+    parts = [rand(n, 96, seed=10 + n, dtype=torch.bfloat16, scale=0.05) for n in (256, 32, 32)]
+    fused = ops.linear(x, torch.cat(parts).contiguous())
+    offset = 0
+    for part in parts:
+        expected = (x.cpu().double() @ part.cpu().double().T)
+        torch.testing.assert_close(fused[:, offset : offset + part.shape[0]].cpu().double(), expected, atol=2e-2, rtol=2e-2)
+        offset += part.shape[0]
+    x32 = x.float()
+    fused32 = ops.linear(x32, torch.cat(parts).float().contiguous())
+    assert torch.equal(fused32[:, 256:288], ops.linear(x32, parts[1].float()))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,inter", [(1, 1), (3, 63), (5, 200), (64, 3072), (2, 1031)])
+def test_silu_mul(ops, dtype, rows, inter):
+    gate_up = rand(rows, 2 * inter, seed=inter, dtype=dtype, scale=3.0)
+    out = ops.silu_mul(gate_up)
+    g, u = gate_up.cpu().double()[:, :inter], gate_up.cpu().double()[:, inter:]
+    expected = torch.nn.functional.silu(g) * u
+    tol = tolerance(dtype, 1e-6, 8e-3)
+    torch.testing.assert_close(out.cpu().double(), expected, atol=tol, rtol=tol)
+    zero_gate = gate_up.clone()
+    zero_gate[:, :inter] = 0
+    assert torch.all(ops.silu_mul(zero_gate) == 0)
+
+
+def test_residual_add(ops):
+    h, delta = rand(5, 77, seed=1), rand(5, 77, seed=2, dtype=torch.bfloat16)
+    expected = h + delta.float()
+    ops.residual_add(h, delta)
+    assert torch.equal(h, expected)
+
+
+# ---- sampling -------------------------------------------------------------------------------
+
+def test_greedy_is_argmax_with_the_lowest_index_among_equals(ops):
+    logits = rand(9, 1031, seed=3)
+    logits[2, 700] = logits[2, 30] = 50.0
+    logits[5] = 1.25
+    out = ops.sample_rows(logits)
+    expected = torch.argmax(logits, dim=-1).cpu()
+    expected[2], expected[5] = 30, 0
+    assert out.cpu().tolist() == expected.tolist()
+    assert ops.sample_rows(torch.tensor([[0.1, 4.0, 3.0]], device=DEVICE)).tolist() == [1]     # test_sampling.py:38-41
+
+
+def test_non_finite_logits_are_reported(ops):
+    # reference: tests/unit/test_sampling.py:90-102
+    logits = rand(4, 300, seed=1)
+    logits[1, 5], logits[2, 7], logits[3, 9] = float("nan"), float("inf"), float("-inf")
+    assert ops.sample_rows(logits).tolist()[1:] == [-1, -1, -1]
+
+
+@pytest.mark.parametrize("vocab", [2, 64, 509, 1031, 151936])
+def test_sampling_matches_the_plain_implementation(ops, vocab):
+    generator = torch.Generator().manual_seed(vocab)
+    rows = 24
+    logits = (torch.randn(rows, vocab, generator=generator) * 3).to(DEVICE)
+    temperature = torch.tensor([0.0, 0.3, 0.8, 1.0, 1.5, 2.0] * 4)
+    top_k = torch.tensor(([0] * 6 + [1] * 6 + [min(5, vocab)] * 6 + [min(50, vocab)] * 6), dtype=torch.int32)
+    top_p = torch.tensor([1.0, 0.9, 0.5, 1.0, 0.1, 0.99] * 4)[torch.randperm(rows, generator=generator)]
+    uniform = torch.rand(rows, generator=generator)
+    out = ops.sample_rows(logits, temperature=temperature.to(DEVICE), top_k=top_k.to(DEVICE),
+                          top_p=top_p.to(DEVICE), uniform=uniform.to(DEVICE)).cpu().tolist()
+    for row in range(rows):
+        expected = plain_sampling.sample_row(
+            logits[row].cpu(), float(temperature[row]), int(top_k[row]), float(top_p[row]), float(uniform[row])
+        )
+        assert out[row] == expected, f"row {row}: T={temperature[row]} k={top_k[row]} p={top_p[row]} u={uniform[row]}"
+
+
+def test_sampling_vectors_of_the_reference(ops):
+    # [5,4,3,2], T=1, k=2, p=0.6 -> always 0 (tests/unit/test_sampling.py:44-49)
+    logits = torch.tensor([[5.0, 4.0, 3.0, 2.0]] * 20, device=DEVICE)
+    out = ops.sample_rows(
+        logits, temperature=torch.ones(20, device=DEVICE), top_k=torch.full((20,), 2, dtype=torch.int32, device=DEVICE),
+        top_p=torch.full((20,), 0.6, device=DEVICE), uniform=(torch.arange(20, device=DEVICE) / 20.0),
+    )
+    assert out.tolist() == [0] * 20
+    # ties keep exactly k (tests/unit/test_sampling.py:123-125): [5,5,5,1] with k=2 never gives index 2 or 3
+    tied = torch.tensor([[5.0, 5.0, 5.0, 1.0]] * 50, device=DEVICE)
+    out = ops.sample_rows(
+        tied, temperature=torch.ones(50, device=DEVICE), top_k=torch.full((50,), 2, dtype=torch.int32, device=DEVICE),
+        top_p=torch.ones(50, device=DEVICE), uniform=(torch.arange(50, device=DEVICE) + 0.5) / 50.0,
+    )
+    assert set(out.tolist()) == {0, 1}
+
+
+def test_the_draw_follows_the_distribution(ops):
+    probabilities = torch.tensor([0.5, 0.3, 0.15, 0.05])
+    n = 4000
+    logits = torch.log(probabilities).repeat(n, 1).to(DEVICE)
+    out = ops.sample_rows(logits, temperature=torch.ones(n, device=DEVICE), uniform=((torch.arange(n) + 0.5) / n).to(DEVICE))
+    counts = torch.bincount(out.cpu().long(), minlength=4).float() / n
+    torch.testing.assert_close(counts, probabilities, atol=1e-3, rtol=0)
+
+
+def test_sampler_stages_without_advancing_the_stream(ops):
+    # reference: tests/unit/test_sampling.py:71-87
+    from miniserve_amd.engine import SamplingParams
+    from miniserve_amd.sampling import NonFiniteLogitsError, Sampler
+
+    sampler = Sampler()
+    logits = torch.tensor([[0.1, 1.0, 2.0, 3.0]], device=DEVICE)
+    params = SamplingParams(temperature=1.0, seed=17)
+    first = sampler.stage(logits, [("staged", params)])
+    second = sampler.stage(logits, [("staged", params)])
+    assert first[0].token_id == second[0].token_id and sampler.active_request_ids == ()
+    stream = torch.Generator().manual_seed(17)
+    draws = [Sampler.draw_uniform(stream) for _ in range(2)]
+    expected = [plain_sampling.sample_row(logits[0].cpu(), 1.0, 0, 1.0, u) for u in draws]
+    assert first[0].token_id == expected[0]
+    sampler.commit(first)
+    assert sampler.active_request_ids == ("staged",)
+    assert sampler.stage(logits, [("staged", params)])[0].token_id == expected[1]
+    sampler.release("staged")
+    sampler.release("staged")
+    assert sampler.active_request_ids == ()
+    greedy = sampler.sample(logits, [("g", SamplingParams())])
+    assert greedy == [3] and sampler.active_request_ids == ()                  # greedy makes no stream
+    with pytest.raises(NonFiniteLogitsError, match="finite"):
+        sampler.sample(torch.tensor([[0.0, float("nan")]], device=DEVICE), [("n", SamplingParams())])
+    with pytest.raises(ValueError, match="vocabulary"):
+        sampler.sample(logits, [("k", SamplingParams(temperature=1.0, top_k=5))])
+    with pytest.raises(TypeError, match="floating-point"):
+        sampler.sample(torch.tensor([[1, 2, 3]], device=DEVICE), [("i", SamplingParams())])

@@ -1,0 +1,251 @@
+"""Each part of a layer alone against the plain implementation, and a toy mixer with
+state of its own that is registered, built and stepped without a change to the
+framework's files."""
+
+from __future__ import annotations
+
+import plain_qwen3 as plain
+import pytest
+import torch
+from helpers import make_model_folder, random_tokens, read_config, read_weights, tiny_a, tiny_b
+
+pytestmark = pytest.mark.gpu
+
+DEVICE = "cuda:0"
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 1e-5, "bfloat16": 2e-2}
+
+
+def to_device(weights, dtype):
+    return {name: tensor.to(dtype).to(DEVICE).contiguous() for name, tensor in weights.items()}
+
+
+def oracle_weights(weights, dtype):
+    return {name: tensor.to(dtype).double() for name, tensor in weights.items()}
+
+
+def rand(*shape, seed=0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed))
+
+
+def step_context(query_lens, starts, block_size, *, tables=None):
+    """A StepContext over one cache group, pages handed out in order (or ``tables``)."""
+
+    from miniserve_amd.parts import GroupStepView, StepContext
+
+    token_pos, seq_of, slots, table_rows = [], [], [], []
+    next_page = 0
+    for index, (qlen, start) in enumerate(zip(query_lens, starts)):
+        pages_needed = -(-(start + qlen) // block_size)
+        if tables is None:
+            row = list(range(next_page, next_page + pages_needed))
+            next_page += pages_needed
+        else:
+            row = tables[index]
+        table_rows.append(row)
+        for position in range(start, start + qlen):
+            token_pos.append(position)
+            seq_of.append(index)
+            slots.append(row[position // block_size] * block_size + position % block_size)
+    width = max(len(r) for r in table_rows)
+    table = torch.tensor([r + [0] * (width - len(r)) for r in table_rows], dtype=torch.int32, device=DEVICE)
+    i32 = lambda values: torch.tensor(values, dtype=torch.int32, device=DEVICE)
+    starts_q = [0]
+    for qlen in query_lens:
+        starts_q.append(starts_q[-1] + qlen)
+    return StepContext(
+        num_tokens=len(token_pos), num_seqs=len(query_lens), token_ids=i32([0] * len(token_pos)), positions=i32(token_pos),
+        seq_of_token=i32(seq_of), query_start=i32(starts_q), context_lens=i32([s + q for s, q in zip(starts, query_lens)]),
+        state_slots=i32(list(range(len(query_lens)))), groups=[GroupStepView(table, i32(slots))],
+        query_lens=list(query_lens), context_lens_host=[s + q for s, q in zip(starts, query_lens)],
+        query_start_host=starts_q, state_slots_host=list(range(len(query_lens))), first_positions_host=list(starts),
+    ), table_rows
+
+
+@pytest.fixture(scope="module", params=["a", "b"])
+def model(request, tmp_path_factory):
+    make, block = {"a": (tiny_a, 16), "b": (tiny_b, 8)}[request.param]
+    folder = make_model_folder(tmp_path_factory.mktemp("parts") / request.param, make(), seed=31)
+    from miniserve_amd.config import load_config
+
+    return {"config": read_config(folder), "weights": read_weights(folder), "spec": load_config(folder).model_spec(), "block": block}
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+def test_norm_part(model, dtype):
+    from miniserve_amd.parts import build_part
+
+    spec = model["spec"].layers[0].norms["pre_mixer"]
+    part = build_part("norm", spec, DTYPES[dtype])
+    part.load_weights(to_device(model["weights"], DTYPES[dtype]))
+    assert [w.name for w in part.weight_specs()] == ["model.layers.0.input_layernorm.weight"]
+    x = rand(9, spec.params["dim"], seed=1).to(DTYPES[dtype])
+    expected = plain.rms_norm(x.double(), oracle_weights(model["weights"], DTYPES[dtype])[spec.prefix + "weight"], spec.params["eps"])
+    torch.testing.assert_close(part.forward(x.to(DEVICE)).cpu().double(), expected, atol=TOL[dtype], rtol=TOL[dtype])
+    residual, delta = rand(9, spec.params["dim"], seed=2).to(DEVICE), x.to(DEVICE)
+    total = residual + delta.float()
+    out = part.add_forward(residual, delta)
+    assert torch.equal(residual, total)
+    expected = plain.rms_norm(total.cpu().double(), oracle_weights(model["weights"], DTYPES[dtype])[spec.prefix + "weight"], spec.params["eps"])
+    torch.testing.assert_close(out.cpu().double(), expected, atol=TOL[dtype], rtol=TOL[dtype])
+
+
+def test_position_part(model):
+    from miniserve_amd.parts import build_part
+
+    spec = model["spec"].layers[0].mixer.params["position"]
+    part = build_part("position", spec, torch.float32)
+    assert part.weight_specs() == []
+    dim, theta = spec.params["dim"], spec.params["theta"]
+    x = rand(6, 3, dim, seed=4)
+    positions = torch.tensor([0, 1, 7, 64, 300, 511], dtype=torch.int32, device=DEVICE)
+    cos, sin = plain.rope_angles(positions.cpu().long(), dim, theta)
+    expected = plain.apply_rope(x.double().transpose(0, 1), cos, sin).transpose(0, 1)
+    out = part.apply(x.to(DEVICE), positions)
+    torch.testing.assert_close(out.cpu().double(), expected, atol=1e-5, rtol=1e-5)
+    # only distances count: <rope(q, m), rope(k, n)> is the same for equal m - n
+    q, k = x[:1, :1].to(DEVICE), x[1:2, :1].to(DEVICE)
+    at = lambda t, p: part.apply(t, torch.tensor([p], dtype=torch.int32, device=DEVICE))
+    dots = [float((at(q, m) * at(k, n)).sum()) for m, n in ((9, 4), (205, 200))]
+    assert abs(dots[0] - dots[1]) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+def test_feed_forward_part(model, dtype):
+    from miniserve_amd.parts import build_part
+
+    spec = model["spec"].layers[1].feed_forward
+    part = build_part("feed_forward", spec, DTYPES[dtype])
+    part.load_weights(to_device(model["weights"], DTYPES[dtype]))
+    assert part.w_gate_up.shape == (2 * spec.params["intermediate_size"], spec.params["hidden_size"])
+    x = rand(13, spec.params["hidden_size"], seed=5).to(DTYPES[dtype])
+    expected = plain.swiglu(x.double(), oracle_weights(model["weights"], DTYPES[dtype]), spec.prefix)
+    torch.testing.assert_close(part.forward(x.to(DEVICE)).cpu().double(), expected, atol=TOL[dtype] * 0.1, rtol=TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+def test_attention_part_whole_and_in_portions(model, dtype):
+    """The mixer alone over its own cache: one request whole, the same request in
+    portions beside another request's decoded token, on scattered pages."""
+
+    from miniserve_amd.parts import KVCacheNeed, KVCacheView, build_part
+
+    config, block = model["config"], model["block"]
+    spec = model["spec"].layers[0].mixer
+    part = build_part("mixer", spec, DTYPES[dtype])
+    from miniserve_amd.parts.base import load_part_weights
+
+    load_part_weights(part, to_device(model["weights"], DTYPES[dtype]))
+    assert part.cache_need() == KVCacheNeed(config["num_key_value_heads"], config["head_dim"], None)
+    assert part.w_qkv.shape[0] == (config["num_attention_heads"] + 2 * config["num_key_value_heads"]) * config["head_dim"]
+    hidden, length = config["hidden_size"], 45
+    x = rand(length, hidden, seed=6).to(DTYPES[dtype])
+    other = rand(20, hidden, seed=7).to(DTYPES[dtype])
+    weights = oracle_weights(model["weights"], DTYPES[dtype])
+    expected, _ = plain.attention_block(x.double(), weights, spec.prefix, config, torch.arange(length))
+    expected_other, _ = plain.attention_block(other.double(), weights, spec.prefix, config, torch.arange(20))
+
+    def fresh_cache(pages):
+        shape = (pages, config["num_key_value_heads"], block, config["head_dim"])
+        return KVCacheView(0, torch.full(shape, float("nan"), dtype=DTYPES[dtype], device=DEVICE),
+                           torch.full(shape, float("nan"), dtype=DTYPES[dtype], device=DEVICE), block)
+
+    cache = fresh_cache(8)
+    ctx, _ = step_context([length], [0], block)
+    out = part.forward(x.to(DEVICE), ctx, cache)
+    torch.testing.assert_close(out.cpu().double(), expected, atol=TOL[dtype] * 0.1, rtol=TOL[dtype])
+
+    cache = fresh_cache(16)
+    tables = [[15, 3, 9, 0, 7, 12], [5, 1, 14]]
+    outs, position = [], 0
+    ctx, _ = step_context([19], [0], block, tables=[tables[1]])
+    part.forward(other[:19].to(DEVICE), ctx, cache)                                    # the other request's history
+    for size in (7, 2, 13, 23):
+        if position == 9:      # this portion runs beside the other request's decoded token
+            ctx, _ = step_context([size, 1], [position, 19], block, tables=tables)
+            batch = torch.cat([x[position : position + size], other[19:20]]).to(DEVICE)
+            result = part.forward(batch, ctx, cache)
+            outs.append(result[:size])
+            torch.testing.assert_close(result[size:].cpu().double(), expected_other[19:20], atol=TOL[dtype] * 0.1, rtol=TOL[dtype])
+        else:
+            ctx, _ = step_context([size], [position], block, tables=[tables[0]])
+            outs.append(part.forward(x[position : position + size].to(DEVICE), ctx, cache))
+        position += size
+    torch.testing.assert_close(torch.cat(outs).cpu().double(), expected, atol=TOL[dtype] * 0.1, rtol=TOL[dtype])
+
+
+def test_attention_part_composed_from_its_parts_equals_the_fused_kernel(model):
+    """With a position part that the fused kernel does not know, the mixer runs the
+    norms and the position encoding through their own parts; same result."""
+
+    from miniserve_amd.config import PartSpec
+    from miniserve_amd.parts import KVCacheView, Part, build_part, register_part, unregister_part
+    from miniserve_amd.parts.base import load_part_weights
+    from miniserve_amd.parts.rotary import RotaryHalf
+
+    class WrappedRotary(Part):
+        """The same function behind a class that the attention part does not recognise."""
+
+        def __init__(self, spec, dtype):
+            self.inner = RotaryHalf(spec, dtype)
+
+        def apply(self, x, positions):
+            return self.inner.apply(x, positions)
+
+    register_part("position", "test_wrapped_rotary", WrappedRotary)
+    try:
+        spec = model["spec"].layers[0].mixer
+        params = dict(spec.params)
+        params["position"] = PartSpec("test_wrapped_rotary", spec.params["position"].params)
+        fused = build_part("mixer", spec, torch.float32)
+        composed = build_part("mixer", PartSpec("attention", params, spec.prefix), torch.float32)
+        assert fused._fused and not composed._fused
+        config, block = model["config"], model["block"]
+        weights = to_device(model["weights"], torch.float32)
+        x = rand(21, config["hidden_size"], seed=8).to(DEVICE)
+        results = []
+        for part in (fused, composed):
+            load_part_weights(part, weights)
+            shape = (4, config["num_key_value_heads"], block, config["head_dim"])
+            cache = KVCacheView(0, torch.zeros(shape, device=DEVICE), torch.zeros(shape, device=DEVICE), block)
+            ctx, _ = step_context([21], [0], block)
+            results.append((part.forward(x, ctx, cache), cache.key.clone(), cache.value.clone()))
+        for got, want in zip(results[1], results[0]):
+            torch.testing.assert_close(got, want, atol=1e-6, rtol=1e-6)
+    finally:
+        unregister_part("position", "test_wrapped_rotary")
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+def test_block_embedding_and_head(model, dtype):
+    from miniserve_amd.parts import KVCacheView, build_block, build_part
+    from miniserve_amd.parts.base import load_part_weights
+
+    config, block_size, spec = model["config"], model["block"], model["spec"]
+    device_weights = to_device(model["weights"], DTYPES[dtype])
+    weights = oracle_weights(model["weights"], DTYPES[dtype])
+    tokens = random_tokens(30, config["vocab_size"], 3)
+    embedding = build_part("embedding", spec.embedding, DTYPES[dtype])
+    embedding.load_weights(device_weights)
+    h = embedding.forward(torch.tensor(tokens, dtype=torch.int32, device=DEVICE))
+    assert h.dtype == torch.float32
+    assert torch.equal(h.cpu().double(), weights["model.embed_tokens.weight"][tokens])
+
+    layer = build_block(spec.layers[1], DTYPES[dtype])
+    load_part_weights(layer, device_weights)
+    shape = (4, config["num_key_value_heads"], block_size, config["head_dim"])
+    cache = KVCacheView(0, torch.zeros(shape, dtype=DTYPES[dtype], device=DEVICE), torch.zeros(shape, dtype=DTYPES[dtype], device=DEVICE), block_size)
+    ctx, _ = step_context([30], [0], block_size)
+    residual, delta = layer.forward(h.clone(), None, ctx, cache)
+    expected, _ = plain.decoder_layer(h.cpu().double(), weights, 1, config, torch.arange(30))
+    torch.testing.assert_close((residual + delta.float()).cpu().double(), expected, atol=TOL[dtype], rtol=TOL[dtype])
+
+    head = build_part("head", spec.head, DTYPES[dtype])
+    head.load_weights(device_weights)
+    y = rand(5, config["hidden_size"], seed=9).to(DTYPES[dtype])
+    matrix = weights["model.embed_tokens.weight"] if config["tie_word_embeddings"] else weights["lm_head.weight"]
+    logits = head.forward(y.to(DEVICE))
+    assert logits.dtype == torch.float32 and logits.shape == (5, config["vocab_size"])
+    torch.testing.assert_close(logits.cpu().double(), y.double() @ matrix.T, atol=TOL[dtype], rtol=TOL[dtype])
+    if config["tie_word_embeddings"]:
+        assert head.weight.data_ptr() == embedding.weight.data_ptr()                   # the very same tensor
