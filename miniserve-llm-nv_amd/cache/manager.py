@@ -115,8 +115,10 @@ class CacheManager:
 
     # ---- storage --------------------------------------------------------------------
     def allocate_storage(self, dtype, device) -> None:
-        """Pools ``[calls, pages, kv_heads, block_size, head_dim]`` per group, allocated
-        once and never initialised (a page's content is read only below the
+        """Per group a key pool ``[calls, pages, kv_heads, block_size, head_dim]`` and a
+        value pool ``[calls, pages, kv_heads, head_dim, block_size]`` (values lie
+        transposed inside a page: the matrix-core kernels read 4 consecutive keys
+        of one column in one load), allocated once and never initialised (a page's content is read only below the
         committed length; reference: miniserve/kv/paged.py:39-41), and zeroed
         state tensors ``[slots, *shape]``."""
 
@@ -124,9 +126,13 @@ class CacheManager:
 
         self.key_pools, self.value_pools, self.state_tensors = [], [], []
         for group, count in zip(self.layout.groups, self.num_blocks):
-            shape = (len(group.calls), count, group.need.num_kv_heads, self.block_size, group.need.head_dim)
-            self.key_pools.append(torch.empty(shape, dtype=dtype, device=device))
-            self.value_pools.append(torch.empty(shape, dtype=dtype, device=device))
+            heads, dim = group.need.num_kv_heads, group.need.head_dim
+            self.key_pools.append(
+                torch.empty((len(group.calls), count, heads, self.block_size, dim), dtype=dtype, device=device)
+            )
+            self.value_pools.append(
+                torch.empty((len(group.calls), count, heads, dim, self.block_size), dtype=dtype, device=device)
+            )
         for need in self.layout.states:
             self.state_tensors.append(torch.zeros((self.max_num_seqs, *need.shape), dtype=need.dtype, device=device))
 

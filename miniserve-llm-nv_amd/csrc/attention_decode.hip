@@ -1,0 +1,319 @@
+// Paged attention for rows that each bring ONE query token (decoding), bfloat16
+// storage, matrix cores, split over the keys.
+//
+// Work is cut as (split of the keys, kv head x group of 16 query heads, token).
+// All query heads that share a kv head are the 16 columns of one MFMA tile, so
+// every key and value is read once for all of them.  A workgroup of 4 waves walks
+// its share of the keys in tiles of 16 keys, two tiles (32 keys) per MFMA; each
+// wave keeps an online softmax (running max m, sum l) in 32-bit and an
+// unnormalised output tile in 32-bit; the waves are merged through LDS; a split
+// writes its (m, l, O) and a second kernel merges the splits.
+//
+//   S^T[key, head] = K[key, :] . Q[head, :]      A = K tile (16 keys x 32 d), B = Q^T
+//   P = exp(S * scale - m)                        (scale after the product, as the
+//                                                  reference does: qwen3.py:243)
+//   O[head, d]   += P[head, keys] . V[keys, d]    A = P (the S^T accumulator, as it
+//                                                  lies in the registers), B = V
+// The cache layout serves the operands directly: keys as [page, kv_head, offset, d]
+// (8 consecutive d per lane, 16 bytes), values as [page, kv_head, d, offset]
+// (4 consecutive keys per lane, 8 bytes).
+//
+// Formula of the one-token form: reference csrc/paged_decode_attention.cu:44-94.
+// Unlike there, no shared memory grows with the context.
+#include "mfma.hpp"
+
+namespace {
+
+using ms::bf16;
+using ms::bf16x4;
+using ms::bf16x8;
+using ms::floatx4;
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * ms::kWave;
+constexpr int kTileKeys = 16;
+
+template <int D>
+__global__ __launch_bounds__(kThreads) void attention_decode_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ key_pool, const bf16* __restrict__ value_pool,
+    const int32_t* __restrict__ block_table, const int32_t* __restrict__ seq_of_token,
+    const int32_t* __restrict__ positions, bf16* __restrict__ out, float* __restrict__ partial_o,
+    float* __restrict__ partial_ml, int num_q_heads, int num_kv_heads, int block_size, int max_blocks, float scale,
+    int window, int num_splits) {
+  constexpr int KS = (D + 31) / 32;   // 32-wide slices of d for Q.K
+  constexpr int CS = D / 16;          // 16-wide slices of d for P.V
+
+  __shared__ float o_s[kWaves - 1][16][D];
+  __shared__ float m_s[kWaves][16];
+  __shared__ float l_s[kWaves][16];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int g = lane >> 4;
+  const int r = lane & 15;
+
+  const int split = blockIdx.x;
+  const int group = num_q_heads / num_kv_heads;
+  const int head_groups = (group + 15) / 16;
+  const int kv_head = blockIdx.y / head_groups;
+  const int head_group = blockIdx.y - kv_head * head_groups;
+  const int64_t token = blockIdx.z;
+  const int head0 = kv_head * group + head_group * 16;
+  const int heads_here = min(16, group - head_group * 16);
+
+  const int pos = positions[token];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int32_t* table = block_table + static_cast<int64_t>(seq_of_token[token]) * max_blocks;
+
+  const int first_tile = lo / kTileKeys;
+  const int last_tile = pos / kTileKeys;
+  const int tiles_per_split = (last_tile - first_tile + num_splits) / num_splits;
+  const int t0 = first_tile + split * tiles_per_split;
+  const int t1 = min(t0 + tiles_per_split, last_tile + 1);
+
+  // Q^T operand: column r = head, k-slots d = 32 s + 8 g + 0..7
+  bf16x8 q_reg[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    const int d0 = 32 * s + 8 * g;
+    q_reg[s] = (r < heads_here && d0 < D) ? ms::load_bf16x8(q + (token * num_q_heads + head0 + r) * D + d0)
+                                          : ms::zero_bf16x8();
+  }
+
+  floatx4 o[CS];
+#pragma unroll
+  for (int c = 0; c < CS; ++c) o[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float run_max = -INFINITY;   // of head r
+  float run_sum = 0.f;
+
+  for (int t = t0 + 2 * wave; t < t1; t += 2 * kWaves) {
+    const bool has_b = t + 1 < t1;
+    const int key_a = t * kTileKeys;
+    const int key_b = key_a + kTileKeys;
+    const int64_t page_a = table[key_a / block_size];
+    const int off_a = key_a % block_size;
+    const int64_t page_b = has_b ? table[key_b / block_size] : page_a;
+    const int off_b = has_b ? key_b % block_size : off_a;
+
+    // ---- S^T = K . Q^T ------------------------------------------------------
+    const bf16* k_row_a = key_pool + ((page_a * num_kv_heads + kv_head) * block_size + off_a + r) * D;
+    const bf16* k_row_b = key_pool + ((page_b * num_kv_heads + kv_head) * block_size + off_b + r) * D;
+    floatx4 s_a = {0.f, 0.f, 0.f, 0.f}, s_b = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int d0 = 32 * s + 8 * g;
+      const bf16x8 ka = d0 < D ? ms::load_bf16x8(k_row_a + d0) : ms::zero_bf16x8();
+      s_a = ms::mfma_16x16x32(ka, q_reg[s], s_a);
+      if (has_b) {
+        const bf16x8 kb = d0 < D ? ms::load_bf16x8(k_row_b + d0) : ms::zero_bf16x8();
+        s_b = ms::mfma_16x16x32(kb, q_reg[s], s_b);
+      }
+    }
+    // this lane: head r, keys key_a + 4 g + e and key_b + 4 g + e
+    bool ok_a[4], ok_b[4];
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int ka = key_a + 4 * g + e, kb = key_b + 4 * g + e;
+      ok_a[e] = ka >= lo && ka <= pos;
+      ok_b[e] = has_b && kb >= lo && kb <= pos;
+      s_a[e] = ok_a[e] ? s_a[e] * scale : -INFINITY;
+      s_b[e] = ok_b[e] ? s_b[e] * scale : -INFINITY;
+      tile_max = fmaxf(tile_max, fmaxf(s_a[e], s_b[e]));
+    }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, ms::kWave));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, ms::kWave));
+    const float new_max = fmaxf(run_max, tile_max);   // finite: every tile of the range holds a visible key
+    const float alpha = __expf(run_max - new_max);
+    float tile_sum = 0.f;
+    bf16x8 p;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float pa = __expf(s_a[e] - new_max);
+      const float pb = __expf(s_b[e] - new_max);
+      tile_sum += pa + pb;
+      p[e] = static_cast<__bf16>(pa);
+      p[e + 4] = static_cast<__bf16>(pb);
+    }
+    tile_sum += __shfl_xor(tile_sum, 16, ms::kWave);
+    tile_sum += __shfl_xor(tile_sum, 32, ms::kWave);
+    run_sum = run_sum * alpha + tile_sum;
+    run_max = new_max;
+
+    // ---- O = alpha O + P . V ------------------------------------------------
+    // O's rows in this lane are the heads 4 g + e; their alpha lives in lane 4 g + e.
+    float alpha_row[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) alpha_row[e] = __shfl(alpha, 4 * g + e, ms::kWave);
+    const bool partial = !(ok_a[0] && ok_a[3] && ok_b[0] && ok_b[3]);
+    const bf16* v_a = value_pool + (page_a * num_kv_heads + kv_head) * D * block_size + off_a + 4 * g;
+    const bf16* v_b = value_pool + (page_b * num_kv_heads + kv_head) * D * block_size + off_b + 4 * g;
+#pragma unroll
+    for (int c = 0; c < CS; ++c) {
+      const int d = 16 * c + r;
+      bf16x4 va = ms::load_bf16x4(v_a + static_cast<int64_t>(d) * block_size);
+      bf16x4 vb = has_b ? ms::load_bf16x4(v_b + static_cast<int64_t>(d) * block_size) : ms::zero_bf16x4();
+      if (partial) {   // a stale value times a zero weight must not become NaN
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (!ok_a[e]) va[e] = static_cast<__bf16>(0.0f);
+          if (!ok_b[e]) vb[e] = static_cast<__bf16>(0.0f);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[c][e] *= alpha_row[e];
+      o[c] = ms::mfma_16x16x32(p, ms::concat(va, vb), o[c]);
+    }
+  }
+
+  // ---- merge the waves ------------------------------------------------------
+  if (g == 0) {
+    m_s[wave][r] = run_max;
+    l_s[wave][r] = run_sum;
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int c = 0; c < CS; ++c)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o_s[wave - 1][4 * g + e][16 * c + r] = o[c][e];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+
+  float total_max[4], total_sum[4], factor[kWaves][4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int row = 4 * g + e;
+    float mx = m_s[0][row];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, m_s[w][row]);
+    total_max[e] = mx;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      factor[w][e] = (mx == -INFINITY) ? 0.f : __expf(m_s[w][row] - mx);
+      sum += factor[w][e] * l_s[w][row];
+    }
+    total_sum[e] = sum;
+  }
+#pragma unroll
+  for (int c = 0; c < CS; ++c) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float acc = o[c][e] * factor[0][e];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) acc += o_s[w - 1][4 * g + e][16 * c + r] * factor[w][e];
+      o[c][e] = acc;
+    }
+  }
+
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int row = 4 * g + e;
+    if (row >= heads_here) continue;
+    const int64_t head = head0 + row;
+    if (num_splits == 1) {
+      const float inv = 1.0f / total_sum[e];
+      bf16* dst = out + (token * num_q_heads + head) * D;
+#pragma unroll
+      for (int c = 0; c < CS; ++c) dst[16 * c + r] = ms::from_float<bf16>(o[c][e] * inv);
+    } else {
+      const int64_t slot = (token * num_q_heads + head) * num_splits + split;
+      float* dst = partial_o + slot * D;
+#pragma unroll
+      for (int c = 0; c < CS; ++c) dst[16 * c + r] = o[c][e];
+      if (r == 0) {
+        partial_ml[2 * slot] = total_max[e];
+        partial_ml[2 * slot + 1] = total_sum[e];
+      }
+    }
+  }
+}
+
+// One wave per (token, head): out = sum_s e^{m_s - M} O_s / sum_s e^{m_s - M} l_s.
+__global__ void attention_merge_splits_kernel(const float* __restrict__ partial_o,
+                                              const float* __restrict__ partial_ml, bf16* __restrict__ out,
+                                              int head_dim, int num_splits) {
+  const int64_t row = blockIdx.x;
+  const float* ml = partial_ml + row * num_splits * 2;
+  float mx = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) mx = fmaxf(mx, ml[2 * s]);
+  float sum = 0.f;
+  for (int s = 0; s < num_splits; ++s) sum += __expf(ml[2 * s] - mx) * ml[2 * s + 1];
+  const float inv = 1.0f / sum;
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < num_splits; ++s)
+      acc += __expf(ml[2 * s] - mx) * partial_o[(row * num_splits + s) * head_dim + d];
+    out[row * head_dim + d] = ms::from_float<bf16>(acc * inv);
+  }
+}
+
+template <int D>
+void launch_decode(const void* q, const void* key_pool, const void* value_pool, const void* block_table,
+                   const void* seq_of_token, const void* positions, void* out, void* partial_o, void* partial_ml,
+                   int num_tokens, int num_q_heads, int num_kv_heads, int block_size, int max_blocks, float scale,
+                   int window, int num_splits, hipStream_t stream) {
+  const int head_groups = (num_q_heads / num_kv_heads + 15) / 16;
+  const dim3 grid(num_splits, num_kv_heads * head_groups, num_tokens);
+  hipLaunchKernelGGL((attention_decode_kernel<D>), grid, dim3(kThreads), 0, stream, static_cast<const bf16*>(q),
+                     static_cast<const bf16*>(key_pool), static_cast<const bf16*>(value_pool),
+                     static_cast<const int32_t*>(block_table), static_cast<const int32_t*>(seq_of_token),
+                     static_cast<const int32_t*>(positions), static_cast<bf16*>(out), static_cast<float*>(partial_o),
+                     static_cast<float*>(partial_ml), num_q_heads, num_kv_heads, block_size, max_blocks, scale,
+                     window, num_splits);
+}
+
+}  // namespace
+
+// Whether ms_attention_decode takes this geometry (else the caller uses the
+// generic kernel): head size a multiple of 16 up to 256, pages of a multiple of
+// 16 keys.
+extern "C" int ms_attention_decode_supported(int head_dim, int block_size) {
+  return head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0 && block_size % kTileKeys == 0;
+}
+
+// q, out: bfloat16 [num_tokens, num_q_heads, head_dim]; key_pool: [pages, kv_heads,
+// block_size, head_dim]; value_pool: [pages, kv_heads, head_dim, block_size];
+// partial_o: float [num_tokens, num_q_heads, num_splits, head_dim] and partial_ml:
+// float [num_tokens, num_q_heads, num_splits, 2], both unused when num_splits == 1.
+extern "C" int ms_attention_decode(const void* q, const void* key_pool, const void* value_pool,
+                                   const void* block_table, const void* seq_of_token, const void* positions,
+                                   void* out, void* partial_o, void* partial_ml, int num_tokens, int num_q_heads,
+                                   int num_kv_heads, int head_dim, int block_size, int max_blocks, float scale,
+                                   int window, int num_splits, hipStream_t stream) {
+  MS_REQUIRE(num_tokens > 0 && num_tokens <= 65535, "attention_decode: %d tokens are outside 1..65535", num_tokens);
+  MS_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0,
+             "attention_decode: %d query heads are not a multiple of %d kv heads", num_q_heads, num_kv_heads);
+  MS_REQUIRE(ms_attention_decode_supported(head_dim, block_size),
+             "attention_decode: head_dim %d (multiples of 16 up to 256) or block_size %d (multiples of 16) "
+             "is not supported",
+             head_dim, block_size);
+  MS_REQUIRE(num_splits >= 1 && num_splits <= 1024, "attention_decode: %d splits", num_splits);
+  MS_REQUIRE(num_splits == 1 || (partial_o && partial_ml), "attention_decode: splits need partial buffers");
+  MS_REQUIRE(max_blocks > 0 && window >= 0, "attention_decode: bad table width or window");
+  MS_REQUIRE(num_kv_heads * ((num_q_heads / num_kv_heads + 15) / 16) <= 65535, "attention_decode: too many heads");
+#define MS_DECODE_CASE(DIM)                                                                                     \
+  case DIM:                                                                                                     \
+    launch_decode<DIM>(q, key_pool, value_pool, block_table, seq_of_token, positions, out, partial_o, partial_ml, \
+                       num_tokens, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, num_splits,  \
+                       stream);                                                                                 \
+    break;
+  switch (head_dim) {
+    MS_DECODE_CASE(16) MS_DECODE_CASE(32) MS_DECODE_CASE(48) MS_DECODE_CASE(64) MS_DECODE_CASE(80)
+    MS_DECODE_CASE(96) MS_DECODE_CASE(112) MS_DECODE_CASE(128) MS_DECODE_CASE(144) MS_DECODE_CASE(160)
+    MS_DECODE_CASE(176) MS_DECODE_CASE(192) MS_DECODE_CASE(208) MS_DECODE_CASE(224) MS_DECODE_CASE(240)
+    MS_DECODE_CASE(256)
+    default:
+      return ms_fail("attention_decode: head_dim %d", head_dim);
+  }
+#undef MS_DECODE_CASE
+  MS_CHECK_LAUNCH("attention_decode");
+  if (num_splits > 1) {
+    hipLaunchKernelGGL(attention_merge_splits_kernel, dim3(num_tokens * num_q_heads), dim3(ms::kWave), 0, stream,
+                       static_cast<const float*>(partial_o), static_cast<const float*>(partial_ml),
+                       static_cast<bf16*>(out), head_dim, num_splits);
+    MS_CHECK_LAUNCH("attention_merge_splits");
+  }
+  return 0;
+}

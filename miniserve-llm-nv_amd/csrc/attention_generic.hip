@@ -41,7 +41,7 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, const T* __res
                                          int max_blocks, float scale, int window) {
   __shared__ float q_s[kMaxHeadDim];
   __shared__ float p_s[ms::kWave];
-  __shared__ int64_t row_s[ms::kWave];
+  __shared__ int64_t value_s[ms::kWave];   // where each key's value column starts
 
   const int64_t token = blockIdx.x;
   const int head = blockIdx.y;
@@ -67,12 +67,13 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, const T* __res
     const int j = tile * ms::kWave + lane;
     const bool valid = j >= lo && j <= pos;
     float score = -INFINITY;
-    int64_t row = 0;
+    int64_t value_start = 0;
     if (valid) {
       const int logical = j / block_size;
       const int offset = j - logical * block_size;
       const int64_t page = table[logical];
-      row = ((page * num_kv_heads + kv_head) * block_size + offset) * head_dim;
+      const int64_t row = ((page * num_kv_heads + kv_head) * block_size + offset) * head_dim;
+      value_start = (page * num_kv_heads + kv_head) * head_dim * block_size + offset;
       score = dot_row(q_s, key_pool + row, head_dim) * scale;
     }
     const float new_max = fmaxf(running_max, ms::wave_max(score));
@@ -83,7 +84,7 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, const T* __res
 
     __syncthreads();  // the previous tile's readers are done
     p_s[lane] = p;
-    row_s[lane] = row;
+    value_s[lane] = value_start;
     __syncthreads();
 
     const int first = lo > tile * ms::kWave ? lo - tile * ms::kWave : 0;
@@ -93,7 +94,8 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, const T* __res
       const int d = lane + c * ms::kWave;
       if (d < head_dim) {
         float a = acc[c] * alpha;
-        for (int jj = first; jj <= last; ++jj) a = fmaf(p_s[jj], ms::to_float(value_pool[row_s[jj] + d]), a);
+        for (int jj = first; jj <= last; ++jj)
+          a = fmaf(p_s[jj], ms::to_float(value_pool[value_s[jj] + static_cast<int64_t>(d) * block_size]), a);
         acc[c] = a;
       }
     }
@@ -110,8 +112,9 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, const T* __res
 
 }  // namespace
 
-// q, out: [num_tokens, num_q_heads, head_dim]; pools: [num_blocks, num_kv_heads,
-// block_size, head_dim]; block_table: int32 [num_seqs, max_blocks];
+// q, out: [num_tokens, num_q_heads, head_dim]; key_pool: [num_blocks, num_kv_heads,
+// block_size, head_dim]; value_pool: [num_blocks, num_kv_heads, head_dim,
+// block_size]; block_table: int32 [num_seqs, max_blocks];
 // seq_of_token, positions: int32 [num_tokens]; window: 0 = all keys.
 extern "C" int ms_attention_generic(const void* q, const void* key_pool, const void* value_pool,
                                     const void* block_table, const void* seq_of_token, const void* positions,

@@ -7,7 +7,9 @@
 //        y'[i]     = y[i]*cos - y[i+D/2]*sin
 //        y'[i+D/2] = y[i+D/2]*cos + y[i]*sin
 //        reference: miniserve/model/rope.py:24-52
-//   cache write: slot = page*block_size + offset; pool[page, kv_head, offset, :]
+//   cache write: slot = page*block_size + offset; keys to key_pool[page, kv_head,
+//        offset, :], values transposed to value_pool[page, kv_head, :, offset]
+//        (the layout the matrix-core attention kernels read without a shuffle)
 //        reference: csrc/paged_kv_append.cu:28-43
 //
 // The rotation is done in 32-bit on the storage-rounded norm output and rounded
@@ -37,14 +39,19 @@ __global__ void qk_norm_rope_append_kernel(const T* __restrict__ packed, const T
   const int kv_head = is_q ? 0 : (is_k ? head - num_q_heads : head - num_q_heads - num_kv_heads);
 
   T* dst;
+  int64_t dst_stride = 1;   // distance between consecutive d
   if (is_q) {
     dst = q_out + (token * num_q_heads + head) * head_dim;
   } else {
     const int64_t slot = slot_mapping[token];
     const int64_t page = slot / block_size;
     const int64_t offset = slot - page * block_size;
-    T* pool = is_k ? key_pool : value_pool;
-    dst = pool + ((page * num_kv_heads + kv_head) * block_size + offset) * head_dim;
+    if (is_k) {
+      dst = key_pool + ((page * num_kv_heads + kv_head) * block_size + offset) * head_dim;
+    } else {
+      dst = value_pool + (page * num_kv_heads + kv_head) * head_dim * block_size + offset;
+      dst_stride = block_size;
+    }
   }
 
   float lo[kMaxPairsPerLane], hi[kMaxPairsPerLane];
@@ -91,8 +98,8 @@ __global__ void qk_norm_rope_append_kernel(const T* __restrict__ packed, const T
         a = ra;
         b = rb;
       }
-      dst[i] = ms::from_float<T>(a);
-      dst[i + half] = ms::from_float<T>(b);
+      dst[i * dst_stride] = ms::from_float<T>(a);
+      dst[(i + half) * dst_stride] = ms::from_float<T>(b);
     }
   }
 }

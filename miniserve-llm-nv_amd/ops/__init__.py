@@ -136,8 +136,9 @@ def qk_norm_rope_append(
 
     ``packed [N, (num_q_heads + 2*num_kv_heads) * head_dim]`` holds q heads, then
     k heads, then v heads.  Returns q ``[N, num_q_heads, head_dim]`` (None when
-    there are no q heads); k and v go to ``pool[page, kv_head, offset]`` with
-    ``slot = page * block_size + offset`` from ``slot_mapping`` (int32)."""
+    there are no q heads); with ``slot = page * block_size + offset`` from
+    ``slot_mapping`` (int32), k goes to ``key_pool[page, kv_head, offset, :]`` and v,
+    transposed, to ``value_pool[page, kv_head, :, offset]``."""
 
     _check(packed, "packed")
     heads = num_q_heads + 2 * num_kv_heads
@@ -162,13 +163,13 @@ def qk_norm_rope_append(
             raise KernelError("qk_norm_rope_append: a cache write needs slot_mapping and both pools.")
         _check(slot_mapping, "slot_mapping", dtype=torch.int32, shape=(n,))
         _check(key_pool, "key_pool", dtype=dtype)
-        _check(value_pool, "value_pool", dtype=dtype, shape=tuple(key_pool.shape))
         if key_pool.ndim != 4 or key_pool.shape[1] != num_kv_heads or key_pool.shape[3] != head_dim:
             raise KernelError(
                 f"qk_norm_rope_append: pool {tuple(key_pool.shape)} is not "
                 f"[pages, {num_kv_heads}, block_size, {head_dim}]."
             )
         block_size = key_pool.shape[2]
+        _check(value_pool, "value_pool", dtype=dtype, shape=_value_pool_shape(key_pool))
     q_out = None
     if num_q_heads > 0:
         q_out = torch.empty((n, num_q_heads, head_dim), dtype=dtype, device=packed.device)
@@ -176,6 +177,30 @@ def qk_norm_rope_append(
          _ptr(slot_mapping), _ptr(q_out), _ptr(key_pool), _ptr(value_pool), n, num_q_heads, num_kv_heads,
          head_dim, block_size, float(eps), _code(dtype), _stream())
     return q_out
+
+
+def _value_pool_shape(key_pool: torch.Tensor) -> tuple[int, ...]:
+    pages, kv_heads, block_size, head_dim = key_pool.shape
+    return (pages, kv_heads, head_dim, block_size)
+
+
+# Workgroups that the key-split attention aims to launch: a few per compute unit
+# (the chip has 256), so that short batches still fill it.
+_DECODE_TARGET_WORKGROUPS = 1024
+_DECODE_MAX_SPLITS = 64
+# Above this many query tokens per sequence the rows are better served as tiles of
+# queries than one by one.
+_DECODE_MAX_QUERY_LEN = 1
+
+
+def decode_splits(num_tokens: int, num_kv_heads: int, group: int, max_context: int) -> int:
+    """How many parts the keys of each row are cut into: enough workgroups to fill
+    the chip, at least 64 keys per part."""
+
+    rows = num_tokens * num_kv_heads * ((group + 15) // 16)
+    by_chip = -(-_DECODE_TARGET_WORKGROUPS // rows)
+    by_keys = max(1, max_context // 64)
+    return max(1, min(by_chip, by_keys, _DECODE_MAX_SPLITS))
 
 
 def attention(
@@ -188,23 +213,34 @@ def attention(
     positions: torch.Tensor,
     scale: float,
     window: int | None = None,
+    max_query_len: int | None = None,
+    max_context: int | None = None,
+    splits: int | None = None,
 ) -> torch.Tensor:
-    """Causal attention of ``q [N, heads, head_dim]`` over the paged cache.
+    """Causal attention of ``q [N, heads, head_dim]`` over the paged cache
+    (``key_pool [pages, kv_heads, block_size, head_dim]``, ``value_pool [pages,
+    kv_heads, head_dim, block_size]``).
 
     Token ``t`` belongs to sequence ``seq_of_token[t]``, stands at absolute
     position ``positions[t]`` and sees the keys ``lo..positions[t]`` of that
     sequence through ``block_table [S, max_blocks]`` (int32), ``lo`` being 0 or
     ``positions[t] - window + 1``.  The caller guarantees that every page the
-    table names for those keys lies inside the pool."""
+    table names for those keys lies inside the pool.
+
+    float32 runs the generic kernel, whose result for a position is bit-identical
+    for any batch.  bfloat16 runs the matrix-core kernels where they take the
+    geometry: ``max_query_len`` (the longest run of tokens of one sequence in this
+    batch; None = unknown) and ``max_context`` (the largest position + 1) choose
+    between them and size the key split; ``splits`` overrides it."""
 
     _check(q, "q")
     if q.ndim != 3 or q.shape[0] == 0:
         raise KernelError("attention: q must be [N>0, heads, head_dim].")
     n, heads, head_dim = q.shape
     _check(key_pool, "key_pool", dtype=q.dtype)
-    _check(value_pool, "value_pool", dtype=q.dtype, shape=tuple(key_pool.shape))
     if key_pool.ndim != 4 or key_pool.shape[3] != head_dim:
         raise KernelError(f"attention: pool {tuple(key_pool.shape)} is not [pages, kv_heads, block_size, {head_dim}].")
+    _check(value_pool, "value_pool", dtype=q.dtype, shape=_value_pool_shape(key_pool))
     _, kv_heads, block_size, _ = key_pool.shape
     if heads % kv_heads != 0:
         raise KernelError(f"attention: {heads} query heads are not a multiple of {kv_heads} kv heads.")
@@ -217,6 +253,23 @@ def attention(
     if window < 0:
         raise KernelError("attention: window must be positive or None.")
     out = torch.empty_like(q)
+    lib = load()
+    if (
+        q.dtype == torch.bfloat16
+        and max_query_len is not None
+        and max_query_len <= _DECODE_MAX_QUERY_LEN
+        and lib.ms_attention_decode_supported(head_dim, block_size)
+    ):
+        if splits is None:
+            splits = decode_splits(n, kv_heads, heads // kv_heads, max_context or block_table.shape[1] * block_size)
+        partial_o = partial_ml = None
+        if splits > 1:
+            partial_o = torch.empty((n, heads, splits, head_dim), dtype=torch.float32, device=q.device)
+            partial_ml = torch.empty((n, heads, splits, 2), dtype=torch.float32, device=q.device)
+        call("ms_attention_decode", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(seq_of_token),
+             _ptr(positions), _ptr(out), _ptr(partial_o), _ptr(partial_ml), n, heads, kv_heads, head_dim, block_size,
+             block_table.shape[1], float(scale), window, int(splits), _stream())
+        return out
     call("ms_attention_generic", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(seq_of_token),
          _ptr(positions), _ptr(out), n, heads, kv_heads, head_dim, block_size, block_table.shape[1], float(scale),
          window, _code(q.dtype), _stream())

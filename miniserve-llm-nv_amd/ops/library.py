@@ -27,6 +27,8 @@ _SIGNATURES: dict[str, list] = {
     "ms_residual_add": [_P, _P, _I, _I, _I, _P],
     "ms_qk_norm_rope_append": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
     "ms_attention_generic": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "ms_attention_decode": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "ms_attention_decode_supported": [_I, _I],
     "ms_gemm_f32": [_P, _P, _P, _I, _I, _I, _I, _P],
     "ms_silu_mul": [_P, _P, _I, _I, _I, _P],
     "ms_sample_rows": [_P, _P, _P, _P, _P, _P, _I, _I, _P],

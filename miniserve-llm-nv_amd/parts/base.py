@@ -78,7 +78,8 @@ class StateNeed:
 
 @dataclass
 class KVCacheView:
-    """One call's slice of its group's pools: ``[pages, kv_heads, block_size, head_dim]``."""
+    """One call's slice of its group's pools: keys ``[pages, kv_heads, block_size,
+    head_dim]``, values ``[pages, kv_heads, head_dim, block_size]``."""
 
     group: int
     key: torch.Tensor

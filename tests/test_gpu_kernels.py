@@ -137,7 +137,7 @@ def test_qk_norm_rope_append(ops, dtype, heads, kv_heads, dim, block):
     positions = torch.tensor([0, 1, 2, 63, 64, 65, 1000, 4095, 7, 7, 30000], dtype=torch.int32, device=DEVICE)
     slots = torch.randperm(pages * block, generator=torch.Generator().manual_seed(3))[:n].to(torch.int32).to(DEVICE)
     key_pool = torch.zeros(pages, kv_heads, block, dim, dtype=dtype, device=DEVICE)
-    value_pool = torch.zeros_like(key_pool)
+    value_pool = torch.zeros(pages, kv_heads, dim, block, dtype=dtype, device=DEVICE)     # transposed inside a page
     q = ops.qk_norm_rope_append(
         packed, num_q_heads=heads, num_kv_heads=kv_heads, head_dim=dim, q_weight=qw, k_weight=kw, eps=eps,
         inv_freq=inverse_frequencies(dim, theta).to(DEVICE), positions=positions, slot_mapping=slots,
@@ -157,11 +157,12 @@ def test_qk_norm_rope_append(ops, dtype, heads, kv_heads, dim, block):
     torch.testing.assert_close(q.cpu().double(), expected_q, atol=tol, rtol=tol)
     page, offset = slots.cpu().long() // block, slots.cpu().long() % block
     torch.testing.assert_close(key_pool.cpu().double()[page, :, offset], expected_k, atol=tol, rtol=tol)
-    assert torch.equal(value_pool.cpu().double()[page, :, offset], expected_v)
+    values = value_pool.cpu().double().transpose(2, 3)                                     # [page, head, offset, d]
+    assert torch.equal(values[page, :, offset], expected_v)
     touched = torch.zeros(pages, block, dtype=torch.bool)
     touched[page, offset] = True
-    untouched = lambda pool: pool.cpu().permute(0, 2, 1, 3)[~touched]
-    assert torch.all(untouched(key_pool) == 0) and torch.all(untouched(value_pool) == 0)
+    untouched = lambda pool: pool.permute(0, 2, 1, 3)[~touched]
+    assert torch.all(untouched(key_pool.cpu()) == 0) and torch.all(untouched(values) == 0)
 
 
 def test_rotation_and_norm_alone(ops):
@@ -220,7 +221,7 @@ def paged_case(batch_contexts, heads, kv_heads, dim, block, dtype, *, query_lens
     return {
         "q": torch.cat(queries).to(dtype).to(DEVICE),
         "key_pool": key_pool.to(dtype).to(DEVICE),
-        "value_pool": value_pool.to(dtype).to(DEVICE),
+        "value_pool": value_pool.transpose(2, 3).contiguous().to(dtype).to(DEVICE),      # [page, head, d, offset]
         "block_table": table.to(DEVICE),
         "seq_of_token": torch.tensor(seq_of_token, dtype=torch.int32, device=DEVICE),
         "positions": torch.tensor(positions, dtype=torch.int32, device=DEVICE),
@@ -239,9 +240,11 @@ def attention_reference(case, scale, window=None):
     return torch.cat(outs)
 
 
-def run_attention(ops, case, scale, window=None):
+def run_attention(ops, case, scale, window=None, splits=None):
     return ops.attention(case["q"], case["key_pool"], case["value_pool"], block_table=case["block_table"],
-                         seq_of_token=case["seq_of_token"], positions=case["positions"], scale=scale, window=window)
+                         seq_of_token=case["seq_of_token"], positions=case["positions"], scale=scale, window=window,
+                         max_query_len=max(case["query_lens"]), max_context=int(case["positions"].max()) + 1,
+                         splits=splits)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -285,7 +288,7 @@ def test_one_far_key_among_hundreds_stands_out(ops, dtype):
         v[far] = 100.0
         case["q"] = q.to(dtype).to(DEVICE)
         case["key_pool"][page, :, offset] = k[far].to(dtype).to(DEVICE)
-        case["value_pool"][page, :, offset] = v[far].to(dtype).to(DEVICE)
+        case["value_pool"][page, :, :, offset] = v[far].to(dtype).to(DEVICE)
         out = run_attention(ops, case, 64**-0.5)
         expected = attention_reference(case, 64**-0.5)
         assert float(expected.min()) > 10.0                                     # the far key dominates
@@ -308,11 +311,53 @@ def test_window_edges(ops, dtype, window):
             if position >= 0:
                 v[position] = value
                 page = int(case["block_table"][index, position // 8])
-                case["value_pool"][page, :, position % 8] = value
+                case["value_pool"][page, :, :, position % 8] = value
     out = run_attention(ops, case, 32**-0.5, window=window)
     expected = attention_reference(case, 32**-0.5, window=window)
     tol = tolerance(dtype, 2e-4, 8e-3)
     torch.testing.assert_close(out.cpu().double(), expected, atol=tol * 50, rtol=tol)
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,block", [(16, 8, 128, 16), (8, 1, 64, 16), (4, 4, 32, 32), (20, 1, 16, 16), (6, 2, 80, 48), (32, 2, 256, 64), (3, 1, 112, 16)])
+def test_decode_kernel_sizes_splits_and_windows(ops, heads, kv_heads, dim, block):
+    """The matrix-core kernel for single-token rows: groups of 1 to 20 query heads
+    (more than 16 take two passes), head sizes in steps of 16, contexts around
+    tile (16), pair (32) and split edges, any number of key splits, windows."""
+
+    contexts = [1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 129, 700, 2500]
+    case = paged_case(contexts, heads, kv_heads, dim, block, torch.bfloat16, seed=dim + heads)
+    assert ops.load().ms_attention_decode_supported(dim, block)
+    expected = attention_reference(case, dim**-0.5)
+    for splits in (1, 2, 5, 16, 64, None):
+        out = run_attention(ops, case, dim**-0.5, splits=splits)
+        torch.testing.assert_close(out.cpu().double(), expected, atol=8e-3, rtol=8e-3, msg=lambda m: f"splits {splits}: {m}")
+    for window in (1, 16, 17, 100, 1000):
+        expected = attention_reference(case, dim**-0.5, window=window)
+        for splits in (1, 3, None):
+            out = run_attention(ops, case, dim**-0.5, window=window, splits=splits)
+            torch.testing.assert_close(out.cpu().double(), expected, atol=8e-3, rtol=8e-3,
+                                       msg=lambda m: f"window {window} splits {splits}: {m}")
+
+
+def test_decode_kernel_ignores_stale_values(ops):
+    """Slots past the context inside the last page hold NaN (as fresh pages may):
+    a zero weight times NaN must not reach the output."""
+
+    case = paged_case([5, 21, 40], 8, 2, 64, 16, torch.bfloat16, seed=1)       # paged_case fills unused slots with NaN
+    assert torch.isnan(case["value_pool"]).any() and torch.isnan(case["key_pool"]).any()
+    out = run_attention(ops, case, 0.125)
+    assert torch.isfinite(out).all()
+    torch.testing.assert_close(out.cpu().double(), attention_reference(case, 0.125), atol=8e-3, rtol=8e-3)
+
+
+def test_decode_kernel_is_refused_for_other_geometries(ops):
+    lib = ops.load()
+    assert not lib.ms_attention_decode_supported(128, 8)          # pages of 8 keys
+    assert not lib.ms_attention_decode_supported(24, 16)          # head size off the 16 grid
+    assert not lib.ms_attention_decode_supported(272, 16)
+    case = paged_case([30, 9], 8, 1, 32, 8, torch.bfloat16, seed=2)
+    out = run_attention(ops, case, 32**-0.5)                       # falls to the generic kernel
+    torch.testing.assert_close(out.cpu().double(), attention_reference(case, 32**-0.5), atol=8e-3, rtol=8e-3)
 
 
 def test_attention_is_bit_identical_across_batches_in_float32(ops):

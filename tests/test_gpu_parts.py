@@ -146,9 +146,9 @@ def test_attention_part_whole_and_in_portions(model, dtype):
     expected_other, _ = plain.attention_block(other.double(), weights, spec.prefix, config, torch.arange(20))
 
     def fresh_cache(pages):
-        shape = (pages, config["num_key_value_heads"], block, config["head_dim"])
-        return KVCacheView(0, torch.full(shape, float("nan"), dtype=DTYPES[dtype], device=DEVICE),
-                           torch.full(shape, float("nan"), dtype=DTYPES[dtype], device=DEVICE), block)
+        heads, dim = config["num_key_value_heads"], config["head_dim"]
+        return KVCacheView(0, torch.full((pages, heads, block, dim), float("nan"), dtype=DTYPES[dtype], device=DEVICE),
+                           torch.full((pages, heads, dim, block), float("nan"), dtype=DTYPES[dtype], device=DEVICE), block)
 
     cache = fresh_cache(8)
     ctx, _ = step_context([length], [0], block)
@@ -206,8 +206,9 @@ def test_attention_part_composed_from_its_parts_equals_the_fused_kernel(model):
         results = []
         for part in (fused, composed):
             load_part_weights(part, weights)
-            shape = (4, config["num_key_value_heads"], block, config["head_dim"])
-            cache = KVCacheView(0, torch.zeros(shape, device=DEVICE), torch.zeros(shape, device=DEVICE), block)
+            heads, dim = config["num_key_value_heads"], config["head_dim"]
+            cache = KVCacheView(0, torch.zeros((4, heads, block, dim), device=DEVICE),
+                                torch.zeros((4, heads, dim, block), device=DEVICE), block)
             ctx, _ = step_context([21], [0], block)
             results.append((part.forward(x, ctx, cache), cache.key.clone(), cache.value.clone()))
         for got, want in zip(results[1], results[0]):
@@ -233,8 +234,9 @@ def test_block_embedding_and_head(model, dtype):
 
     layer = build_block(spec.layers[1], DTYPES[dtype])
     load_part_weights(layer, device_weights)
-    shape = (4, config["num_key_value_heads"], block_size, config["head_dim"])
-    cache = KVCacheView(0, torch.zeros(shape, dtype=DTYPES[dtype], device=DEVICE), torch.zeros(shape, dtype=DTYPES[dtype], device=DEVICE), block_size)
+    heads, dim = config["num_key_value_heads"], config["head_dim"]
+    cache = KVCacheView(0, torch.zeros((4, heads, block_size, dim), dtype=DTYPES[dtype], device=DEVICE),
+                        torch.zeros((4, heads, dim, block_size), dtype=DTYPES[dtype], device=DEVICE), block_size)
     ctx, _ = step_context([30], [0], block_size)
     residual, delta = layer.forward(h.clone(), None, ctx, cache)
     expected, _ = plain.decoder_layer(h.cpu().double(), weights, 1, config, torch.arange(30))
