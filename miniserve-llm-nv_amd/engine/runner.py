@@ -17,12 +17,121 @@ from ..cache import CacheLayout, CacheManager, StepItem
 from ..config import EngineConfig, load_config
 from ..parts.model import TORCH_DTYPES, DecoderModel
 from ..weights import WeightLoadReport, load_weights, random_device_tensors
+from ..parts.base import GroupStepView, StepContext
 from .batch import StepEntry, build_step_context
 
 
 def _require_gpu(device: torch.device) -> None:
     if device.type != "cuda" or not torch.cuda.is_available():
         raise RuntimeError("the engine runs on the GPU only (HIP kernels); no CPU path exists.")
+
+
+class DecodeGraph:
+    """One decode step of a fixed batch size, recorded as a HIP graph.
+
+    A step in which every request brings one token launches a few hundred small
+    kernels; recorded once and replayed, the launches cost next to nothing.  The
+    integer metadata of the step lives in one static device buffer that every
+    replay reads; a step copies its own values there (one copy from pinned host
+    memory) and replays.  Block tables have the static width of the longest
+    request the engine admits.  The graph holds no memset node: nothing in the
+    recorded step clears memory.
+    """
+
+    def __init__(self, runner: "ModelRunner", batch: int) -> None:
+        self.batch = batch
+        self.runner = runner
+        groups = len(runner.cache.layout.groups)
+        width = runner.max_blocks_per_seq
+        sizes = [("token_ids", batch), ("positions", batch), ("seq_of_token", batch), ("query_start", batch + 1),
+                 ("context_lens", batch), ("state_slots", batch), ("logit_rows", batch)]
+        for group in range(groups):
+            sizes += [(f"slots{group}", batch), (f"table{group}", batch * width)]
+        self.offsets: dict[str, tuple[int, int]] = {}
+        total = 0
+        for name, size in sizes:
+            self.offsets[name] = (total, size)
+            total += size
+        self.host = torch.zeros(total, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.meta = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        self.width = width
+        view = lambda name: self.meta[self.offsets[name][0] : self.offsets[name][0] + self.offsets[name][1]]
+        self.ctx = StepContext(
+            num_tokens=batch,
+            num_seqs=batch,
+            token_ids=view("token_ids"),
+            positions=view("positions"),
+            seq_of_token=view("seq_of_token"),
+            query_start=view("query_start"),
+            context_lens=view("context_lens"),
+            state_slots=view("state_slots"),
+            groups=[
+                GroupStepView(block_table=view(f"table{g}").view(batch, width), slot_mapping=view(f"slots{g}"))
+                for g in range(groups)
+            ],
+            query_lens=[1] * batch,
+            # launch decisions inside the graph must hold for every later step
+            context_lens_host=[runner.max_model_len] * batch,
+            query_start_host=list(range(batch + 1)),
+            state_slots_host=[0] * batch,
+            first_positions_host=[0] * batch,
+        )
+        self.rows = view("logit_rows")
+        self.graph: torch.cuda.CUDAGraph | None = None
+        self.logits: torch.Tensor | None = None
+        self.replays = 0
+
+    def _fill(self, entries: Sequence[StepEntry], reservation) -> None:
+        host, offsets, batch, width = self.host_np, self.offsets, self.batch, self.width
+
+        def put(name: str, values) -> None:
+            start, size = offsets[name]
+            host[start : start + size] = values
+
+        metas = reservation.sequences
+        put("token_ids", [entry.token_ids[0] for entry in entries])
+        put("positions", [meta.before for meta in metas])
+        put("seq_of_token", range(batch))
+        put("query_start", range(batch + 1))
+        put("context_lens", [meta.after for meta in metas])
+        put("state_slots", [meta.state_slot for meta in metas])
+        put("logit_rows", range(batch))
+        block_size = self.runner.block_size
+        for group in range(len(self.runner.cache.layout.groups)):
+            pool_pages = self.runner.cache.num_blocks[group]
+            slots = []
+            start, _ = offsets[f"table{group}"]
+            for row, meta in enumerate(metas):
+                table = meta.block_tables[group]
+                slot = meta.slot_mappings[group][0]
+                page = table[meta.before // block_size]
+                if not 0 <= page < pool_pages or slot != page * block_size + meta.before % block_size:
+                    raise RuntimeError(f"request {meta.request_id!r}: slot {slot} disagrees with its block table.")
+                slots.append(slot)
+                # a page that was given back is never read; 0 keeps the entry inside the pool
+                host[start + row * width : start + row * width + len(table)] = [p if p >= 0 else 0 for p in table]
+            put(f"slots{group}", slots)
+
+    def run(self, entries: Sequence[StepEntry], reservation) -> torch.Tensor:
+        """Logits ``[batch, vocab]`` of the step; the tensor is the graph's own output
+        buffer and holds these values until the next step of this batch size."""
+
+        self._fill(entries, reservation)
+        self.meta.copy_(self.host, non_blocking=True)
+        model, views = self.runner.model, self.runner._call_views
+        if self.graph is None:
+            # Once eagerly, so that libraries set themselves up outside the recording;
+            # running the same step twice writes the same cache slots twice.
+            model.forward(self.ctx, views, self.rows)
+            torch.cuda.synchronize(self.runner.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self.runner._graph_pool):
+                self.logits = model.forward(self.ctx, views, self.rows)
+            self.graph = graph
+        self.graph.replay()
+        self.replays += 1
+        return self.logits
 
 
 class ModelRunner:
@@ -65,8 +174,12 @@ class ModelRunner:
         )
         self.cache.allocate_storage(self.dtype, self.device)
         self._call_views = self.cache.call_views()
+        self.max_blocks_per_seq = -(-self.max_model_len // self.block_size)
+        self._decode_graphs: dict[int, DecodeGraph] = {}
+        self._graph_pool = None
         self.steps_run = 0
         self.tokens_run = 0
+        self.graph_steps = 0
 
     # ---- construction -----------------------------------------------------------------
     @classmethod
@@ -111,6 +224,27 @@ class ModelRunner:
         blocks = max(1, min(by_memory, by_need))
         return blocks
 
+    def _decode_graph_step(self, entries: Sequence[StepEntry], reservation) -> torch.Tensor | None:
+        """A step of single tokens through the recorded graph of its batch size.  The
+        graph computes the logits of every row; the wanted ones are picked."""
+
+        for entry in entries:
+            if entry.token_ids[0] >= self.spec.vocab_size:
+                raise ValueError(f"entry {entry.request_id!r}: a token id is outside the vocabulary.")
+        batch = len(entries)
+        graph = self._decode_graphs.get(batch)
+        if graph is None:
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            graph = self._decode_graphs[batch] = DecodeGraph(self, batch)
+        logits = graph.run(entries, reservation)
+        wanted = [index for index, entry in enumerate(entries) if entry.want]
+        if len(wanted) == batch:
+            return logits
+        if not wanted:
+            return None
+        return logits[torch.tensor(wanted, device=self.device)]
+
     # ---- requests -------------------------------------------------------------------
     def admit(self, request_id: str) -> int:
         return self.cache.admit(request_id)
@@ -134,6 +268,17 @@ class ModelRunner:
             start = self.cache.committed_tokens(entry.request_id)
             items.append(StepItem(entry.request_id, start, start + len(entry.token_ids)))
         reservation = self.cache.prepare_step(items)
+        if self.engine_config.decode_graphs and all(len(entry.token_ids) == 1 for entry in entries):
+            try:
+                logits = self._decode_graph_step(entries, reservation)
+            except BaseException:
+                self.cache.abort_step(reservation)
+                raise
+            self.cache.commit_step(reservation)
+            self.steps_run += 1
+            self.tokens_run += len(entries)
+            self.graph_steps += 1
+            return logits
         try:
             ctx, rows = build_step_context(
                 entries,

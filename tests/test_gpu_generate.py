@@ -205,3 +205,53 @@ def test_command_line(model_folders):
     assert [line["prompt_token_ids"] for line in lines] == [[5, 9, 200, 31], [7]]
     for line in lines:
         assert check_greedy(line["token_ids"], line["prompt_token_ids"], weights, config, "float32") == 5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_graphs_replay_like_eager_steps(dtype, model_folders):
+    """Decode steps recorded as HIP graphs, replayed many times with eager steps
+    (prompt portions, other batch sizes) and synchronisations between the
+    replays: every replay gives what the eager step gives."""
+
+    from miniserve_amd.config import EngineConfig
+    from miniserve_amd.engine import ModelRunner, StepEntry
+
+    folder, block = model_folders["a"]
+    config = read_config(folder)
+    runners = [
+        ModelRunner.from_folder(folder, EngineConfig(dtype=dtype, kv_block_size=block, num_kv_blocks=64, max_num_seqs=4,
+                                                    enable_chunked_prefill=True, decode_graphs=graphs))
+        for graphs in (True, False)
+    ]
+    tokens = {name: random_tokens(90, config["vocab_size"], seed) for seed, name in enumerate("abcd")}
+    position = {name: 0 for name in tokens}
+
+    def both(entries_of):
+        outs = []
+        for runner in runners:
+            for name in entries_of:
+                if not runner.cache.is_live(name):
+                    runner.admit(name)
+            entries = [StepEntry(n, tuple(tokens[n][position[n] : position[n] + size]), (size - 1,)) for n, size in entries_of.items()]
+            outs.append(runner.step(entries).clone())
+            torch.cuda.synchronize()
+        for name, size in entries_of.items():
+            position[name] += size
+        if dtype == "float32":
+            assert torch.equal(outs[0], outs[1])
+        else:
+            torch.testing.assert_close(outs[0], outs[1], atol=2e-2, rtol=2e-2)
+
+    both({"a": 20, "b": 33})                       # eager: prompts
+    for _ in range(6):
+        both({"a": 1, "b": 1})                     # graph of batch 2, replayed
+    both({"c": 17})                                # eager work in between
+    for _ in range(5):
+        both({"a": 1, "b": 1, "c": 1})             # graph of batch 3
+    both({"a": 1, "b": 1})                         # batch 2 again, after another graph ran
+    both({"d": 40, "a": 1})                        # a portion beside a decoded token: eager
+    for _ in range(20):
+        both({"a": 1, "b": 1, "c": 1, "d": 1})     # crosses page edges of 16
+    both({"b": 1})
+    assert runners[0].graph_steps == 33 and runners[1].graph_steps == 0
+    assert sorted(runners[0]._decode_graphs) == [1, 2, 3, 4]
