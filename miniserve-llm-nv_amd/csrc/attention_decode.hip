@@ -7,7 +7,9 @@
 // its share of the keys in tiles of 16 keys, two tiles (32 keys) per MFMA; each
 // wave keeps an online softmax (running max m, sum l) in 32-bit and an
 // unnormalised output tile in 32-bit; the waves are merged through LDS; a split
-// writes its (m, l, O) and a second kernel merges the splits.
+// writes its (m, l, O) and a second kernel merges the splits.  (Merging in the
+// split that finishes last would need a device-wide fence per workgroup, which
+// on this chip writes back the whole L2 of its die: measured 3x slower.)
 //
 //   S^T[key, head] = K[key, :] . Q[head, :]      A = K tile (16 keys x 32 d), B = Q^T
 //   P = exp(S * scale - m)                        (scale after the product, as the
@@ -33,15 +35,128 @@ constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * ms::kWave;
 constexpr int kTileKeys = 16;
 
+// The keys and values of two tiles (32 keys), as they are loaded: operands of the
+// matrix cores without any rearrangement.
 template <int D>
-__global__ __launch_bounds__(kThreads) void attention_decode_kernel(
+struct TilePair {
+  static constexpr int KS = (D + 31) / 32;   // 32-wide slices of d for Q.K
+  static constexpr int CS = D / 16;          // 16-wide slices of d for P.V
+  bf16x8 k_a[KS], k_b[KS];
+  bf16x4 v_a[CS], v_b[CS];
+  bool has_b;
+};
+
+template <int D>
+__device__ __forceinline__ void load_pair(TilePair<D>& pair, int tile, int end_tile, const int32_t* __restrict__ table,
+                                          const bf16* __restrict__ key_pool, const bf16* __restrict__ value_pool,
+                                          int num_kv_heads, int kv_head, int block_size, int g, int r) {
+  const bool has_b = tile + 1 < end_tile;
+  pair.has_b = has_b;
+  const int key_a = tile * kTileKeys;
+  const int key_b = key_a + kTileKeys;
+  const int64_t page_a = table[key_a / block_size];
+  const int off_a = key_a % block_size;
+  const int64_t page_b = has_b ? table[key_b / block_size] : page_a;
+  const int off_b = has_b ? key_b % block_size : off_a;
+  const bf16* k_row_a = key_pool + ((page_a * num_kv_heads + kv_head) * block_size + off_a + r) * D;
+  const bf16* k_row_b = key_pool + ((page_b * num_kv_heads + kv_head) * block_size + off_b + r) * D;
+  const bf16* v_a = value_pool + (page_a * num_kv_heads + kv_head) * D * block_size + off_a + 4 * g;
+  const bf16* v_b = value_pool + (page_b * num_kv_heads + kv_head) * D * block_size + off_b + 4 * g;
+#pragma unroll
+  for (int s = 0; s < TilePair<D>::KS; ++s) {
+    const int d0 = 32 * s + 8 * g;
+    pair.k_a[s] = d0 < D ? ms::load_bf16x8(k_row_a + d0) : ms::zero_bf16x8();
+    pair.k_b[s] = (has_b && d0 < D) ? ms::load_bf16x8(k_row_b + d0) : ms::zero_bf16x8();
+  }
+#pragma unroll
+  for (int c = 0; c < TilePair<D>::CS; ++c) {
+    const int64_t d = 16 * c + r;
+    pair.v_a[c] = ms::load_bf16x4(v_a + d * block_size);
+    pair.v_b[c] = has_b ? ms::load_bf16x4(v_b + d * block_size) : ms::zero_bf16x4();
+  }
+}
+
+// Online-softmax state of one wave: head r's running max and sum (the same in all
+// four lane groups) and the unnormalised output tile.
+template <int D>
+struct WaveState {
+  floatx4 o[D / 16];
+  float run_max, run_sum;
+};
+
+template <int D>
+__device__ __forceinline__ void consume_pair(WaveState<D>& st, TilePair<D>& pair, const bf16x8* q_reg, int tile,
+                                             int lo, int pos, float scale, int g) {
+  constexpr int KS = TilePair<D>::KS, CS = TilePair<D>::CS;
+  const int key_a = tile * kTileKeys, key_b = key_a + kTileKeys;
+  // ---- S^T = K . Q^T ---------------------------------------------------------
+  floatx4 s_a = {0.f, 0.f, 0.f, 0.f}, s_b = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    s_a = ms::mfma_16x16x32(pair.k_a[s], q_reg[s], s_a);
+    s_b = ms::mfma_16x16x32(pair.k_b[s], q_reg[s], s_b);
+  }
+  // this lane: head r, keys key_a + 4 g + e and key_b + 4 g + e
+  bool ok_a[4], ok_b[4];
+  float tile_max = -INFINITY;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int ka = key_a + 4 * g + e, kb = key_b + 4 * g + e;
+    ok_a[e] = ka >= lo && ka <= pos;
+    ok_b[e] = pair.has_b && kb >= lo && kb <= pos;
+    s_a[e] = ok_a[e] ? s_a[e] * scale : -INFINITY;
+    s_b[e] = ok_b[e] ? s_b[e] * scale : -INFINITY;
+    tile_max = fmaxf(tile_max, fmaxf(s_a[e], s_b[e]));
+  }
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, ms::kWave));
+  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, ms::kWave));
+  const float new_max = fmaxf(st.run_max, tile_max);   // finite: every tile of the range holds a visible key
+  const float alpha = __expf(st.run_max - new_max);
+  float tile_sum = 0.f;
+  bf16x8 p;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float pa = __expf(s_a[e] - new_max);
+    const float pb = __expf(s_b[e] - new_max);
+    tile_sum += pa + pb;
+    p[e] = static_cast<__bf16>(pa);
+    p[e + 4] = static_cast<__bf16>(pb);
+  }
+  tile_sum += __shfl_xor(tile_sum, 16, ms::kWave);
+  tile_sum += __shfl_xor(tile_sum, 32, ms::kWave);
+  st.run_sum = st.run_sum * alpha + tile_sum;
+  st.run_max = new_max;
+
+  // ---- O = alpha O + P . V ---------------------------------------------------
+  // O's rows in this lane are the heads 4 g + e; their alpha lives in lane 4 g + e.
+  float alpha_row[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) alpha_row[e] = __shfl(alpha, 4 * g + e, ms::kWave);
+  const bool partial = !(ok_a[0] && ok_a[3] && ok_b[0] && ok_b[3]);
+#pragma unroll
+  for (int c = 0; c < CS; ++c) {
+    bf16x4 va = pair.v_a[c], vb = pair.v_b[c];
+    if (partial) {   // a stale value times a zero weight must not become NaN
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (!ok_a[e]) va[e] = static_cast<__bf16>(0.0f);
+        if (!ok_b[e]) vb[e] = static_cast<__bf16>(0.0f);
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) st.o[c][e] *= alpha_row[e];
+    st.o[c] = ms::mfma_16x16x32(p, ms::concat(va, vb), st.o[c]);
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(kThreads) MS_WAVES_PER_EU(D <= 128 ? 2 : 1, 2) void attention_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ key_pool, const bf16* __restrict__ value_pool,
     const int32_t* __restrict__ block_table, const int32_t* __restrict__ seq_of_token,
     const int32_t* __restrict__ positions, bf16* __restrict__ out, float* __restrict__ partial_o,
     float* __restrict__ partial_ml, int num_q_heads, int num_kv_heads, int block_size, int max_blocks, float scale,
     int window, int num_splits) {
-  constexpr int KS = (D + 31) / 32;   // 32-wide slices of d for Q.K
-  constexpr int CS = D / 16;          // 16-wide slices of d for P.V
+  constexpr int KS = TilePair<D>::KS, CS = TilePair<D>::CS;
 
   __shared__ float o_s[kWaves - 1][16][D];
   __shared__ float m_s[kWaves][16];
@@ -80,104 +195,53 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
                                           : ms::zero_bf16x8();
   }
 
-  floatx4 o[CS];
+  WaveState<D> st;
 #pragma unroll
-  for (int c = 0; c < CS; ++c) o[c] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float run_max = -INFINITY;   // of head r
-  float run_sum = 0.f;
+  for (int c = 0; c < CS; ++c) st.o[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+  st.run_max = -INFINITY;
+  st.run_sum = 0.f;
 
-  for (int t = t0 + 2 * wave; t < t1; t += 2 * kWaves) {
-    const bool has_b = t + 1 < t1;
-    const int key_a = t * kTileKeys;
-    const int key_b = key_a + kTileKeys;
-    const int64_t page_a = table[key_a / block_size];
-    const int off_a = key_a % block_size;
-    const int64_t page_b = has_b ? table[key_b / block_size] : page_a;
-    const int off_b = has_b ? key_b % block_size : off_a;
-
-    // ---- S^T = K . Q^T ------------------------------------------------------
-    const bf16* k_row_a = key_pool + ((page_a * num_kv_heads + kv_head) * block_size + off_a + r) * D;
-    const bf16* k_row_b = key_pool + ((page_b * num_kv_heads + kv_head) * block_size + off_b + r) * D;
-    floatx4 s_a = {0.f, 0.f, 0.f, 0.f}, s_b = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int d0 = 32 * s + 8 * g;
-      const bf16x8 ka = d0 < D ? ms::load_bf16x8(k_row_a + d0) : ms::zero_bf16x8();
-      s_a = ms::mfma_16x16x32(ka, q_reg[s], s_a);
-      if (has_b) {
-        const bf16x8 kb = d0 < D ? ms::load_bf16x8(k_row_b + d0) : ms::zero_bf16x8();
-        s_b = ms::mfma_16x16x32(kb, q_reg[s], s_b);
-      }
+  // The wave's pairs of tiles, the loads of the next pair in flight while the
+  // current one is consumed.
+  constexpr int kStep = 2 * kWaves;
+  constexpr bool kPrefetch = D <= 128;      // larger heads would spill registers
+  int t = t0 + 2 * wave;
+  if (!kPrefetch) {
+    for (; t < t1; t += kStep) {
+      TilePair<D> pair;
+      load_pair<D>(pair, t, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+      consume_pair<D>(st, pair, q_reg, t, lo, pos, scale, g);
     }
-    // this lane: head r, keys key_a + 4 g + e and key_b + 4 g + e
-    bool ok_a[4], ok_b[4];
-    float tile_max = -INFINITY;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int ka = key_a + 4 * g + e, kb = key_b + 4 * g + e;
-      ok_a[e] = ka >= lo && ka <= pos;
-      ok_b[e] = has_b && kb >= lo && kb <= pos;
-      s_a[e] = ok_a[e] ? s_a[e] * scale : -INFINITY;
-      s_b[e] = ok_b[e] ? s_b[e] * scale : -INFINITY;
-      tile_max = fmaxf(tile_max, fmaxf(s_a[e], s_b[e]));
-    }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, ms::kWave));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, ms::kWave));
-    const float new_max = fmaxf(run_max, tile_max);   // finite: every tile of the range holds a visible key
-    const float alpha = __expf(run_max - new_max);
-    float tile_sum = 0.f;
-    bf16x8 p;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float pa = __expf(s_a[e] - new_max);
-      const float pb = __expf(s_b[e] - new_max);
-      tile_sum += pa + pb;
-      p[e] = static_cast<__bf16>(pa);
-      p[e + 4] = static_cast<__bf16>(pb);
-    }
-    tile_sum += __shfl_xor(tile_sum, 16, ms::kWave);
-    tile_sum += __shfl_xor(tile_sum, 32, ms::kWave);
-    run_sum = run_sum * alpha + tile_sum;
-    run_max = new_max;
-
-    // ---- O = alpha O + P . V ------------------------------------------------
-    // O's rows in this lane are the heads 4 g + e; their alpha lives in lane 4 g + e.
-    float alpha_row[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) alpha_row[e] = __shfl(alpha, 4 * g + e, ms::kWave);
-    const bool partial = !(ok_a[0] && ok_a[3] && ok_b[0] && ok_b[3]);
-    const bf16* v_a = value_pool + (page_a * num_kv_heads + kv_head) * D * block_size + off_a + 4 * g;
-    const bf16* v_b = value_pool + (page_b * num_kv_heads + kv_head) * D * block_size + off_b + 4 * g;
-#pragma unroll
-    for (int c = 0; c < CS; ++c) {
-      const int d = 16 * c + r;
-      bf16x4 va = ms::load_bf16x4(v_a + static_cast<int64_t>(d) * block_size);
-      bf16x4 vb = has_b ? ms::load_bf16x4(v_b + static_cast<int64_t>(d) * block_size) : ms::zero_bf16x4();
-      if (partial) {   // a stale value times a zero weight must not become NaN
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (!ok_a[e]) va[e] = static_cast<__bf16>(0.0f);
-          if (!ok_b[e]) vb[e] = static_cast<__bf16>(0.0f);
-        }
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o[c][e] *= alpha_row[e];
-      o[c] = ms::mfma_16x16x32(p, ms::concat(va, vb), o[c]);
+  } else if (t < t1) {
+    TilePair<D> ping, pong;
+    load_pair<D>(ping, t, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+    while (true) {
+      int next = t + kStep;
+      if (next < t1) load_pair<D>(pong, next, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+      consume_pair<D>(st, ping, q_reg, t, lo, pos, scale, g);
+      t = next;
+      if (t >= t1) break;
+      next = t + kStep;
+      if (next < t1) load_pair<D>(ping, next, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+      consume_pair<D>(st, pong, q_reg, t, lo, pos, scale, g);
+      t = next;
+      if (t >= t1) break;
     }
   }
 
-  // ---- merge the waves ------------------------------------------------------
+  // ---- merge the waves through LDS, into wave 0 -------------------------------
   if (g == 0) {
-    m_s[wave][r] = run_max;
-    l_s[wave][r] = run_sum;
+    m_s[wave][r] = st.run_max;
+    l_s[wave][r] = st.run_sum;
   }
   if (wave > 0) {
 #pragma unroll
     for (int c = 0; c < CS; ++c)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o_s[wave - 1][4 * g + e][16 * c + r] = o[c][e];
+      for (int e = 0; e < 4; ++e) o_s[wave - 1][4 * g + e][16 * c + r] = st.o[c][e];
   }
   __syncthreads();
+
   if (wave != 0) return;
 
   float total_max[4], total_sum[4], factor[kWaves][4];
@@ -200,13 +264,12 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
   for (int c = 0; c < CS; ++c) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      float acc = o[c][e] * factor[0][e];
+      float acc = st.o[c][e] * factor[0][e];
 #pragma unroll
       for (int w = 1; w < kWaves; ++w) acc += o_s[w - 1][4 * g + e][16 * c + r] * factor[w][e];
-      o[c][e] = acc;
+      st.o[c][e] = acc;
     }
   }
-
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int row = 4 * g + e;
@@ -216,12 +279,12 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
       const float inv = 1.0f / total_sum[e];
       bf16* dst = out + (token * num_q_heads + head) * D;
 #pragma unroll
-      for (int c = 0; c < CS; ++c) dst[16 * c + r] = ms::from_float<bf16>(o[c][e] * inv);
+      for (int c = 0; c < CS; ++c) dst[16 * c + r] = ms::from_float<bf16>(st.o[c][e] * inv);
     } else {
       const int64_t slot = (token * num_q_heads + head) * num_splits + split;
       float* dst = partial_o + slot * D;
 #pragma unroll
-      for (int c = 0; c < CS; ++c) dst[16 * c + r] = o[c][e];
+      for (int c = 0; c < CS; ++c) dst[16 * c + r] = st.o[c][e];
       if (r == 0) {
         partial_ml[2 * slot] = total_max[e];
         partial_ml[2 * slot + 1] = total_sum[e];
@@ -230,22 +293,32 @@ __global__ __launch_bounds__(kThreads) void attention_decode_kernel(
   }
 }
 
-// One wave per (token, head): out = sum_s e^{m_s - M} O_s / sum_s e^{m_s - M} l_s.
+// Merge of the splits, one workgroup per (token, head):
+//   out = sum_s e^{m_s - M} O_s / sum_s e^{m_s - M} l_s,  M = max_s m_s.
+// The first wave turns the (m_s, l_s) into weights, then every thread owns one
+// column of the head.  At most 64 splits.
 __global__ void attention_merge_splits_kernel(const float* __restrict__ partial_o,
                                               const float* __restrict__ partial_ml, bf16* __restrict__ out,
                                               int head_dim, int num_splits) {
+  __shared__ float weight_s[ms::kWave];
   const int64_t row = blockIdx.x;
-  const float* ml = partial_ml + row * num_splits * 2;
-  float mx = -INFINITY;
-  for (int s = 0; s < num_splits; ++s) mx = fmaxf(mx, ml[2 * s]);
-  float sum = 0.f;
-  for (int s = 0; s < num_splits; ++s) sum += __expf(ml[2 * s] - mx) * ml[2 * s + 1];
-  const float inv = 1.0f / sum;
+  if (threadIdx.x < ms::kWave) {
+    const int s = threadIdx.x;
+    const bool live = s < num_splits;
+    const float m = live ? partial_ml[2 * (row * num_splits + s)] : -INFINITY;
+    const float l = live ? partial_ml[2 * (row * num_splits + s) + 1] : 0.f;
+    const float mx = ms::wave_max(m);
+    const float f = live ? __expf(m - mx) : 0.f;
+    const float total = ms::wave_sum(f * l);
+    weight_s[s] = f / total;
+  }
+  __syncthreads();
   for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    const float* column = partial_o + row * num_splits * head_dim + d;
     float acc = 0.f;
-    for (int s = 0; s < num_splits; ++s)
-      acc += __expf(ml[2 * s] - mx) * partial_o[(row * num_splits + s) * head_dim + d];
-    out[row * head_dim + d] = ms::from_float<bf16>(acc * inv);
+#pragma unroll 8
+    for (int s = 0; s < num_splits; ++s) acc = fmaf(weight_s[s], column[static_cast<int64_t>(s) * head_dim], acc);
+    out[row * head_dim + d] = ms::from_float<bf16>(acc);
   }
 }
 
@@ -276,7 +349,8 @@ extern "C" int ms_attention_decode_supported(int head_dim, int block_size) {
 // q, out: bfloat16 [num_tokens, num_q_heads, head_dim]; key_pool: [pages, kv_heads,
 // block_size, head_dim]; value_pool: [pages, kv_heads, head_dim, block_size];
 // partial_o: float [num_tokens, num_q_heads, num_splits, head_dim] and partial_ml:
-// float [num_tokens, num_q_heads, num_splits, 2], both unused when num_splits == 1.
+// float [num_tokens, num_q_heads, num_splits, 2], both unused when num_splits == 1
+// (at most 64 splits).
 extern "C" int ms_attention_decode(const void* q, const void* key_pool, const void* value_pool,
                                    const void* block_table, const void* seq_of_token, const void* positions,
                                    void* out, void* partial_o, void* partial_ml, int num_tokens, int num_q_heads,
@@ -289,7 +363,7 @@ extern "C" int ms_attention_decode(const void* q, const void* key_pool, const vo
              "attention_decode: head_dim %d (multiples of 16 up to 256) or block_size %d (multiples of 16) "
              "is not supported",
              head_dim, block_size);
-  MS_REQUIRE(num_splits >= 1 && num_splits <= 1024, "attention_decode: %d splits", num_splits);
+  MS_REQUIRE(num_splits >= 1 && num_splits <= ms::kWave, "attention_decode: %d splits are outside 1..64", num_splits);
   MS_REQUIRE(num_splits == 1 || (partial_o && partial_ml), "attention_decode: splits need partial buffers");
   MS_REQUIRE(max_blocks > 0 && window >= 0, "attention_decode: bad table width or window");
   MS_REQUIRE(num_kv_heads * ((num_q_heads / num_kv_heads + 15) / 16) <= 65535, "attention_decode: too many heads");
@@ -310,7 +384,8 @@ extern "C" int ms_attention_decode(const void* q, const void* key_pool, const vo
 #undef MS_DECODE_CASE
   MS_CHECK_LAUNCH("attention_decode");
   if (num_splits > 1) {
-    hipLaunchKernelGGL(attention_merge_splits_kernel, dim3(num_tokens * num_q_heads), dim3(ms::kWave), 0, stream,
+    const int threads = head_dim <= 64 ? 64 : (head_dim <= 128 ? 128 : 256);
+    hipLaunchKernelGGL(attention_merge_splits_kernel, dim3(num_tokens * num_q_heads), dim3(threads), 0, stream,
                        static_cast<const float*>(partial_o), static_cast<const float*>(partial_ml),
                        static_cast<bf16*>(out), head_dim, num_splits);
     MS_CHECK_LAUNCH("attention_merge_splits");

@@ -4,6 +4,11 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// Occupancy hint for a kernel: the register budget is set for `lo`..`hi` waves per SIMD.
+#ifndef MS_WAVES_PER_EU
+#define MS_WAVES_PER_EU(lo, hi) __attribute__((amdgpu_waves_per_eu(lo, hi)))
+#endif
+
 namespace ms {
 
 constexpr int kWave = 64;

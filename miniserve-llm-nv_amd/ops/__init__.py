@@ -186,7 +186,7 @@ def _value_pool_shape(key_pool: torch.Tensor) -> tuple[int, ...]:
 
 # Workgroups that the key-split attention aims to launch: a few per compute unit
 # (the chip has 256), so that short batches still fill it.
-_DECODE_TARGET_WORKGROUPS = 1024
+_DECODE_TARGET_WORKGROUPS = 512
 _DECODE_MAX_SPLITS = 64
 # Above this many query tokens per sequence the rows are better served as tiles of
 # queries than one by one.
