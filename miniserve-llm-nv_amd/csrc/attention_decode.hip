@@ -22,7 +22,7 @@
 //
 // Formula of the one-token form: reference csrc/paged_decode_attention.cu:44-94.
 // Unlike there, no shared memory grows with the context.
-#include "mfma.hpp"
+#include "attention_tiles.hpp"
 
 namespace {
 
@@ -31,50 +31,12 @@ using ms::bf16x4;
 using ms::bf16x8;
 using ms::floatx4;
 
+using ms::kTileKeys;
+using ms::load_pair;
+using ms::TilePair;
+
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * ms::kWave;
-constexpr int kTileKeys = 16;
-
-// The keys and values of two tiles (32 keys), as they are loaded: operands of the
-// matrix cores without any rearrangement.
-template <int D>
-struct TilePair {
-  static constexpr int KS = (D + 31) / 32;   // 32-wide slices of d for Q.K
-  static constexpr int CS = D / 16;          // 16-wide slices of d for P.V
-  bf16x8 k_a[KS], k_b[KS];
-  bf16x4 v_a[CS], v_b[CS];
-  bool has_b;
-};
-
-template <int D>
-__device__ __forceinline__ void load_pair(TilePair<D>& pair, int tile, int end_tile, const int32_t* __restrict__ table,
-                                          const bf16* __restrict__ key_pool, const bf16* __restrict__ value_pool,
-                                          int num_kv_heads, int kv_head, int block_size, int g, int r) {
-  const bool has_b = tile + 1 < end_tile;
-  pair.has_b = has_b;
-  const int key_a = tile * kTileKeys;
-  const int key_b = key_a + kTileKeys;
-  const int64_t page_a = table[key_a / block_size];
-  const int off_a = key_a % block_size;
-  const int64_t page_b = has_b ? table[key_b / block_size] : page_a;
-  const int off_b = has_b ? key_b % block_size : off_a;
-  const bf16* k_row_a = key_pool + ((page_a * num_kv_heads + kv_head) * block_size + off_a + r) * D;
-  const bf16* k_row_b = key_pool + ((page_b * num_kv_heads + kv_head) * block_size + off_b + r) * D;
-  const bf16* v_a = value_pool + (page_a * num_kv_heads + kv_head) * D * block_size + off_a + 4 * g;
-  const bf16* v_b = value_pool + (page_b * num_kv_heads + kv_head) * D * block_size + off_b + 4 * g;
-#pragma unroll
-  for (int s = 0; s < TilePair<D>::KS; ++s) {
-    const int d0 = 32 * s + 8 * g;
-    pair.k_a[s] = d0 < D ? ms::load_bf16x8(k_row_a + d0) : ms::zero_bf16x8();
-    pair.k_b[s] = (has_b && d0 < D) ? ms::load_bf16x8(k_row_b + d0) : ms::zero_bf16x8();
-  }
-#pragma unroll
-  for (int c = 0; c < TilePair<D>::CS; ++c) {
-    const int64_t d = 16 * c + r;
-    pair.v_a[c] = ms::load_bf16x4(v_a + d * block_size);
-    pair.v_b[c] = has_b ? ms::load_bf16x4(v_b + d * block_size) : ms::zero_bf16x4();
-  }
-}
 
 // Online-softmax state of one wave: head r's running max and sum (the same in all
 // four lane groups) and the unnormalised output tile.

@@ -1,0 +1,191 @@
+// Matrix product for few rows (decoding): out[M, N] = x[M, K] . W[N, K]^T with
+// M <= 64, bfloat16 inputs, 32-bit accumulation on the matrix cores.  The weight
+// matrix is streamed exactly once at 16 bytes a lane; the step is bound by that
+// stream, so the kernel is built around keeping many loads in flight.
+//
+//   C^T[n, m] += W[n, k] x[m, k]        A = W tile (16 rows x 32 k), B = x^T
+//
+// A workgroup of 8 waves owns RB blocks of 16 rows of W; the waves split K between
+// them in steps of 32 (wave w takes steps w, w + 8, ...), so that one round of the
+// workgroup reads 512 contiguous bytes of every row.  The waves' partial tiles are
+// summed through LDS in a fixed order; every output element is written by one
+// workgroup: results do not depend on anything but their own row of x and of W.
+//
+// Epilogues (what the reference does in separate torch calls):
+//   0  out = bf16(C)                                   nn.Linear (qwen3.py:174-176)
+//   1  out_f32 = C                                     logits (qwen3.py:558)
+//   2  out_f32 += C                                    residual add (qwen3.py:367-368, 381-382)
+//   3  out = bf16(silu(C[gate row]) * C[up row])       gated activation (layers.py:86-87);
+//      the workgroup owns row n of the gate half and row n + N/2 of the up half
+#include "mfma.hpp"
+
+namespace {
+
+using ms::bf16;
+using ms::bf16x8;
+using ms::floatx4;
+
+constexpr int kWavesPerGroup = 8;
+constexpr int kGroupThreads = kWavesPerGroup * ms::kWave;
+constexpr int kUnroll = 4;   // k-steps whose loads are issued together
+
+enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAddF32 = 2, kSiluMul = 3 };
+
+template <int MB, int RB>
+__global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* __restrict__ x,
+                                                                    const bf16* __restrict__ w, bf16* out_bf16,
+                                                                    float* out_f32, int m, int n, int k,
+                                                                    int epilogue) {
+  __shared__ float c_s[kWavesPerGroup][RB * MB][16][16];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int g = lane >> 4;
+  const int r = lane & 15;
+
+  // Rows of W of this workgroup: block rb starts at row_start[rb].
+  const int half = n / 2;
+  int row_start[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    if (epilogue == kSiluMul) {
+      // RB is even: blocks 0..RB/2-1 are gate rows, the others the matching up rows
+      const int pair = rb % (RB / 2 > 0 ? RB / 2 : 1);
+      row_start[rb] = (blockIdx.x * (RB / 2 > 0 ? RB / 2 : 1) + pair) * 16 + (rb >= RB / 2 ? half : 0);
+    } else {
+      row_start[rb] = (blockIdx.x * RB + rb) * 16;
+    }
+  }
+  const int row_limit = epilogue == kSiluMul ? half : n;   // rows of one half for the gated form
+
+  const bf16* w_row[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    // a row past the end is read from the last row and never stored
+    int local = row_start[rb] - (epilogue == kSiluMul && rb >= RB / 2 ? half : 0) + r;
+    local = min(local, row_limit - 1);
+    const int row = local + (epilogue == kSiluMul && rb >= RB / 2 ? half : 0);
+    w_row[rb] = w + static_cast<int64_t>(row) * k;
+  }
+  const bf16* x_row[MB];
+  bool x_live[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int row = 16 * mb + r;
+    x_live[mb] = row < m;
+    x_row[mb] = x + static_cast<int64_t>(min(row, m - 1)) * k;
+  }
+
+  floatx4 acc[RB][MB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int steps = (k + 31) / 32;
+  for (int base = wave; base < steps; base += kWavesPerGroup * kUnroll) {
+    bf16x8 a[kUnroll][RB], b[kUnroll][MB];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int k0 = 32 * (base + u * kWavesPerGroup) + 8 * g;
+      const bool live = k0 < k;      // k is a multiple of 8
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) a[u][rb] = live ? ms::load_bf16x8(w_row[rb] + k0) : ms::zero_bf16x8();
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        b[u][mb] = (live && x_live[mb]) ? ms::load_bf16x8(x_row[mb] + k0) : ms::zero_bf16x8();
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = ms::mfma_16x16x32(a[u][rb], b[u][mb], acc[rb][mb]);
+  }
+
+  // this lane: column m = 16 mb + r, rows 4 g + e of block rb
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) c_s[wave][rb * MB + mb][r][4 * g + e] = acc[rb][mb][e];
+  __syncthreads();
+
+  // c_s[wave][tile][m_local][n_local]; consecutive threads take consecutive n
+  constexpr int kOutBlocks = RB;     // for the gated form half of them are outputs
+  const int out_blocks = epilogue == kSiluMul ? RB / 2 : kOutBlocks;
+  for (int index = threadIdx.x; index < out_blocks * MB * 256; index += kGroupThreads) {
+    const int n_local = index & 15;
+    const int m_local = (index >> 4) & 15;
+    const int tile = index >> 8;
+    const int rb = tile / MB, mb = tile - rb * MB;
+    const int row_m = 16 * mb + m_local;
+    const int col_n = row_start[rb] + n_local;
+    if (row_m >= m || col_n >= row_limit) continue;
+    float sum = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < kWavesPerGroup; ++wv) sum += c_s[wv][tile][m_local][n_local];
+    if (epilogue == kStoreBf16) {
+      out_bf16[static_cast<int64_t>(row_m) * n + col_n] = ms::from_float<bf16>(sum);
+    } else if (epilogue == kStoreF32) {
+      out_f32[static_cast<int64_t>(row_m) * n + col_n] = sum;
+    } else if (epilogue == kAddF32) {
+      out_f32[static_cast<int64_t>(row_m) * n + col_n] += sum;
+    } else {
+      float up = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < kWavesPerGroup; ++wv) up += c_s[wv][(rb + RB / 2) * MB + mb][m_local][n_local];
+      const float gate = ms::round_to<bf16>(sum);
+      up = ms::round_to<bf16>(up);
+      out_bf16[static_cast<int64_t>(row_m) * half + col_n] = ms::from_float<bf16>(gate / (1.0f + __expf(-gate)) * up);
+    }
+  }
+}
+
+template <int MB, int RB>
+void launch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, int n, int k, int epilogue,
+            hipStream_t stream) {
+  const int rows = epilogue == kSiluMul ? n / 2 : n;
+  const int blocks_per_group = epilogue == kSiluMul ? RB / 2 : RB;
+  const int groups = (rows + 16 * blocks_per_group - 1) / (16 * blocks_per_group);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB>), dim3(groups), dim3(kGroupThreads), 0, stream,
+                     static_cast<const bf16*>(x), static_cast<const bf16*>(w), static_cast<bf16*>(out_bf16),
+                     static_cast<float*>(out_f32), m, n, k, epilogue);
+}
+
+}  // namespace
+
+extern "C" int ms_gemm_skinny_supported(int m, int n, int k, int epilogue) {
+  if (m < 1 || m > 64 || n < 1 || k < 8 || k % 8 != 0) return 0;
+  if (epilogue == kSiluMul && n % 2 != 0) return 0;
+  return epilogue >= 0 && epilogue <= 3;
+}
+
+// x: bfloat16 [m, k]; w: bfloat16 [n, k]; the output by epilogue: 0 bfloat16 [m, n],
+// 1 and 2 float [m, n], 3 bfloat16 [m, n / 2].
+extern "C" int ms_gemm_skinny(const void* x, const void* w, void* out_bf16, void* out_f32, int m, int n, int k,
+                              int epilogue, hipStream_t stream) {
+  MS_REQUIRE(ms_gemm_skinny_supported(m, n, k, epilogue),
+             "gemm_skinny: m %d (1..64), n %d, k %d (a multiple of 8) or epilogue %d is not supported", m, n, k,
+             epilogue);
+  MS_REQUIRE((epilogue == kStoreBf16 || epilogue == kSiluMul) ? out_bf16 != nullptr : out_f32 != nullptr,
+             "gemm_skinny: the output of epilogue %d is null", epilogue);
+  const int mb = (m + 15) / 16;
+  const bool many_rows = (epilogue == kSiluMul ? n / 2 : n) >= 32768;   // the head: larger tiles, fewer workgroups
+  if (epilogue == kSiluMul) {
+    if (mb == 1) launch<1, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+    else if (mb == 2) launch<2, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+    else launch<4, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+  } else if (mb == 1) {
+    if (many_rows) launch<1, 4>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+    else launch<1, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+  } else if (mb == 2) {
+    if (many_rows) launch<2, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+    else launch<2, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+  } else {
+    launch<4, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+  }
+  MS_CHECK_LAUNCH("gemm_skinny");
+  return 0;
+}

@@ -5,8 +5,9 @@
 // the weight, the order of the reference (miniserve/model/layers.py:30-34,
 // csrc/rmsnorm.cu:92-105).  In 32-bit storage the rounding is the identity.
 //
-// One workgroup per output row.  The number of threads depends on the row
-// length only, so a row's result never depends on the rest of the batch.
+// One workgroup per output row.  The number of threads and the kernel variant
+// depend on the row length only, so a row's result never depends on the rest of
+// the batch.
 #include "common.hpp"
 
 namespace {
@@ -44,6 +45,70 @@ __global__ void rmsnorm_kernel(TIn* __restrict__ x, const T* __restrict__ delta,
   }
 }
 
+// The same with the row kept in registers between the two passes: one read of the
+// row instead of two.  EPT values per thread; the row has at most EPT * blockDim.x.
+template <typename TIn, typename T, int EPT>
+__global__ void rmsnorm_registers_kernel(TIn* __restrict__ x, const T* __restrict__ delta,
+                                         const T* __restrict__ weight, T* __restrict__ out,
+                                         const int32_t* __restrict__ rows, int dim, float eps, int write_back) {
+  __shared__ float scratch[16];
+  const int64_t out_row = blockIdx.x;
+  const int64_t in_row = rows ? static_cast<int64_t>(rows[out_row]) : out_row;
+  TIn* xr = x + in_row * dim;
+  const T* dr = delta ? delta + in_row * dim : nullptr;
+  T* yr = out + out_row * dim;
+
+  float v[EPT];
+  float partial = 0.f;
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int i = threadIdx.x + e * blockDim.x;
+    v[e] = 0.f;
+    if (i < dim) {
+      v[e] = ms::to_float(xr[i]);
+      if (dr) {
+        v[e] += ms::to_float(dr[i]);
+        if (write_back) {
+          xr[i] = ms::from_float<TIn>(v[e]);
+          v[e] = ms::round_to<TIn>(v[e]);     // what a second read of x would see
+        }
+      }
+      partial = fmaf(v[e], v[e], partial);
+    }
+  }
+  const float total = ms::block_sum(partial, scratch);
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(dim) + eps);
+#pragma unroll
+  for (int e = 0; e < EPT; ++e) {
+    const int i = threadIdx.x + e * blockDim.x;
+    if (i < dim) yr[i] = ms::from_float<T>(ms::to_float(weight[i]) * ms::round_to<T>(v[e] * inv));
+  }
+}
+
+template <typename TIn, typename T>
+void launch_rmsnorm(void* x, const void* delta, const void* weight, void* out, const void* rows, int n_out, int dim,
+                    float eps, int write_back, hipStream_t stream) {
+  const dim3 grid(n_out);
+  TIn* xp = static_cast<TIn*>(x);
+  const T* dp = static_cast<const T*>(delta);
+  const T* wp = static_cast<const T*>(weight);
+  T* op = static_cast<T*>(out);
+  const int32_t* rp = static_cast<const int32_t*>(rows);
+  if (dim <= 64) {
+    hipLaunchKernelGGL((rmsnorm_registers_kernel<TIn, T, 1>), grid, dim3(64), 0, stream, xp, dp, wp, op, rp, dim, eps, write_back);
+  } else if (dim <= 256) {
+    hipLaunchKernelGGL((rmsnorm_registers_kernel<TIn, T, 4>), grid, dim3(64), 0, stream, xp, dp, wp, op, rp, dim, eps, write_back);
+  } else if (dim <= 1024) {
+    hipLaunchKernelGGL((rmsnorm_registers_kernel<TIn, T, 4>), grid, dim3(256), 0, stream, xp, dp, wp, op, rp, dim, eps, write_back);
+  } else if (dim <= 4096) {
+    hipLaunchKernelGGL((rmsnorm_registers_kernel<TIn, T, 8>), grid, dim3(512), 0, stream, xp, dp, wp, op, rp, dim, eps, write_back);
+  } else if (dim <= 16384) {
+    hipLaunchKernelGGL((rmsnorm_registers_kernel<TIn, T, 16>), grid, dim3(1024), 0, stream, xp, dp, wp, op, rp, dim, eps, write_back);
+  } else {
+    hipLaunchKernelGGL((rmsnorm_kernel<TIn, T>), grid, dim3(1024), 0, stream, xp, dp, wp, op, rp, dim, eps, write_back);
+  }
+}
+
 }  // namespace
 
 // x: [n_in, dim] (float when x_is_f32, else the storage type); delta: null or
@@ -56,22 +121,13 @@ extern "C" int ms_rmsnorm(void* x, const void* delta, const void* weight, void* 
   MS_REQUIRE(eps > 0.f, "rmsnorm: eps must be positive");
   MS_REQUIRE(!(write_back && rows), "rmsnorm: write_back with gathered rows is not defined");
   MS_REQUIRE(!(write_back && !delta), "rmsnorm: write_back needs a delta");
-  const int threads = dim >= 2048 ? 512 : (dim >= 512 ? 256 : (dim >= 128 ? 128 : 64));
-  const dim3 grid(n_out);
-  const int32_t* r = static_cast<const int32_t*>(rows);
   if (dtype == MS_F32) {
-    hipLaunchKernelGGL((rmsnorm_kernel<float, float>), dim3(grid), dim3(threads), 0, stream, 
-        static_cast<float*>(x), static_cast<const float*>(delta), static_cast<const float*>(weight),
-        static_cast<float*>(out), r, dim, eps, write_back);
+    launch_rmsnorm<float, float>(x, delta, weight, out, rows, n_out, dim, eps, write_back, stream);
   } else if (dtype == MS_BF16) {
     if (x_is_f32) {
-      hipLaunchKernelGGL((rmsnorm_kernel<float, ms::bf16>), dim3(grid), dim3(threads), 0, stream, 
-          static_cast<float*>(x), static_cast<const ms::bf16*>(delta), static_cast<const ms::bf16*>(weight),
-          static_cast<ms::bf16*>(out), r, dim, eps, write_back);
+      launch_rmsnorm<float, ms::bf16>(x, delta, weight, out, rows, n_out, dim, eps, write_back, stream);
     } else {
-      hipLaunchKernelGGL((rmsnorm_kernel<ms::bf16, ms::bf16>), dim3(grid), dim3(threads), 0, stream, 
-          static_cast<ms::bf16*>(x), static_cast<const ms::bf16*>(delta), static_cast<const ms::bf16*>(weight),
-          static_cast<ms::bf16*>(out), r, dim, eps, write_back);
+      launch_rmsnorm<ms::bf16, ms::bf16>(x, delta, weight, out, rows, n_out, dim, eps, write_back, stream);
     }
   } else {
     return ms_fail("rmsnorm: unknown dtype code %d", dtype);

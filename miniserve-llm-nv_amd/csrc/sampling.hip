@@ -217,7 +217,79 @@ __global__ __launch_bounds__(kThreads) void sample_rows_kernel(const float* __re
   if (tid == 0) out[row] = shared_index;
 }
 
+// Greedy choice for large vocabularies in two stages, so that a row is read by many
+// workgroups: stage 1 finds (maximum, its lowest index, any non-finite value) per
+// chunk of the row, stage 2 per row.
+constexpr int kArgmaxThreads = 256;
+
+__global__ __launch_bounds__(kArgmaxThreads) void argmax_chunks_kernel(const float* __restrict__ logits,
+                                                                       float* __restrict__ chunk_max,
+                                                                       int32_t* __restrict__ chunk_index, int vocab,
+                                                                       int chunks) {
+  __shared__ float f_scratch[kArgmaxThreads / ms::kWave];
+  __shared__ int i_scratch[kArgmaxThreads / ms::kWave];
+  __shared__ int shared_index;
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const int per_chunk = (vocab + chunks - 1) / chunks;
+  const int begin = chunk * per_chunk, end = min(begin + per_chunk, vocab);
+  const float* x = logits + static_cast<int64_t>(row) * vocab;
+  float best = -INFINITY;
+  int best_index = vocab, bad = 0;
+  for (int i = begin + threadIdx.x; i < end; i += kArgmaxThreads) {
+    const float v = x[i];
+    if (!(fabsf(v) <= 3.402823466e38f)) bad = 1;
+    if (v > best) {
+      best = v;
+      best_index = i;
+    }
+  }
+  bad = ms::wave_sum_int(bad);
+  if ((threadIdx.x & (ms::kWave - 1)) == 0) i_scratch[threadIdx.x / ms::kWave] = bad;
+  if (threadIdx.x == 0) shared_index = vocab;
+  const float chunk_best = ms::block_max(best, f_scratch);    // has barriers: i_scratch and shared_index are visible
+  if (best == chunk_best) atomicMin(&shared_index, best_index);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int any_bad = 0;
+    for (int w = 0; w < kArgmaxThreads / ms::kWave; ++w) any_bad += i_scratch[w];
+    chunk_max[row * chunks + chunk] = chunk_best;
+    chunk_index[row * chunks + chunk] = any_bad ? -1 : shared_index;
+  }
+}
+
+// One wave per row over at most 64 chunks.
+__global__ void argmax_rows_kernel(const float* __restrict__ chunk_max, const int32_t* __restrict__ chunk_index,
+                                   int32_t* __restrict__ out, int chunks) {
+  const int row = blockIdx.x, lane = threadIdx.x;
+  const bool live = lane < chunks;
+  const float value = live ? chunk_max[row * chunks + lane] : -INFINITY;
+  const int index = live ? chunk_index[row * chunks + lane] : 0x7fffffff;
+  const int bad = ms::wave_sum_int(live && index < 0);
+  const float best = ms::wave_max(value);
+  int candidate = (live && value == best && index >= 0) ? index : 0x7fffffff;
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) candidate = min(candidate, __shfl_xor(candidate, offset, ms::kWave));
+  if (lane == 0) out[row] = bad ? -1 : candidate;
+}
+
 }  // namespace
+
+// Greedy tokens of float logits [rows, vocab] through `chunks` (1..64) partial
+// results per row: chunk_max float [rows, chunks], chunk_index int32 [rows, chunks].
+extern "C" int ms_argmax_rows(const void* logits, void* chunk_max, void* chunk_index, void* out, int rows,
+                              int vocab, int chunks, hipStream_t stream) {
+  MS_REQUIRE(rows > 0 && rows <= 65535 && vocab > 0, "argmax_rows: bad shape %d x %d", rows, vocab);
+  MS_REQUIRE(chunks >= 1 && chunks <= ms::kWave && chunks <= vocab, "argmax_rows: %d chunks", chunks);
+  hipLaunchKernelGGL(argmax_chunks_kernel, dim3(chunks, rows), dim3(kArgmaxThreads), 0, stream,
+                     static_cast<const float*>(logits), static_cast<float*>(chunk_max),
+                     static_cast<int32_t*>(chunk_index), vocab, chunks);
+  MS_CHECK_LAUNCH("argmax_chunks");
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(ms::kWave), 0, stream,
+                     static_cast<const float*>(chunk_max), static_cast<const int32_t*>(chunk_index),
+                     static_cast<int32_t*>(out), chunks);
+  MS_CHECK_LAUNCH("argmax_rows");
+  return 0;
+}
 
 // logits: float [rows, vocab]; temperature, top_p, uniform: float [rows] (null
 // temperature = all rows greedy); top_k: int32 [rows]; out: int32 [rows].

@@ -15,7 +15,7 @@ from typing import Sequence
 import torch
 
 from ..cache.manager import StepReservation
-from ..parts.base import GroupStepView, StepContext
+from ..parts.base import GroupStepView, QueryTiles, StepContext
 
 
 @dataclass(frozen=True)
@@ -49,6 +49,11 @@ def build_step_context(
 
     if len(entries) != len(reservation.sequences):
         raise ValueError("entries and reservation disagree.")
+    # Sequences that bring one token are laid out first; the logits keep the order of
+    # the entries as given.
+    layout = sorted(range(len(entries)), key=lambda i: len(entries[i].token_ids) != 1)
+    decode_prefix = sum(1 for entry in entries if len(entry.token_ids) == 1)
+    base_of_entry = [0] * len(entries)
     token_ids: list[int] = []
     positions: list[int] = []
     seq_of_token: list[int] = []
@@ -62,12 +67,23 @@ def build_step_context(
     slot_mappings: list[list[int]] = [[] for _ in range(num_groups)]
     widest = [1] * num_groups
 
-    for index, (entry, meta) in enumerate(zip(entries, reservation.sequences)):
+    tile_seq: list[int] = []
+    tile_token: list[int] = []
+    tile_length: list[int] = []
+    metas_in_layout = [reservation.sequences[i] for i in layout]
+    for index, original in enumerate(layout):
+        entry, meta = entries[original], reservation.sequences[original]
         if entry.request_id != meta.request_id or len(entry.token_ids) != meta.after - meta.before:
             raise ValueError(f"entry {entry.request_id!r} does not match its reservation.")
         if any(token >= vocab_size for token in entry.token_ids):
             raise ValueError(f"entry {entry.request_id!r}: a token id is outside the vocabulary of {vocab_size}.")
         base = len(token_ids)
+        base_of_entry[original] = base
+        if index >= decode_prefix:
+            for start in range(0, len(entry.token_ids), 16):
+                tile_seq.append(index)
+                tile_token.append(base + start)
+                tile_length.append(min(16, len(entry.token_ids) - start))
         token_ids.extend(entry.token_ids)
         positions.extend(range(meta.before, meta.after))
         seq_of_token.extend([index] * len(entry.token_ids))
@@ -76,7 +92,6 @@ def build_step_context(
         state_slots.append(meta.state_slot)
         query_lens.append(len(entry.token_ids))
         first_positions.append(meta.before)
-        logit_rows.extend(base + place for place in entry.want)
         for group in range(num_groups):
             table = meta.block_tables[group]
             slots = meta.slot_mappings[group]
@@ -87,6 +102,9 @@ def build_step_context(
                     raise RuntimeError(f"request {entry.request_id!r}: slot {slot} disagrees with its block table.")
             slot_mappings[group].extend(slots)
             widest[group] = max(widest[group], len(table))
+
+    for original, entry in enumerate(entries):
+        logit_rows.extend(base_of_entry[original] + place for place in entry.want)
 
     n, s = len(token_ids), len(entries)
     packed: list[int] = []
@@ -103,10 +121,13 @@ def build_step_context(
     put("context_lens", context_lens)
     put("state_slots", state_slots)
     put("logit_rows", logit_rows)
+    put("tile_seq", tile_seq)
+    put("tile_token", tile_token)
+    put("tile_length", tile_length)
     for group in range(num_groups):
         put(f"slots{group}", slot_mappings[group])
         flat: list[int] = []
-        for meta in reservation.sequences:
+        for meta in metas_in_layout:
             table = meta.block_tables[group]
             # a page that was given back is never read; 0 keeps the entry inside the pool
             flat.extend(page if page >= 0 else 0 for page in table)
@@ -141,6 +162,8 @@ def build_step_context(
         query_start_host=query_start,
         state_slots_host=state_slots,
         first_positions_host=first_positions,
+        decode_prefix=decode_prefix,
+        tiles=QueryTiles(len(tile_seq), view("tile_seq"), view("tile_token"), view("tile_length")) if tile_seq else None,
     )
     rows = view("logit_rows") if logit_rows else None
     return ctx, rows

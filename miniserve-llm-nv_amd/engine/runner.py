@@ -76,6 +76,7 @@ class DecodeGraph:
             query_start_host=list(range(batch + 1)),
             state_slots_host=[0] * batch,
             first_positions_host=[0] * batch,
+            decode_prefix=batch,
         )
         self.rows = view("logit_rows")
         self.graph: torch.cuda.CUDAGraph | None = None

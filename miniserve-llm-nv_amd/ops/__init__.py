@@ -16,6 +16,7 @@ __all__ = [
     "embedding_gather",
     "library_path",
     "linear",
+    "linear_silu_mul",
     "load",
     "qk_norm_rope_append",
     "residual_add",
@@ -188,9 +189,6 @@ def _value_pool_shape(key_pool: torch.Tensor) -> tuple[int, ...]:
 # (the chip has 256), so that short batches still fill it.
 _DECODE_TARGET_WORKGROUPS = 512
 _DECODE_MAX_SPLITS = 64
-# Above this many query tokens per sequence the rows are better served as tiles of
-# queries than one by one.
-_DECODE_MAX_QUERY_LEN = 1
 
 
 def decode_splits(num_tokens: int, num_kv_heads: int, group: int, max_context: int) -> int:
@@ -213,7 +211,8 @@ def attention(
     positions: torch.Tensor,
     scale: float,
     window: int | None = None,
-    max_query_len: int | None = None,
+    decode_prefix: int = 0,
+    tiles=None,
     max_context: int | None = None,
     splits: int | None = None,
 ) -> torch.Tensor:
@@ -229,9 +228,12 @@ def attention(
 
     float32 runs the generic kernel, whose result for a position is bit-identical
     for any batch.  bfloat16 runs the matrix-core kernels where they take the
-    geometry: ``max_query_len`` (the longest run of tokens of one sequence in this
-    batch; None = unknown) and ``max_context`` (the largest position + 1) choose
-    between them and size the key split; ``splits`` overrides it."""
+    geometry: the first ``decode_prefix`` tokens are single tokens of their
+    sequences and go to the key-split kernel (``max_context``, the largest
+    position + 1, sizes the split; ``splits`` overrides it); the other tokens go,
+    cut into ``tiles`` (a ``QueryTiles``: at most 16 consecutive tokens of one
+    sequence each), to the tiled kernel.  Without ``tiles`` and ``decode_prefix``
+    the generic kernel serves every token."""
 
     _check(q, "q")
     if q.ndim != 3 or q.shape[0] == 0:
@@ -252,36 +254,72 @@ def attention(
     window = 0 if window is None else int(window)
     if window < 0:
         raise KernelError("attention: window must be positive or None.")
+    if not 0 <= decode_prefix <= n:
+        raise KernelError("attention: decode_prefix lies outside the batch.")
     out = torch.empty_like(q)
     lib = load()
-    if (
-        q.dtype == torch.bfloat16
-        and max_query_len is not None
-        and max_query_len <= _DECODE_MAX_QUERY_LEN
-        and lib.ms_attention_decode_supported(head_dim, block_size)
-    ):
-        if splits is None:
-            splits = decode_splits(n, kv_heads, heads // kv_heads, max_context or block_table.shape[1] * block_size)
-        partial_o = partial_ml = None
-        if splits > 1:
-            partial_o = torch.empty((n, heads, splits, head_dim), dtype=torch.float32, device=q.device)
-            partial_ml = torch.empty((n, heads, splits, 2), dtype=torch.float32, device=q.device)
-        call("ms_attention_decode", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(seq_of_token),
-             _ptr(positions), _ptr(out), _ptr(partial_o), _ptr(partial_ml), n, heads, kv_heads, head_dim, block_size,
-             block_table.shape[1], float(scale), window, int(splits), _stream())
+    max_blocks = block_table.shape[1]
+    covered = decode_prefix == n or (tiles is not None and tiles.count > 0)
+    if q.dtype == torch.bfloat16 and covered and lib.ms_attention_decode_supported(head_dim, block_size):
+        tiled = lib.ms_attention_prefill_supported(head_dim, block_size)
+        single = decode_prefix if tiled else n          # without the tiled kernel every token is served as a single one
+        if single > 0:
+            if splits is None:
+                splits = decode_splits(single, kv_heads, heads // kv_heads, max_context or max_blocks * block_size)
+            partial_o = partial_ml = None
+            if splits > 1:
+                partial_o = torch.empty((single, heads, splits, head_dim), dtype=torch.float32, device=q.device)
+                partial_ml = torch.empty((single, heads, splits, 2), dtype=torch.float32, device=q.device)
+            call("ms_attention_decode", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table),
+                 _ptr(seq_of_token), _ptr(positions), _ptr(out), _ptr(partial_o), _ptr(partial_ml), single, heads,
+                 kv_heads, head_dim, block_size, max_blocks, float(scale), window, int(splits), _stream())
+        if tiled and decode_prefix < n:
+            for name in ("seq", "token", "length"):
+                _check(getattr(tiles, name), f"tiles.{name}", dtype=torch.int32, shape=(tiles.count,))
+            call("ms_attention_prefill", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(positions),
+                 _ptr(tiles.seq), _ptr(tiles.token), _ptr(tiles.length), _ptr(out), tiles.count, heads, kv_heads,
+                 head_dim, block_size, max_blocks, float(scale), window, _stream())
         return out
     call("ms_attention_generic", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(seq_of_token),
-         _ptr(positions), _ptr(out), n, heads, kv_heads, head_dim, block_size, block_table.shape[1], float(scale),
+         _ptr(positions), _ptr(out), n, heads, kv_heads, head_dim, block_size, max_blocks, float(scale),
          window, _code(q.dtype), _stream())
     return out
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, *, accumulate_into: torch.Tensor | None = None) -> torch.Tensor:
+_EPILOGUE_BF16, _EPILOGUE_F32, _EPILOGUE_ADD_F32, _EPILOGUE_SILU_MUL = 0, 1, 2, 3
+# Rows up to which this library's product is used in bfloat16; the kernel takes up
+# to 64, but from 17 rows on the library product is faster (measured on MI355X at
+# the layer sizes of Qwen3-0.6B and 8B), so it serves those.
+SKINNY_MAX_ROWS = 16
+
+
+def _use_skinny(m: int, n: int, k: int, epilogue: int) -> bool:
+    return m <= SKINNY_MAX_ROWS and bool(load().ms_gemm_skinny_supported(m, n, k, epilogue))
+
+
+def _skinny(x: torch.Tensor, weight: torch.Tensor, epilogue: int, out: torch.Tensor) -> None:
+    m, k = x.shape
+    n = weight.shape[0]
+    bf16_out = out if out.dtype == torch.bfloat16 else None
+    f32_out = out if out.dtype == torch.float32 else None
+    call("ms_gemm_skinny", _ptr(x), _ptr(weight), _ptr(bf16_out), _ptr(f32_out), m, n, k, epilogue, _stream())
+
+
+def linear(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    *,
+    accumulate_into: torch.Tensor | None = None,
+    out_float32: bool = False,
+) -> torch.Tensor:
     """``x [M, K] @ weight [N, K]^T``.
 
     float32: this library's FMA kernel (true 32-bit; row results do not depend on
-    M); ``accumulate_into`` (float32 ``[M, N]``) receives ``+=``.  bfloat16: the
-    library matrix product (hipBLASLt through torch) with 32-bit accumulation."""
+    M).  bfloat16 with at most ``SKINNY_MAX_ROWS`` rows: this library's matrix-core
+    kernel that streams the weights once; more rows: the library matrix product
+    (hipBLASLt through torch), both with 32-bit accumulation.  ``accumulate_into`` (float32
+    ``[M, N]``) receives ``+=`` and is returned; ``out_float32`` returns the
+    32-bit sums without a rounding to bfloat16 in between."""
 
     _check(x, "x")
     _check(weight, "weight", dtype=x.dtype)
@@ -289,20 +327,43 @@ def linear(x: torch.Tensor, weight: torch.Tensor, *, accumulate_into: torch.Tens
         raise KernelError(f"linear: x {tuple(x.shape)} does not match weight {tuple(weight.shape)}.")
     m, k = x.shape
     n = weight.shape[0]
+    if accumulate_into is not None:
+        _check(accumulate_into, "accumulate_into", dtype=torch.float32, shape=(m, n))
     if x.dtype == torch.float32:
-        if accumulate_into is not None:
-            _check(accumulate_into, "accumulate_into", dtype=torch.float32, shape=(m, n))
-            out = accumulate_into
-        else:
-            out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+        out = accumulate_into if accumulate_into is not None else torch.empty((m, n), dtype=torch.float32, device=x.device)
         call("ms_gemm_f32", _ptr(x), _ptr(weight), _ptr(out), m, n, k, int(accumulate_into is not None), _stream())
         return out
     _code(x.dtype)
+    if _use_skinny(m, n, k, _EPILOGUE_BF16):
+        if accumulate_into is not None:
+            _skinny(x, weight, _EPILOGUE_ADD_F32, accumulate_into)
+            return accumulate_into
+        out = torch.empty((m, n), dtype=torch.float32 if out_float32 else torch.bfloat16, device=x.device)
+        _skinny(x, weight, _EPILOGUE_F32 if out_float32 else _EPILOGUE_BF16, out)
+        return out
     out = torch.mm(x, weight.t())
     if accumulate_into is not None:
         residual_add(accumulate_into, out)
         return accumulate_into
-    return out
+    return out.float() if out_float32 else out
+
+
+def linear_silu_mul(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``silu(x Wg^T) * (x Wu^T)`` for ``weight [2 I, K]`` = gate rows, then up rows ->
+    ``[M, I]``.  bfloat16 with at most ``SKINNY_MAX_ROWS`` rows: one kernel, the
+    activation in the product's epilogue; otherwise the product and :func:`silu_mul`."""
+
+    _check(x, "x")
+    _check(weight, "weight", dtype=x.dtype)
+    if x.ndim != 2 or weight.ndim != 2 or x.shape[1] != weight.shape[1] or x.shape[0] == 0 or weight.shape[0] % 2:
+        raise KernelError(f"linear_silu_mul: x {tuple(x.shape)} does not match weight {tuple(weight.shape)}.")
+    m, k = x.shape
+    n = weight.shape[0]
+    if x.dtype == torch.bfloat16 and _use_skinny(m, n, k, _EPILOGUE_SILU_MUL):
+        out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
+        _skinny(x, weight, _EPILOGUE_SILU_MUL, out)
+        return out
+    return silu_mul(linear(x, weight))
 
 
 def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
@@ -345,6 +406,14 @@ def sample_rows(
         if top_p is not None:
             _check(top_p, "top_p", dtype=torch.float32, shape=(rows,))
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    if temperature is None and vocab >= 4096:
+        # all rows greedy: two stages, so that many workgroups share the read of a row
+        chunks = 64
+        chunk_max = torch.empty((rows, chunks), dtype=torch.float32, device=logits.device)
+        chunk_index = torch.empty((rows, chunks), dtype=torch.int32, device=logits.device)
+        call("ms_argmax_rows", _ptr(logits), _ptr(chunk_max), _ptr(chunk_index), _ptr(out), rows, vocab, chunks,
+             _stream())
+        return out
     call("ms_sample_rows", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(out),
          rows, vocab, _stream())
     return out

@@ -114,7 +114,8 @@ class Attention(Part):
             positions=ctx.positions,
             scale=self.scale,
             window=self.window,
-            max_query_len=ctx.max_query_len,
+            decode_prefix=ctx.decode_prefix,
+            tiles=ctx.tiles,
             max_context=ctx.max_context_len,
         )
         return ops.linear(attended.reshape(n, self.num_heads * self.head_dim), self.w_o)

@@ -106,9 +106,22 @@ class GroupStepView:
 
 
 @dataclass
+class QueryTiles:
+    """The tokens after the single-token prefix of a batch, cut into tiles of at most
+    16 consecutive tokens of one sequence (what the tiled attention kernel walks)."""
+
+    count: int
+    seq: torch.Tensor       # int32 [count]: the tile's sequence (row of the block tables)
+    token: torch.Tensor     # int32 [count]: index of the tile's first token in the batch
+    length: torch.Tensor    # int32 [count]: 1..16
+
+
+@dataclass
 class StepContext:
     """A flat ragged batch: ``N`` tokens of ``S`` sequences, each sequence's tokens
-    contiguous and at consecutive absolute positions."""
+    contiguous and at consecutive absolute positions.  Sequences that bring one
+    token come first (``decode_prefix`` of them), so that kernels made for single
+    tokens and kernels made for runs of tokens can each take their share."""
 
     num_tokens: int
     num_seqs: int
@@ -125,6 +138,8 @@ class StepContext:
     query_start_host: list[int] = field(default_factory=list)
     state_slots_host: list[int] = field(default_factory=list)
     first_positions_host: list[int] = field(default_factory=list)
+    decode_prefix: int = 0
+    tiles: QueryTiles | None = None
 
     @property
     def max_query_len(self) -> int:

@@ -54,7 +54,7 @@ class LinearHead(Part):
         self.weight = tensors[self.tied_to] if self.tied_to else tensors[self.weight_name]
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.linear(x, self.weight).float()
+        return ops.linear(x, self.weight, out_float32=True)
 
 
 register_part("embedding", "token_embedding", TokenEmbedding)

@@ -11,7 +11,8 @@ from .. import ops
 from ..config.model_spec import PartSpec
 from .base import Part, StepContext, WeightSpec, register_part, require_params
 
-_ACTIVATIONS = {"silu": ops.silu_mul}
+# activation name -> (gated activation of a packed [N, 2 I] row, the same fused with the product)
+_ACTIVATIONS = {"silu": (ops.silu_mul, ops.linear_silu_mul)}
 
 
 class GatedMLP(Part):
@@ -22,7 +23,7 @@ class GatedMLP(Part):
         activation = params["activation"]
         if activation not in _ACTIVATIONS:
             raise ValueError(f"gated_mlp knows the activations {sorted(_ACTIVATIONS)}, not {activation!r}.")
-        self._gated_activation = _ACTIVATIONS[activation]
+        self._gated_activation, self._gated_product = _ACTIVATIONS[activation]
         self.dtype = dtype
         self.prefix = spec.prefix
         self.w_gate_up: torch.Tensor | None = None
@@ -44,7 +45,7 @@ class GatedMLP(Part):
         self.w_down = tensors[self.prefix + "down_proj.weight"]
 
     def forward(self, x: torch.Tensor, ctx: StepContext | None = None) -> torch.Tensor:
-        return ops.linear(self._gated_activation(ops.linear(x, self.w_gate_up)), self.w_down)
+        return ops.linear(self._gated_product(x, self.w_gate_up), self.w_down)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

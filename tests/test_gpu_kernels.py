@@ -29,6 +29,12 @@ def tolerance(dtype, f32=2e-5, bf16=4e-3):
     return f32 if dtype == torch.float32 else bf16
 
 
+# Attention in bfloat16: the reference allows 8e-3 for float16 (11 significant bits);
+# bfloat16 carries 8, and the weights P are rounded to it before the second product,
+# as in the reference's chunk form.  Twice the float16 figure.
+ATTENTION_BF16 = 1.6e-2
+
+
 @pytest.fixture(scope="module")
 def ops():
     from miniserve_amd import ops as module
@@ -240,11 +246,38 @@ def attention_reference(case, scale, window=None):
     return torch.cat(outs)
 
 
+def query_tiles(case, first_sequence):
+    """Tiles of at most 16 consecutive tokens for the sequences from ``first_sequence`` on."""
+
+    from miniserve_amd.parts import QueryTiles
+
+    seqs, tokens, lengths, base = [], [], [], 0
+    for index, qlen in enumerate(case["query_lens"]):
+        if index >= first_sequence:
+            for start in range(0, qlen, 16):
+                seqs.append(index)
+                tokens.append(base + start)
+                lengths.append(min(16, qlen - start))
+        base += qlen
+    if not seqs:
+        return None
+    device = case["q"].device
+    as_tensor = lambda values: torch.tensor(values, dtype=torch.int32, device=device)
+    return QueryTiles(len(seqs), as_tensor(seqs), as_tensor(tokens), as_tensor(lengths))
+
+
 def run_attention(ops, case, scale, window=None, splits=None):
+    """As the engine calls it: sequences that bring one token stand first and are
+    served as single tokens, the others in tiles."""
+
+    lens = case["query_lens"]
+    prefix = 0
+    while prefix < len(lens) and lens[prefix] == 1:
+        prefix += 1
     return ops.attention(case["q"], case["key_pool"], case["value_pool"], block_table=case["block_table"],
                          seq_of_token=case["seq_of_token"], positions=case["positions"], scale=scale, window=window,
-                         max_query_len=max(case["query_lens"]), max_context=int(case["positions"].max()) + 1,
-                         splits=splits)
+                         decode_prefix=prefix, tiles=query_tiles(case, prefix),
+                         max_context=int(case["positions"].max()) + 1, splits=splits)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -255,7 +288,7 @@ def test_paged_decode_workloads_of_the_reference(ops, dtype, batch, context):
     case = paged_case([context] * batch, 16, 8, 128, 16, dtype, seed=8800 + 100 * batch + context)
     out = run_attention(ops, case, 128**-0.5)
     expected = attention_reference(case, 128**-0.5)
-    tol = tolerance(dtype, 2e-4, 8e-3)
+    tol = tolerance(dtype, 2e-4, ATTENTION_BF16)
     torch.testing.assert_close(out.cpu().double(), expected, atol=tol, rtol=tol)
 
 
@@ -267,7 +300,7 @@ def test_attention_sizes_chunks_and_decode_rows_in_one_batch(ops, dtype, heads, 
     case = paged_case(contexts, heads, kv_heads, dim, block, dtype, query_lens=query_lens, seed=dim + block)
     out = run_attention(ops, case, dim**-0.5)
     expected = attention_reference(case, dim**-0.5)
-    tol = tolerance(dtype, 2e-4, 8e-3)
+    tol = tolerance(dtype, 2e-4, ATTENTION_BF16)
     torch.testing.assert_close(out.cpu().double(), expected, atol=tol, rtol=tol)
 
 
@@ -292,7 +325,7 @@ def test_one_far_key_among_hundreds_stands_out(ops, dtype):
         out = run_attention(ops, case, 64**-0.5)
         expected = attention_reference(case, 64**-0.5)
         assert float(expected.min()) > 10.0                                     # the far key dominates
-        tol = tolerance(dtype, 2e-4, 8e-3)
+        tol = tolerance(dtype, 2e-4, ATTENTION_BF16)
         torch.testing.assert_close(out.cpu().double(), expected, atol=tol * 100, rtol=tol)
 
 
@@ -314,7 +347,7 @@ def test_window_edges(ops, dtype, window):
                 case["value_pool"][page, :, :, position % 8] = value
     out = run_attention(ops, case, 32**-0.5, window=window)
     expected = attention_reference(case, 32**-0.5, window=window)
-    tol = tolerance(dtype, 2e-4, 8e-3)
+    tol = tolerance(dtype, 2e-4, ATTENTION_BF16)
     torch.testing.assert_close(out.cpu().double(), expected, atol=tol * 50, rtol=tol)
 
 
@@ -330,13 +363,39 @@ def test_decode_kernel_sizes_splits_and_windows(ops, heads, kv_heads, dim, block
     expected = attention_reference(case, dim**-0.5)
     for splits in (1, 2, 5, 16, 64, None):
         out = run_attention(ops, case, dim**-0.5, splits=splits)
-        torch.testing.assert_close(out.cpu().double(), expected, atol=8e-3, rtol=8e-3, msg=lambda m: f"splits {splits}: {m}")
+        torch.testing.assert_close(out.cpu().double(), expected, atol=ATTENTION_BF16, rtol=ATTENTION_BF16, msg=lambda m: f"splits {splits}: {m}")
     for window in (1, 16, 17, 100, 1000):
         expected = attention_reference(case, dim**-0.5, window=window)
         for splits in (1, 3, None):
             out = run_attention(ops, case, dim**-0.5, window=window, splits=splits)
-            torch.testing.assert_close(out.cpu().double(), expected, atol=8e-3, rtol=8e-3,
+            torch.testing.assert_close(out.cpu().double(), expected, atol=ATTENTION_BF16, rtol=ATTENTION_BF16,
                                        msg=lambda m: f"window {window} splits {splits}: {m}")
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim,block", [(16, 8, 128, 16), (8, 1, 64, 16), (4, 4, 32, 32), (3, 1, 16, 16), (6, 2, 80, 48), (32, 8, 128, 64), (5, 1, 112, 16)])
+def test_tiled_kernel_sizes_portions_and_windows(ops, heads, kv_heads, dim, block):
+    """The matrix-core kernel for runs of query tokens: whole prompts, portions that
+    start and end off the tile and page grid, single tokens after the prefix, groups
+    of 1 to 8 heads, head sizes in steps of 16, windows."""
+
+    contexts = [1, 1, 130, 16, 17, 64, 700, 33, 300]
+    query_lens = [1, 1, 130, 16, 2, 31, 150, 1, 300]          # two single tokens first, one more later
+    case = paged_case(contexts, heads, kv_heads, dim, block, torch.bfloat16, query_lens=query_lens, seed=dim + heads)
+    assert ops.load().ms_attention_prefill_supported(dim, block)
+    out = run_attention(ops, case, dim**-0.5)
+    torch.testing.assert_close(out.cpu().double(), attention_reference(case, dim**-0.5), atol=ATTENTION_BF16, rtol=ATTENTION_BF16)
+    for window in (1, 15, 16, 17, 100):
+        out = run_attention(ops, case, dim**-0.5, window=window)
+        expected = attention_reference(case, dim**-0.5, window=window)
+        torch.testing.assert_close(out.cpu().double(), expected, atol=ATTENTION_BF16, rtol=ATTENTION_BF16, msg=lambda m: f"window {window}: {m}")
+
+
+def test_tiled_kernel_ignores_stale_values(ops):
+    case = paged_case([37, 70], 8, 2, 64, 16, torch.bfloat16, query_lens=[20, 70], seed=4)   # unused slots hold NaN
+    assert torch.isnan(case["value_pool"]).any()
+    out = run_attention(ops, case, 0.125)
+    assert torch.isfinite(out).all()
+    torch.testing.assert_close(out.cpu().double(), attention_reference(case, 0.125), atol=ATTENTION_BF16, rtol=ATTENTION_BF16)
 
 
 def test_decode_kernel_ignores_stale_values(ops):
@@ -347,7 +406,7 @@ def test_decode_kernel_ignores_stale_values(ops):
     assert torch.isnan(case["value_pool"]).any() and torch.isnan(case["key_pool"]).any()
     out = run_attention(ops, case, 0.125)
     assert torch.isfinite(out).all()
-    torch.testing.assert_close(out.cpu().double(), attention_reference(case, 0.125), atol=8e-3, rtol=8e-3)
+    torch.testing.assert_close(out.cpu().double(), attention_reference(case, 0.125), atol=ATTENTION_BF16, rtol=ATTENTION_BF16)
 
 
 def test_decode_kernel_is_refused_for_other_geometries(ops):
@@ -355,9 +414,14 @@ def test_decode_kernel_is_refused_for_other_geometries(ops):
     assert not lib.ms_attention_decode_supported(128, 8)          # pages of 8 keys
     assert not lib.ms_attention_decode_supported(24, 16)          # head size off the 16 grid
     assert not lib.ms_attention_decode_supported(272, 16)
+    assert not lib.ms_attention_prefill_supported(144, 16)        # large heads are served token by token
+    assert lib.ms_attention_decode_supported(144, 16)
+    big = paged_case([40, 3], 2, 1, 144, 16, torch.bfloat16, query_lens=[40, 1], seed=3)
+    torch.testing.assert_close(run_attention(ops, big, 144**-0.5).cpu().double(), attention_reference(big, 144**-0.5),
+                               atol=ATTENTION_BF16, rtol=ATTENTION_BF16)
     case = paged_case([30, 9], 8, 1, 32, 8, torch.bfloat16, seed=2)
     out = run_attention(ops, case, 32**-0.5)                       # falls to the generic kernel
-    torch.testing.assert_close(out.cpu().double(), attention_reference(case, 32**-0.5), atol=8e-3, rtol=8e-3)
+    torch.testing.assert_close(out.cpu().double(), attention_reference(case, 32**-0.5), atol=ATTENTION_BF16, rtol=ATTENTION_BF16)
 
 
 def test_attention_is_bit_identical_across_batches_in_float32(ops):
@@ -411,6 +475,47 @@ def test_linear_bfloat16_and_fused_projection_rows(ops):
     assert torch.equal(fused32[:, 256:288], ops.linear(x32, parts[1].float()))
 
 
+@pytest.mark.parametrize("m", [1, 8, 15, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,k", [(16, 32), (509, 96), (100, 200), (4096, 1024), (1024, 3072), (40000, 64)])
+def test_skinny_product_for_few_rows(ops, m, n, k, monkeypatch):
+    """The matrix-core product that decoding uses (at most 64 rows), with its four
+    epilogues, against float64; sizes off the tile grid in every dimension."""
+
+    assert ops.load().ms_gemm_skinny_supported(m, n, k, 0)
+    monkeypatch.setattr(ops, "SKINNY_MAX_ROWS", 64)                        # the kernel itself, beyond the rows it serves
+    x = rand(m, k, seed=m + k, dtype=torch.bfloat16)
+    w = rand(n, k, seed=n, dtype=torch.bfloat16, scale=0.05)
+    exact = x.cpu().double() @ w.cpu().double().T
+    scale = float(exact.abs().max())
+    out = ops.linear(x, w)
+    assert out.dtype == torch.bfloat16
+    torch.testing.assert_close(out.cpu().double(), exact, atol=scale * 2**-8, rtol=2**-8)
+    wide = ops.linear(x, w, out_float32=True)
+    assert wide.dtype == torch.float32
+    torch.testing.assert_close(wide.cpu().double(), exact, atol=scale * 1e-5, rtol=1e-5)
+    assert torch.equal(wide.to(torch.bfloat16), out)                       # one rounding, at the end
+    target = rand(m, n, seed=3)
+    before = target.clone()
+    ops.linear(x, w, accumulate_into=target)
+    torch.testing.assert_close(target, before + wide, atol=1e-6, rtol=1e-6)
+    # a row's result is the same to the bit whatever rows stand beside it
+    alone = ops.linear(x[m // 2 : m // 2 + 1].contiguous(), w, out_float32=True)
+    assert torch.equal(alone[0], wide[m // 2])
+    if n % 2 == 0:
+        fused = ops.linear_silu_mul(x, w)
+        assert torch.equal(fused, ops.silu_mul(out))                        # the same as product, rounding, activation
+
+
+def test_product_beyond_64_rows_uses_the_library(ops):
+    assert not ops.load().ms_gemm_skinny_supported(65, 128, 64, 0)
+    assert not ops.load().ms_gemm_skinny_supported(8, 128, 60, 0)          # k off the 8 grid
+    x, w = rand(65, 60, seed=1, dtype=torch.bfloat16), rand(33, 60, seed=2, dtype=torch.bfloat16)
+    exact = x.cpu().double() @ w.cpu().double().T
+    torch.testing.assert_close(ops.linear(x, w).cpu().double(), exact, atol=0.1, rtol=2**-7)
+    torch.testing.assert_close(ops.linear(x[:8].contiguous(), w, out_float32=True).cpu().double(), exact[:8], atol=0.1, rtol=2**-7)
+    torch.testing.assert_close(ops.linear_silu_mul(x, w[:32].contiguous()), ops.silu_mul(ops.linear(x, w[:32].contiguous())))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rows,inter", [(1, 1), (3, 63), (5, 200), (64, 3072), (2, 1031)])
 def test_silu_mul(ops, dtype, rows, inter):
@@ -443,6 +548,20 @@ def test_greedy_is_argmax_with_the_lowest_index_among_equals(ops):
     expected[2], expected[5] = 30, 0
     assert out.cpu().tolist() == expected.tolist()
     assert ops.sample_rows(torch.tensor([[0.1, 4.0, 3.0]], device=DEVICE)).tolist() == [1]     # test_sampling.py:38-41
+
+
+def test_greedy_over_a_large_vocabulary(ops):
+    """From 4096 tokens on the greedy choice runs in two stages over chunks of the row."""
+
+    for vocab in (4096, 4097, 151936):
+        logits = rand(5, vocab, seed=vocab)
+        logits[1, vocab - 1] = logits[1, 17] = 60.0                      # equal maxima in the first and the last chunk
+        logits[2, vocab // 2] = 70.0
+        logits[3, :] = -3.5
+        logits[4, vocab - 2] = float("inf")
+        expected = torch.argmax(logits, dim=-1).cpu().tolist()
+        expected[1], expected[3], expected[4] = 17, 0, -1
+        assert ops.sample_rows(logits).cpu().tolist() == expected
 
 
 def test_non_finite_logits_are_reported(ops):
