@@ -9,6 +9,11 @@
 #define MS_WAVES_PER_EU(lo, hi) __attribute__((amdgpu_waves_per_eu(lo, hi)))
 #endif
 
+#ifndef MS_FAST_EXP2
+#define MS_FAST_EXP2(x) __builtin_amdgcn_exp2f(x)
+#define MS_UNIFORM(v) __builtin_amdgcn_readfirstlane(v)
+#endif
+
 namespace ms {
 
 constexpr int kWave = 64;
@@ -51,6 +56,14 @@ template <typename T>
 __device__ __forceinline__ float round_to(float v) {
   return to_float(from_float<T>(v));
 }
+
+// 2^x by the hardware instruction alone (no handling of results below the smallest
+// normal number, which are zero weights anyway).
+__device__ __forceinline__ float fast_exp2(float x) { return MS_FAST_EXP2(x); }
+
+// A value that is the same in every lane of the wave, moved to a scalar register so
+// that what is computed from it is scalar work and branches on it are scalar branches.
+__device__ __forceinline__ int uniform(int v) { return MS_UNIFORM(v); }
 
 // Butterfly reductions over the 64 lanes of a wave; every lane gets the result
 // and the order of additions is fixed, so a row's result never depends on what

@@ -18,6 +18,9 @@ from ..cache.manager import StepReservation
 from ..parts.base import GroupStepView, QueryTiles, StepContext
 
 
+QUERY_TILE = 64     # tokens of one sequence that one workgroup of the tiled attention kernel serves
+
+
 @dataclass(frozen=True)
 class StepEntry:
     """A request's next tokens and the places among them whose logits are wanted."""
@@ -80,10 +83,10 @@ def build_step_context(
         base = len(token_ids)
         base_of_entry[original] = base
         if index >= decode_prefix:
-            for start in range(0, len(entry.token_ids), 16):
+            for start in range(0, len(entry.token_ids), QUERY_TILE):
                 tile_seq.append(index)
                 tile_token.append(base + start)
-                tile_length.append(min(16, len(entry.token_ids) - start))
+                tile_length.append(min(QUERY_TILE, len(entry.token_ids) - start))
         token_ids.extend(entry.token_ids)
         positions.extend(range(meta.before, meta.after))
         seq_of_token.extend([index] * len(entry.token_ids))

@@ -126,6 +126,7 @@ class DecodeGraph:
             # running the same step twice writes the same cache slots twice.
             model.forward(self.ctx, views, self.rows)
             torch.cuda.synchronize(self.runner.device)
+            self.ctx.scratch.clear()        # what the step shares between layers is made again inside the recording
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self.runner._graph_pool):
                 self.logits = model.forward(self.ctx, views, self.rows)

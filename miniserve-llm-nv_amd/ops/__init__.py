@@ -21,6 +21,7 @@ __all__ = [
     "qk_norm_rope_append",
     "residual_add",
     "rmsnorm",
+    "rope_table",
     "sample_rows",
     "silu_mul",
 ]
@@ -118,6 +119,21 @@ def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
     call("ms_residual_add", _ptr(h), _ptr(delta), h.shape[0], h.shape[1], _code(delta.dtype), _stream())
 
 
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """cos and sin of ``float(position) * inv_freq`` in float32, ``[N, half]`` each:
+    made once per step, read by every layer."""
+
+    _check(positions, "positions", dtype=torch.int32)
+    _check(inv_freq, "inv_freq", dtype=torch.float32)
+    if positions.ndim != 1 or inv_freq.ndim != 1 or positions.numel() == 0 or inv_freq.numel() == 0:
+        raise KernelError("rope_table takes positions [N>0] and inv_freq [half>0].")
+    shape = (positions.numel(), inv_freq.numel())
+    cos = torch.empty(shape, dtype=torch.float32, device=positions.device)
+    sin = torch.empty(shape, dtype=torch.float32, device=positions.device)
+    call("ms_rope_table", _ptr(positions), _ptr(inv_freq), _ptr(cos), _ptr(sin), shape[0], shape[1], _stream())
+    return cos, sin
+
+
 def qk_norm_rope_append(
     packed: torch.Tensor,
     *,
@@ -127,8 +143,7 @@ def qk_norm_rope_append(
     q_weight: torch.Tensor | None,
     k_weight: torch.Tensor | None,
     eps: float,
-    inv_freq: torch.Tensor | None,
-    positions: torch.Tensor | None,
+    rope: tuple[torch.Tensor, torch.Tensor] | None,
     slot_mapping: torch.Tensor | None = None,
     key_pool: torch.Tensor | None = None,
     value_pool: torch.Tensor | None = None,
@@ -136,7 +151,8 @@ def qk_norm_rope_append(
     """Per-head norm of q and k, rotation, and the cache write, in one kernel.
 
     ``packed [N, (num_q_heads + 2*num_kv_heads) * head_dim]`` holds q heads, then
-    k heads, then v heads.  Returns q ``[N, num_q_heads, head_dim]`` (None when
+    k heads, then v heads.  ``rope``: the (cos, sin) tables of :func:`rope_table` for
+    these N tokens, or None for no rotation.  Returns q ``[N, num_q_heads, head_dim]`` (None when
     there are no q heads); with ``slot = page * block_size + offset`` from
     ``slot_mapping`` (int32), k goes to ``key_pool[page, kv_head, offset, :]`` and v,
     transposed, to ``value_pool[page, kv_head, :, offset]``."""
@@ -152,12 +168,11 @@ def qk_norm_rope_append(
     for name, weight in (("q_weight", q_weight), ("k_weight", k_weight)):
         if weight is not None:
             _check(weight, name, dtype=dtype, shape=(head_dim,))
-    if inv_freq is not None:
-        _check(inv_freq, "inv_freq", dtype=torch.float32, shape=(head_dim // 2,))
-        if positions is None:
-            raise KernelError("qk_norm_rope_append: rotation needs positions.")
-    if positions is not None:
-        _check(positions, "positions", dtype=torch.int32, shape=(n,))
+    cos = sin = None
+    if rope is not None:
+        cos, sin = rope
+        _check(cos, "rope cos", dtype=torch.float32, shape=(n, head_dim // 2))
+        _check(sin, "rope sin", dtype=torch.float32, shape=(n, head_dim // 2))
     block_size = 0
     if num_kv_heads > 0:
         if slot_mapping is None or key_pool is None or value_pool is None:
@@ -174,7 +189,7 @@ def qk_norm_rope_append(
     q_out = None
     if num_q_heads > 0:
         q_out = torch.empty((n, num_q_heads, head_dim), dtype=dtype, device=packed.device)
-    call("ms_qk_norm_rope_append", _ptr(packed), _ptr(q_weight), _ptr(k_weight), _ptr(inv_freq), _ptr(positions),
+    call("ms_qk_norm_rope_append", _ptr(packed), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin),
          _ptr(slot_mapping), _ptr(q_out), _ptr(key_pool), _ptr(value_pool), n, num_q_heads, num_kv_heads,
          head_dim, block_size, float(eps), _code(dtype), _stream())
     return q_out
@@ -231,7 +246,7 @@ def attention(
     geometry: the first ``decode_prefix`` tokens are single tokens of their
     sequences and go to the key-split kernel (``max_context``, the largest
     position + 1, sizes the split; ``splits`` overrides it); the other tokens go,
-    cut into ``tiles`` (a ``QueryTiles``: at most 16 consecutive tokens of one
+    cut into ``tiles`` (a ``QueryTiles``: at most 64 consecutive tokens of one
     sequence each), to the tiled kernel.  Without ``tiles`` and ``decode_prefix``
     the generic kernel serves every token."""
 

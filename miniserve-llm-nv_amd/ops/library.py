@@ -25,6 +25,7 @@ _SIGNATURES: dict[str, list] = {
     "ms_embedding_gather": [_P, _P, _P, _I, _I, _I, _I, _P],
     "ms_rmsnorm": [_P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _I, _P],
     "ms_residual_add": [_P, _P, _I, _I, _I, _P],
+    "ms_rope_table": [_P, _P, _P, _P, _I, _I, _P],
     "ms_qk_norm_rope_append": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
     "ms_attention_generic": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ms_attention_decode": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],

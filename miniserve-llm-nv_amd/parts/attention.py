@@ -97,8 +97,7 @@ class Attention(Part):
                 q_weight=None if self.q_norm is None else self.q_norm.weight,
                 k_weight=None if self.k_norm is None else self.k_norm.weight,
                 eps=next((p.eps for p in (self.q_norm, self.k_norm) if p is not None), 1.0),
-                inv_freq=None if self.position is None else self.position.inv_freq(x.device),
-                positions=ctx.positions,
+                rope=None if self.position is None else self.position.tables(ctx.positions, ctx),
                 slot_mapping=group.slot_mapping if cache.write else None,
                 key_pool=cache.key if cache.write else None,
                 value_pool=cache.value if cache.write else None,
@@ -147,8 +146,7 @@ class Attention(Part):
             q_weight=None,
             k_weight=None,
             eps=1.0,
-            inv_freq=None,
-            positions=None,
+            rope=None,
             slot_mapping=group.slot_mapping,
             key_pool=cache.key,
             value_pool=cache.value,

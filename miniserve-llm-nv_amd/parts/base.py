@@ -108,12 +108,12 @@ class GroupStepView:
 @dataclass
 class QueryTiles:
     """The tokens after the single-token prefix of a batch, cut into tiles of at most
-    16 consecutive tokens of one sequence (what the tiled attention kernel walks)."""
+    64 consecutive tokens of one sequence (what the tiled attention kernel walks)."""
 
     count: int
     seq: torch.Tensor       # int32 [count]: the tile's sequence (row of the block tables)
     token: torch.Tensor     # int32 [count]: index of the tile's first token in the batch
-    length: torch.Tensor    # int32 [count]: 1..16
+    length: torch.Tensor    # int32 [count]: 1..64
 
 
 @dataclass
@@ -140,6 +140,8 @@ class StepContext:
     first_positions_host: list[int] = field(default_factory=list)
     decode_prefix: int = 0
     tiles: QueryTiles | None = None
+    # what parts compute once per step and share between layers (position tables)
+    scratch: dict = field(default_factory=dict)
 
     @property
     def max_query_len(self) -> int:

@@ -36,6 +36,17 @@ class RotaryHalf(Part):
             self._inv_freq = self._inv_freq_host.to(device)
         return self._inv_freq
 
+    def tables(self, positions: torch.Tensor, ctx=None) -> tuple[torch.Tensor, torch.Tensor]:
+        """cos and sin ``[N, dim/2]`` (float32) for ``positions``; with a step context
+        they are made once and shared by every layer of the step."""
+
+        if ctx is None:
+            return ops.rope_table(positions, self.inv_freq(positions.device))
+        key = ("rotary_half", self.dim, self.theta)
+        if key not in ctx.scratch:
+            ctx.scratch[key] = ops.rope_table(ctx.positions, self.inv_freq(ctx.positions.device))
+        return ctx.scratch[key]
+
     def apply(self, x: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
         """``x [N, heads, dim]`` rotated by ``positions [N]`` (int32)."""
 
@@ -50,8 +61,7 @@ class RotaryHalf(Part):
             q_weight=None,
             k_weight=None,
             eps=1.0,
-            inv_freq=self.inv_freq(x.device),
-            positions=positions,
+            rope=self.tables(positions),
         )
 
 

@@ -123,10 +123,10 @@ def test_kernels_refuse_what_they_cannot_do(ops):
         ops.silu_mul(x.t())
     with pytest.raises(KernelError, match="exceeds"):
         ops.qk_norm_rope_append(rand(1, 1026), num_q_heads=1, num_kv_heads=0, head_dim=1026, q_weight=None,
-                                k_weight=None, eps=1.0, inv_freq=None, positions=None)
+                                k_weight=None, eps=1.0, rope=None)
     with pytest.raises(KernelError, match="even"):
         ops.qk_norm_rope_append(rand(1, 15), num_q_heads=1, num_kv_heads=0, head_dim=15, q_weight=None,
-                                k_weight=None, eps=1.0, inv_freq=None, positions=None)
+                                k_weight=None, eps=1.0, rope=None)
 
 
 # ---- q/k norm, rotation, cache write ------------------------------------------------------
@@ -146,7 +146,7 @@ def test_qk_norm_rope_append(ops, dtype, heads, kv_heads, dim, block):
     value_pool = torch.zeros(pages, kv_heads, dim, block, dtype=dtype, device=DEVICE)     # transposed inside a page
     q = ops.qk_norm_rope_append(
         packed, num_q_heads=heads, num_kv_heads=kv_heads, head_dim=dim, q_weight=qw, k_weight=kw, eps=eps,
-        inv_freq=inverse_frequencies(dim, theta).to(DEVICE), positions=positions, slot_mapping=slots,
+        rope=ops.rope_table(positions, inverse_frequencies(dim, theta).to(DEVICE)), slot_mapping=slots,
         key_pool=key_pool, value_pool=value_pool,
     )
     rows = packed.cpu().double().view(n, heads + 2 * kv_heads, dim)
@@ -179,14 +179,14 @@ def test_rotation_and_norm_alone(ops):
     x = rand(5, 3 * 32, seed=9)
     positions = torch.tensor([0, 3, 9, 100, 511], dtype=torch.int32, device=DEVICE)
     only_rope = ops.qk_norm_rope_append(x, num_q_heads=3, num_kv_heads=0, head_dim=32, q_weight=None, k_weight=None,
-                                        eps=1.0, inv_freq=inverse_frequencies(32, 1e4).to(DEVICE), positions=positions)
+                                        eps=1.0, rope=ops.rope_table(positions, inverse_frequencies(32, 1e4).to(DEVICE)))
     cos, sin = plain.rope_angles(positions.cpu().long(), 32, 1e4)
     expected = plain.apply_rope(x.cpu().double().view(5, 3, 32).transpose(0, 1), cos, sin).transpose(0, 1)
     torch.testing.assert_close(only_rope.cpu().double(), expected, atol=1e-5, rtol=1e-5)
     assert torch.equal(only_rope[0], x.view(5, 3, 32)[0])                       # position 0 is the identity
     weight = 1 + 0.1 * rand(32, seed=4)
     only_norm = ops.qk_norm_rope_append(x, num_q_heads=3, num_kv_heads=0, head_dim=32, q_weight=weight, k_weight=None,
-                                        eps=1e-6, inv_freq=None, positions=None)
+                                        eps=1e-6, rope=None)
     torch.testing.assert_close(only_norm.view(15, 32), ops.rmsnorm(x.view(15, 32), weight, 1e-6), atol=1e-6, rtol=1e-6)
 
 
@@ -247,17 +247,17 @@ def attention_reference(case, scale, window=None):
 
 
 def query_tiles(case, first_sequence):
-    """Tiles of at most 16 consecutive tokens for the sequences from ``first_sequence`` on."""
+    """Tiles of at most 64 consecutive tokens for the sequences from ``first_sequence`` on."""
 
     from miniserve_amd.parts import QueryTiles
 
     seqs, tokens, lengths, base = [], [], [], 0
     for index, qlen in enumerate(case["query_lens"]):
         if index >= first_sequence:
-            for start in range(0, qlen, 16):
+            for start in range(0, qlen, 64):
                 seqs.append(index)
                 tokens.append(base + start)
-                lengths.append(min(16, qlen - start))
+                lengths.append(min(64, qlen - start))
         base += qlen
     if not seqs:
         return None

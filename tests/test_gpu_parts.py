@@ -58,10 +58,10 @@ def step_context(query_lens, starts, block_size, *, tables=None):
         prefix += 1
     tile_seq, tile_token, tile_length = [], [], []
     for index in range(prefix, len(query_lens)):
-        for start in range(0, query_lens[index], 16):
+        for start in range(0, query_lens[index], 64):
             tile_seq.append(index)
             tile_token.append(starts_q[index] + start)
-            tile_length.append(min(16, query_lens[index] - start))
+            tile_length.append(min(64, query_lens[index] - start))
     tiles = QueryTiles(len(tile_seq), i32(tile_seq), i32(tile_token), i32(tile_length)) if tile_seq else None
     return StepContext(
         num_tokens=len(token_pos), num_seqs=len(query_lens), token_ids=i32([0] * len(token_pos)), positions=i32(token_pos),
