@@ -31,12 +31,19 @@ constexpr int kUnroll = 4;   // k-steps whose loads are issued together
 
 enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAddF32 = 2, kSiluMul = 3 };
 
-template <int MB, int RB>
+// NORM: x is not given; its rows are made on the fly from the 32-bit residual stream h:
+//   x[m, :] = bf16(w_norm * bf16(h[m, :] * rsqrt(mean(h[m, :]^2) + eps)))      (RMSNorm)
+// Every workgroup computes the statistics of the (at most 16) rows itself, in one
+// fixed order, so all of them see the same x.
+template <int MB, int RB, bool NORM>
 __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* __restrict__ x,
+                                                                    const float* __restrict__ h,
+                                                                    const bf16* __restrict__ norm_weight, float eps,
                                                                     const bf16* __restrict__ w, bf16* out_bf16,
                                                                     float* out_f32, int m, int n, int k,
                                                                     int epilogue) {
   __shared__ float c_s[kWavesPerGroup][RB * MB][16][16];
+  __shared__ float inv_s[16];
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -73,7 +80,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
   for (int mb = 0; mb < MB; ++mb) {
     const int row = 16 * mb + r;
     x_live[mb] = row < m;
-    x_row[mb] = x + static_cast<int64_t>(min(row, m - 1)) * k;
+    x_row[mb] = NORM ? nullptr : x + static_cast<int64_t>(min(row, m - 1)) * k;
   }
 
   floatx4 acc[RB][MB];
@@ -81,6 +88,30 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const float* h_row = nullptr;
+  float inv_rms = 0.f;
+  if (NORM) {
+    // 32 threads a row: thread t of the group takes row t / 32 and every 32nd quad of it
+    const int row = threadIdx.x >> 5, part = threadIdx.x & 31;
+    float partial = 0.f;
+    if (row < m) {
+      const float* source = h + static_cast<int64_t>(row) * k;
+      for (int i = 4 * part; i < k; i += 128) {
+        const float4 v = *reinterpret_cast<const float4*>(source + i);
+        partial = fmaf(v.x, v.x, partial);
+        partial = fmaf(v.y, v.y, partial);
+        partial = fmaf(v.z, v.z, partial);
+        partial = fmaf(v.w, v.w, partial);
+      }
+    }
+#pragma unroll
+    for (int offset = 16; offset > 0; offset >>= 1) partial += __shfl_xor(partial, offset, ms::kWave);
+    if (part == 0) inv_s[row] = 1.0f / sqrtf(partial / static_cast<float>(k) + eps);
+    __syncthreads();
+    inv_rms = inv_s[r];
+    h_row = h + static_cast<int64_t>(min(r, m - 1)) * k;
+  }
 
   const int steps = (k + 31) / 32;
   for (int base = wave; base < steps; base += kWavesPerGroup * kUnroll) {
@@ -91,9 +122,25 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
       const bool live = k0 < k;      // k is a multiple of 8
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) a[u][rb] = live ? ms::load_bf16x8(w_row[rb] + k0) : ms::zero_bf16x8();
+      if (NORM) {
+        bf16x8 made = ms::zero_bf16x8();
+        if (live && x_live[0]) {
+          const float4 lo = *reinterpret_cast<const float4*>(h_row + k0);
+          const float4 hi = *reinterpret_cast<const float4*>(h_row + k0 + 4);
+          const bf16x8 nw = ms::load_bf16x8(norm_weight + k0);
+          const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        b[u][mb] = (live && x_live[mb]) ? ms::load_bf16x8(x_row[mb] + k0) : ms::zero_bf16x8();
+          for (int i = 0; i < 8; ++i) {
+            const float normed = static_cast<float>(static_cast<__bf16>(v[i] * inv_rms));
+            made[i] = static_cast<__bf16>(static_cast<float>(nw[i]) * normed);
+          }
+        }
+        b[u][0] = made;
+      } else {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          b[u][mb] = (live && x_live[mb]) ? ms::load_bf16x8(x_row[mb] + k0) : ms::zero_bf16x8();
+      }
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
@@ -143,15 +190,16 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
   }
 }
 
-template <int MB, int RB>
+template <int MB, int RB, bool NORM = false>
 void launch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, int n, int k, int epilogue,
-            hipStream_t stream) {
+            hipStream_t stream, const void* h = nullptr, const void* norm_weight = nullptr, float eps = 0.f) {
   const int rows = epilogue == kSiluMul ? n / 2 : n;
   const int blocks_per_group = epilogue == kSiluMul ? RB / 2 : RB;
   const int groups = (rows + 16 * blocks_per_group - 1) / (16 * blocks_per_group);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB>), dim3(groups), dim3(kGroupThreads), 0, stream,
-                     static_cast<const bf16*>(x), static_cast<const bf16*>(w), static_cast<bf16*>(out_bf16),
-                     static_cast<float*>(out_f32), m, n, k, epilogue);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM>), dim3(groups), dim3(kGroupThreads), 0, stream,
+                     static_cast<const bf16*>(x), static_cast<const float*>(h),
+                     static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
+                     static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue);
 }
 
 }  // namespace
@@ -187,5 +235,24 @@ extern "C" int ms_gemm_skinny(const void* x, const void* w, void* out_bf16, void
     launch<4, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
   }
   MS_CHECK_LAUNCH("gemm_skinny");
+  return 0;
+}
+
+// The same product with the RMSNorm of the 32-bit residual stream as its input:
+// x = RMSNorm(h; norm_weight, eps), h: float [m, k], m <= 16, k a multiple of 8.
+// Epilogues 0 (bfloat16 [m, n]) and 3 (gated activation, bfloat16 [m, n / 2]).
+extern "C" int ms_gemm_skinny_normed(const void* h, const void* norm_weight, float eps, const void* w,
+                                     void* out_bf16, int m, int n, int k, int epilogue, hipStream_t stream) {
+  MS_REQUIRE(ms_gemm_skinny_supported(m, n, k, epilogue) && m <= 16 && (epilogue == kStoreBf16 || epilogue == kSiluMul),
+             "gemm_skinny_normed: m %d (1..16), n %d, k %d (a multiple of 8) or epilogue %d is not supported", m, n,
+             k, epilogue);
+  MS_REQUIRE(h && norm_weight && w && out_bf16, "gemm_skinny_normed: null operand");
+  MS_REQUIRE(eps > 0.f, "gemm_skinny_normed: eps must be positive");
+  if (epilogue == kSiluMul) {
+    launch<1, 2, true>(nullptr, w, out_bf16, nullptr, m, n, k, epilogue, stream, h, norm_weight, eps);
+  } else {
+    launch<1, 1, true>(nullptr, w, out_bf16, nullptr, m, n, k, epilogue, stream, h, norm_weight, eps);
+  }
+  MS_CHECK_LAUNCH("gemm_skinny_normed");
   return 0;
 }

@@ -16,7 +16,10 @@ __all__ = [
     "embedding_gather",
     "library_path",
     "linear",
+    "linear_normed",
     "linear_silu_mul",
+    "can_fuse_norm",
+    "can_accumulate",
     "load",
     "qk_norm_rope_append",
     "residual_add",
@@ -361,6 +364,44 @@ def linear(
         residual_add(accumulate_into, out)
         return accumulate_into
     return out.float() if out_float32 else out
+
+
+def can_accumulate(rows: int, weight: torch.Tensor) -> bool:
+    """Whether ``linear(..., accumulate_into=...)`` adds in the product's own epilogue
+    (else it would cost a kernel more than handing the sum to the next norm)."""
+
+    n, k = weight.shape
+    return weight.dtype == torch.float32 or _use_skinny(rows, n, k, _EPILOGUE_ADD_F32)
+
+
+def can_fuse_norm(rows: int, weight: torch.Tensor, *, gated: bool = False) -> bool:
+    """Whether :func:`linear_normed` runs as one kernel for this many rows."""
+
+    n, k = weight.shape
+    epilogue = _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16
+    return weight.dtype == torch.bfloat16 and _use_skinny(rows, n, k, epilogue)
+
+
+def linear_normed(
+    residual: torch.Tensor, norm_weight: torch.Tensor, eps: float, weight: torch.Tensor, *, gated: bool = False
+) -> torch.Tensor:
+    """``RMSNorm(residual) @ weight^T`` in one kernel (``gated``: then SiLU(gate) * up of
+    the two halves of the result): the norm of the float32 ``residual [M, K]`` is the
+    product's prologue.  Only where :func:`can_fuse_norm` says so."""
+
+    _check(residual, "residual", dtype=torch.float32)
+    _check(weight, "weight", dtype=torch.bfloat16)
+    if residual.ndim != 2 or weight.ndim != 2 or residual.shape[1] != weight.shape[1] or residual.shape[0] == 0:
+        raise KernelError(f"linear_normed: residual {tuple(residual.shape)} does not match weight {tuple(weight.shape)}.")
+    m, k = residual.shape
+    n = weight.shape[0]
+    _check(norm_weight, "norm_weight", dtype=torch.bfloat16, shape=(k,))
+    if not can_fuse_norm(m, weight, gated=gated):
+        raise KernelError("linear_normed: this shape is not served by the fused kernel.")
+    out = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=residual.device)
+    call("ms_gemm_skinny_normed", _ptr(residual), _ptr(norm_weight), float(eps), _ptr(weight), _ptr(out), m, n, k,
+         _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16, _stream())
+    return out
 
 
 def linear_silu_mul(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:

@@ -35,6 +35,7 @@ _SIGNATURES: dict[str, list] = {
     "ms_gemm_f32": [_P, _P, _P, _I, _I, _I, _I, _P],
     "ms_gemm_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
     "ms_gemm_skinny_supported": [_I, _I, _I, _I],
+    "ms_gemm_skinny_normed": [_P, _P, _F, _P, _P, _I, _I, _I, _I, _P],
     "ms_silu_mul": [_P, _P, _I, _I, _I, _P],
     "ms_sample_rows": [_P, _P, _P, _P, _P, _P, _I, _I, _P],
     "ms_argmax_rows": [_P, _P, _P, _P, _I, _I, _I, _P],

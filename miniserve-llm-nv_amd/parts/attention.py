@@ -14,12 +14,25 @@ import torch
 
 from .. import ops
 from ..config.model_spec import PartSpec
-from .base import KVCacheNeed, KVCacheView, Part, StepContext, WeightSpec, build_part, register_part, require_params
+from .base import (
+    KVCacheNeed,
+    KVCacheView,
+    Part,
+    PendingNorm,
+    StepContext,
+    WeightSpec,
+    build_part,
+    register_part,
+    require_params,
+)
 from .norm import RMSNorm
 from .rotary import RotaryHalf
 
 
 class Attention(Part):
+    accepts_pending_norm = True
+    accumulates_residual = True
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype) -> None:
         params = require_params(spec, "hidden_size", "num_heads", "num_kv_heads", "head_dim")
         self.hidden_size = int(params["hidden_size"])
@@ -81,13 +94,24 @@ class Attention(Part):
         self.w_o = tensors[self.prefix + "o_proj.weight"]
 
     # -- execution ------------------------------------------------------------------
-    def forward(self, x: torch.Tensor, ctx: StepContext, cache: KVCacheView) -> torch.Tensor:
+    def forward(self, x, ctx: StepContext, cache: KVCacheView, *, residual: torch.Tensor | None = None):
+        """``x``: the normed input ``[N, H]``, or a ``PendingNorm`` (then the norm becomes
+        the prologue of the q/k/v product where one kernel serves the shape).  With
+        ``residual`` the output may be added into it (the product's epilogue); None is returned then."""
+
         if not isinstance(cache, KVCacheView):
             raise TypeError("attention needs a paged key/value cache.")
         group = ctx.groups[cache.group]
         n = x.shape[0]
         kv_heads = self.num_kv_heads if cache.write else 0
-        packed = ops.linear(x, self.w_qkv if cache.write else self.w_q)
+        w_in = self.w_qkv if cache.write else self.w_q
+        if isinstance(x, PendingNorm):
+            if x.fusable and ops.can_fuse_norm(n, w_in):
+                packed = ops.linear_normed(x.residual, x.norm.weight, x.norm.eps, w_in)
+            else:
+                packed = ops.linear(x.materialize(), w_in)
+        else:
+            packed = ops.linear(x, w_in)
         if self._fused:
             q = ops.qk_norm_rope_append(
                 packed,
@@ -117,7 +141,11 @@ class Attention(Part):
             tiles=ctx.tiles,
             max_context=ctx.max_context_len,
         )
-        return ops.linear(attended.reshape(n, self.num_heads * self.head_dim), self.w_o)
+        attended = attended.reshape(n, self.num_heads * self.head_dim)
+        if residual is not None and ops.can_accumulate(n, self.w_o):
+            ops.linear(attended, self.w_o, accumulate_into=residual)
+            return None
+        return ops.linear(attended, self.w_o)
 
     def _prepare_unfused(self, packed, ctx, cache, group, kv_heads) -> torch.Tensor:
         """Norms and position encoding through their own parts, then the cache write."""

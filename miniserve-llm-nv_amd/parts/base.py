@@ -152,6 +152,36 @@ class StepContext:
         return max(self.context_lens_host)
 
 
+# ---- a norm that is not yet taken ------------------------------------------------------
+
+class PendingNorm:
+    """``norm(residual + delta)``, not yet computed.  A block hands it to a mixer or a
+    feed-forward that sets ``accepts_pending_norm = True``; such a part may fuse the
+    norm into its first product (when ``fusable``: an RMSNorm whose input is the bare
+    residual stream) or call :meth:`materialize` for the normed tensor.  Every other
+    part receives the materialised tensor."""
+
+    def __init__(self, norm, residual: torch.Tensor, delta: torch.Tensor | None) -> None:
+        self.norm = norm
+        self.residual = residual
+        self.delta = delta
+        self._value: torch.Tensor | None = None
+
+    @property
+    def fusable(self) -> bool:
+        return self.delta is None and hasattr(self.norm, "eps") and getattr(self.norm, "weight", None) is not None
+
+    @property
+    def shape(self):
+        return self.residual.shape
+
+    def materialize(self) -> torch.Tensor:
+        if self._value is None:
+            self._value = self.norm.add_forward(self.residual, self.delta)
+            self.delta = None       # the sum has been stored into the residual stream
+        return self._value
+
+
 # ---- registries -------------------------------------------------------------------
 
 _REGISTRIES: dict[str, dict[str, Callable[..., Any]]] = {category: {} for category in CATEGORIES}

@@ -9,13 +9,16 @@ import torch
 
 from .. import ops
 from ..config.model_spec import PartSpec
-from .base import Part, StepContext, WeightSpec, register_part, require_params
+from .base import Part, PendingNorm, StepContext, WeightSpec, register_part, require_params
 
 # activation name -> (gated activation of a packed [N, 2 I] row, the same fused with the product)
 _ACTIVATIONS = {"silu": (ops.silu_mul, ops.linear_silu_mul)}
 
 
 class GatedMLP(Part):
+    accepts_pending_norm = True
+    accumulates_residual = True
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype) -> None:
         params = require_params(spec, "hidden_size", "intermediate_size", "activation")
         self.hidden_size = int(params["hidden_size"])
@@ -24,6 +27,7 @@ class GatedMLP(Part):
         if activation not in _ACTIVATIONS:
             raise ValueError(f"gated_mlp knows the activations {sorted(_ACTIVATIONS)}, not {activation!r}.")
         self._gated_activation, self._gated_product = _ACTIVATIONS[activation]
+        self._fused_with_norm = activation == "silu"      # the fused kernel's epilogue is SiLU * up
         self.dtype = dtype
         self.prefix = spec.prefix
         self.w_gate_up: torch.Tensor | None = None
@@ -44,8 +48,22 @@ class GatedMLP(Part):
         ).contiguous()
         self.w_down = tensors[self.prefix + "down_proj.weight"]
 
-    def forward(self, x: torch.Tensor, ctx: StepContext | None = None) -> torch.Tensor:
-        return ops.linear(self._gated_product(x, self.w_gate_up), self.w_down)
+    def forward(self, x, ctx: StepContext | None = None, *, residual: torch.Tensor | None = None):
+        """``x``: the normed input, or a ``PendingNorm`` (then the norm becomes the
+        prologue of the gate/up product where one kernel serves the shape).  With
+        ``residual`` the output may be added into it (the product's epilogue); None is returned then."""
+
+        if isinstance(x, PendingNorm):
+            if x.fusable and self._fused_with_norm and ops.can_fuse_norm(x.shape[0], self.w_gate_up, gated=True):
+                hidden = ops.linear_normed(x.residual, x.norm.weight, x.norm.eps, self.w_gate_up, gated=True)
+            else:
+                hidden = self._gated_product(x.materialize(), self.w_gate_up)
+        else:
+            hidden = self._gated_product(x, self.w_gate_up)
+        if residual is not None and ops.can_accumulate(hidden.shape[0], self.w_down):
+            ops.linear(hidden, self.w_down, accumulate_into=residual)
+            return None
+        return ops.linear(hidden, self.w_down)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

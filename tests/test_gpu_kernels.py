@@ -644,3 +644,24 @@ def test_sampler_stages_without_advancing_the_stream(ops):
         sampler.sample(logits, [("k", SamplingParams(temperature=1.0, top_k=5))])
     with pytest.raises(TypeError, match="floating-point"):
         sampler.sample(torch.tensor([[1, 2, 3]], device=DEVICE), [("i", SamplingParams())])
+
+
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("n,k", [(48, 64), (512, 96), (4096, 1024), (200, 200)])
+def test_product_with_the_norm_as_its_prologue(ops, m, n, k):
+    """RMSNorm of the 32-bit residual stream fused into the few-rows product equals the
+    norm kernel followed by the product, also with the gated activation behind it."""
+
+    residual = rand(m, k, seed=m + n, scale=2.0)
+    norm_weight = (1 + 0.1 * rand(k, seed=5)).to(torch.bfloat16)
+    weight = rand(n, k, seed=n + k, dtype=torch.bfloat16, scale=0.05)
+    assert ops.can_fuse_norm(m, weight) and ops.can_fuse_norm(m, weight, gated=True)
+    normed = ops.rmsnorm(residual, norm_weight, 1e-5)
+    fused = ops.linear_normed(residual, norm_weight, 1e-5, weight)
+    torch.testing.assert_close(fused.float(), ops.linear(normed, weight).float(), atol=2e-2, rtol=2e-2)
+    exact = rmsnorm_reference(residual, norm_weight, 1e-5, torch.bfloat16).cpu().double() @ weight.cpu().double().T
+    torch.testing.assert_close(fused.cpu().double(), exact, atol=float(exact.abs().max()) * 2**-7, rtol=2**-7)
+    gated = ops.linear_normed(residual, norm_weight, 1e-5, weight, gated=True)
+    torch.testing.assert_close(gated.float(), ops.linear_silu_mul(normed, weight).float(), atol=2e-2, rtol=2e-2)
+    assert not ops.can_fuse_norm(17, weight)
+    assert not ops.can_fuse_norm(m, weight.float())
