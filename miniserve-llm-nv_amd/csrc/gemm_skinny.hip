@@ -31,10 +31,14 @@ constexpr int kUnroll = 4;   // k-steps whose loads are issued together
 
 enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAddF32 = 2, kSiluMul = 3 };
 
-// NORM: x is not given; its rows are made on the fly from the 32-bit residual stream h:
-//   x[m, :] = bf16(w_norm * bf16(h[m, :] * rsqrt(mean(h[m, :]^2) + eps)))      (RMSNorm)
-// Every workgroup computes the statistics of the (at most 16) rows itself, in one
-// fixed order, so all of them see the same x.
+// NORM: x is not given; the product is taken of the RMSNorm of the 32-bit residual
+// stream h, with the normalisation moved behind the sum so that nothing waits for
+// the row statistics:
+//   out[m, n] = rsqrt(mean(h[m, :]^2) + eps) * sum_k W[n, k] * bf16(w_norm[k] * h[m, k])
+// The squares are summed by the same loop that makes the operands; every workgroup
+// sums them in the same fixed order.  (The separate norm kernel rounds the
+// normalised value before the multiply by the weight, as the reference does; here
+// the one rounding is of w_norm * h.  Both carry 8 significant bits.)
 template <int MB, int RB, bool NORM>
 __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                     const float* __restrict__ h,
@@ -43,7 +47,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
                                                                     float* out_f32, int m, int n, int k,
                                                                     int epilogue) {
   __shared__ float c_s[kWavesPerGroup][RB * MB][16][16];
-  __shared__ float inv_s[16];
+  __shared__ float square_s[kWavesPerGroup][16];
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -89,29 +93,9 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  const float* h_row = nullptr;
-  float inv_rms = 0.f;
-  if (NORM) {
-    // 32 threads a row: thread t of the group takes row t / 32 and every 32nd quad of it
-    const int row = threadIdx.x >> 5, part = threadIdx.x & 31;
-    float partial = 0.f;
-    if (row < m) {
-      const float* source = h + static_cast<int64_t>(row) * k;
-      for (int i = 4 * part; i < k; i += 128) {
-        const float4 v = *reinterpret_cast<const float4*>(source + i);
-        partial = fmaf(v.x, v.x, partial);
-        partial = fmaf(v.y, v.y, partial);
-        partial = fmaf(v.z, v.z, partial);
-        partial = fmaf(v.w, v.w, partial);
-      }
-    }
-#pragma unroll
-    for (int offset = 16; offset > 0; offset >>= 1) partial += __shfl_xor(partial, offset, ms::kWave);
-    if (part == 0) inv_s[row] = 1.0f / sqrtf(partial / static_cast<float>(k) + eps);
-    __syncthreads();
-    inv_rms = inv_s[r];
-    h_row = h + static_cast<int64_t>(min(r, m - 1)) * k;
-  }
+  // NORM: this lane makes column m = r of x from row r of h, and sums its squares
+  const float* h_row = NORM ? h + static_cast<int64_t>(min(r, m - 1)) * k : nullptr;
+  float square_sum = 0.f;
 
   const int steps = (k + 31) / 32;
   for (int base = wave; base < steps; base += kWavesPerGroup * kUnroll) {
@@ -131,8 +115,8 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
           const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
-            const float normed = static_cast<float>(static_cast<__bf16>(v[i] * inv_rms));
-            made[i] = static_cast<__bf16>(static_cast<float>(nw[i]) * normed);
+            square_sum = fmaf(v[i], v[i], square_sum);
+            made[i] = static_cast<__bf16>(static_cast<float>(nw[i]) * v[i]);
           }
         }
         b[u][0] = made;
@@ -157,6 +141,11 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int e = 0; e < 4; ++e) c_s[wave][rb * MB + mb][r][4 * g + e] = acc[rb][mb][e];
+  if (NORM) {
+    square_sum += __shfl_xor(square_sum, 16, ms::kWave);
+    square_sum += __shfl_xor(square_sum, 32, ms::kWave);
+    if (g == 0) square_s[wave][r] = square_sum;
+  }
   __syncthreads();
 
   // c_s[wave][tile][m_local][n_local]; consecutive threads take consecutive n
@@ -173,6 +162,14 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     float sum = 0.f;
 #pragma unroll
     for (int wv = 0; wv < kWavesPerGroup; ++wv) sum += c_s[wv][tile][m_local][n_local];
+    float inv_rms = 1.f;
+    if (NORM) {
+      float squares = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < kWavesPerGroup; ++wv) squares += square_s[wv][m_local];
+      inv_rms = 1.0f / sqrtf(squares / static_cast<float>(k) + eps);
+      sum *= inv_rms;
+    }
     if (epilogue == kStoreBf16) {
       out_bf16[static_cast<int64_t>(row_m) * n + col_n] = ms::from_float<bf16>(sum);
     } else if (epilogue == kStoreF32) {
@@ -183,6 +180,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
       float up = 0.f;
 #pragma unroll
       for (int wv = 0; wv < kWavesPerGroup; ++wv) up += c_s[wv][(rb + RB / 2) * MB + mb][m_local][n_local];
+      up *= inv_rms;
       const float gate = ms::round_to<bf16>(sum);
       up = ms::round_to<bf16>(up);
       out_bf16[static_cast<int64_t>(row_m) * half + col_n] = ms::from_float<bf16>(gate / (1.0f + __expf(-gate)) * up);
