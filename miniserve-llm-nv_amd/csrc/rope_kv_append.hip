@@ -117,6 +117,192 @@ int launch(const void* packed, const void* q_weight, const void* k_weight, const
   return 0;
 }
 
+// ---- the same for head sizes in steps of 16, 16 bytes a lane ----------------
+//
+// A workgroup takes one head of a tile of consecutive tokens; a (token, head) row is
+// held by head_dim / 16 lanes, each with 8 elements of the lower and the matching 8
+// of the upper half.  The squares are summed through LDS in a fixed order.  Values
+// go through LDS to be written transposed: runs of tokens in consecutive slots that
+// fill an aligned 16 bytes of a page's row are written by one store.
+
+constexpr int kTiledThreads = 256;
+constexpr int kTiledMaxElements = kTiledThreads * 16;   // elements of one head of a tile
+
+__device__ __forceinline__ void load8(const ms::bf16* src, float out[8]) {
+  const uint4 raw = *reinterpret_cast<const uint4*>(src);
+  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[2 * i] = ms::bf16_bits_to_float(static_cast<uint16_t>(words[i]));
+    out[2 * i + 1] = ms::bf16_bits_to_float(static_cast<uint16_t>(words[i] >> 16));
+  }
+}
+
+__device__ __forceinline__ void load8(const float* src, float out[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(src);
+  const float4 b = *reinterpret_cast<const float4*>(src + 4);
+  out[0] = a.x, out[1] = a.y, out[2] = a.z, out[3] = a.w;
+  out[4] = b.x, out[5] = b.y, out[6] = b.z, out[7] = b.w;
+}
+
+__device__ __forceinline__ void store8(ms::bf16* dst, const float in[8]) {
+  uint32_t words[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    words[i] = static_cast<uint32_t>(ms::float_to_bf16_bits(in[2 * i])) |
+               (static_cast<uint32_t>(ms::float_to_bf16_bits(in[2 * i + 1])) << 16);
+  *reinterpret_cast<uint4*>(dst) = make_uint4(words[0], words[1], words[2], words[3]);
+}
+
+__device__ __forceinline__ void store8(float* dst, const float in[8]) {
+  *reinterpret_cast<float4*>(dst) = make_float4(in[0], in[1], in[2], in[3]);
+  *reinterpret_cast<float4*>(dst + 4) = make_float4(in[4], in[5], in[6], in[7]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kernel(
+    const T* __restrict__ packed, const T* __restrict__ q_weight, const T* __restrict__ k_weight,
+    const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+    const int32_t* __restrict__ slot_mapping, T* __restrict__ q_out, T* __restrict__ key_pool,
+    T* __restrict__ value_pool, int num_tokens, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+    float eps) {
+  constexpr int kGroup = 16 / static_cast<int>(sizeof(T));   // values of one 16-byte store
+  __shared__ float square_s[kTiledThreads];
+  __shared__ int32_t slot_s[kTiledThreads];
+  __shared__ __align__(16) T tile_s[kTiledMaxElements];
+
+  const int half = head_dim / 2;
+  const int lanes_per_row = half / 8;
+  const int tile_tokens = kTiledThreads / lanes_per_row;
+  const int head = blockIdx.y;
+  const int64_t first_token = static_cast<int64_t>(blockIdx.x) * tile_tokens;
+  const int live_tokens = static_cast<int>(min(static_cast<int64_t>(tile_tokens), num_tokens - first_token));
+  const int item = threadIdx.x / lanes_per_row;
+  const int part = threadIdx.x - item * lanes_per_row;
+  const bool live = item < live_tokens;
+  const int64_t token = first_token + (live ? item : 0);
+  const int packed_heads = num_q_heads + 2 * num_kv_heads;
+  const T* row = packed + (token * packed_heads + head) * head_dim;
+
+  const bool is_q = head < num_q_heads;
+  const bool is_k = !is_q && head < num_q_heads + num_kv_heads;
+
+  float lo[8], hi[8];
+  if (live) {
+    load8(row + 8 * part, lo);
+    load8(row + half + 8 * part, hi);
+  }
+
+  if (!is_q && !is_k) {
+    // values: through LDS, written along the page's offset axis
+    const int kv_head = head - num_q_heads - num_kv_heads;
+    if (live) {
+      store8(tile_s + item * head_dim + 8 * part, lo);
+      store8(tile_s + item * head_dim + half + 8 * part, hi);
+    }
+    if (threadIdx.x < live_tokens) slot_s[threadIdx.x] = slot_mapping[first_token + threadIdx.x];
+    __syncthreads();
+    const bool vector_ok = block_size % kGroup == 0;
+    for (int task = threadIdx.x; task < live_tokens * head_dim; task += kTiledThreads) {
+      const int j = task / head_dim;
+      const int d = task - j * head_dim;
+      const int32_t slot = slot_s[j];
+      // a run starts where the slots stop being consecutive or a 16-byte group begins
+      if (j > 0 && slot == slot_s[j - 1] + 1 && slot % kGroup != 0) continue;
+      int run = 1;
+      while (run < kGroup && j + run < live_tokens && slot_s[j + run] == slot + run && (slot + run) % kGroup != 0)
+        ++run;
+      const int64_t page = slot / block_size;
+      const int offset = slot - static_cast<int32_t>(page) * block_size;
+      T* dst = value_pool + ((page * num_kv_heads + kv_head) * head_dim + d) * block_size + offset;
+      if (vector_ok && run == kGroup && offset % kGroup == 0) {
+        __align__(16) T gathered[kGroup];
+#pragma unroll
+        for (int i = 0; i < kGroup; ++i) gathered[i] = tile_s[(j + i) * head_dim + d];
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(gathered);
+      } else {
+        // the run stays inside one page only if the offsets do
+        for (int i = 0; i < run; ++i) {
+          const int32_t s = slot + i;
+          const int64_t pg = s / block_size;
+          const int off = s - static_cast<int32_t>(pg) * block_size;
+          value_pool[((pg * num_kv_heads + kv_head) * head_dim + d) * block_size + off] = tile_s[(j + i) * head_dim + d];
+        }
+      }
+    }
+    return;
+  }
+
+  const T* weight = is_q ? q_weight : k_weight;
+  if (weight) {
+    float partial = 0.f;
+    if (live) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        partial = fmaf(lo[i], lo[i], partial);
+        partial = fmaf(hi[i], hi[i], partial);
+      }
+    }
+    square_s[threadIdx.x] = partial;
+    __syncthreads();
+    if (live) {
+      float total = 0.f;
+      for (int p = 0; p < lanes_per_row; ++p) total += square_s[item * lanes_per_row + p];
+      const float inv = 1.0f / sqrtf(total / static_cast<float>(head_dim) + eps);
+      float w_lo[8], w_hi[8];
+      load8(weight + 8 * part, w_lo);
+      load8(weight + half + 8 * part, w_hi);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        lo[i] = ms::round_to<T>(w_lo[i] * ms::round_to<T>(lo[i] * inv));
+        hi[i] = ms::round_to<T>(w_hi[i] * ms::round_to<T>(hi[i] * inv));
+      }
+    }
+  }
+  if (!live) return;
+
+  if (cos_table != nullptr) {
+    float cs[8], sn[8];
+    load8(cos_table + token * half + 8 * part, cs);
+    load8(sin_table + token * half + 8 * part, sn);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float a = lo[i], b = hi[i];
+      lo[i] = a * cs[i] - b * sn[i];
+      hi[i] = b * cs[i] + a * sn[i];
+    }
+  }
+
+  T* dst;
+  if (is_q) {
+    dst = q_out + (token * num_q_heads + head) * head_dim;
+  } else {
+    const int kv_head = head - num_q_heads;
+    const int64_t slot = slot_mapping[token];
+    const int64_t page = slot / block_size;
+    const int64_t offset = slot - page * block_size;
+    dst = key_pool + ((page * num_kv_heads + kv_head) * block_size + offset) * head_dim;
+  }
+  store8(dst + 8 * part, lo);
+  store8(dst + half + 8 * part, hi);
+}
+
+template <typename T>
+void launch_tiled(const void* packed, const void* q_weight, const void* k_weight, const void* cos_table,
+                  const void* sin_table, const void* slot_mapping, void* q_out, void* key_pool, void* value_pool,
+                  int num_tokens, int num_q_heads, int num_kv_heads, int head_dim, int block_size, float eps,
+                  hipStream_t stream) {
+  const int tile_tokens = kTiledThreads / (head_dim / 16);
+  const dim3 grid((num_tokens + tile_tokens - 1) / tile_tokens, num_q_heads + 2 * num_kv_heads);
+  hipLaunchKernelGGL((qk_norm_rope_append_tiled_kernel<T>), grid, dim3(kTiledThreads), 0, stream,
+      static_cast<const T*>(packed), static_cast<const T*>(q_weight), static_cast<const T*>(k_weight),
+      static_cast<const float*>(cos_table), static_cast<const float*>(sin_table),
+      static_cast<const int32_t*>(slot_mapping), static_cast<T*>(q_out), static_cast<T*>(key_pool),
+      static_cast<T*>(value_pool), num_tokens, num_q_heads, num_kv_heads, head_dim, block_size, eps);
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
 // cos and sin of float(position) * inv_freq[i], in 32-bit, for every token of the step.
 __global__ void rope_table_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
                                   float* __restrict__ cos_table, float* __restrict__ sin_table, int64_t total, int half) {
@@ -168,6 +354,24 @@ extern "C" int ms_qk_norm_rope_append(const void* packed, const void* q_weight, 
   }
   MS_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "qk_norm_rope_append: rotation needs both tables");
   MS_REQUIRE(num_q_heads + 2 * num_kv_heads <= 65535, "qk_norm_rope_append: too many heads");
+  // 16 bytes a lane where the head size is a multiple of 16 and every operand is
+  // aligned to 16 bytes (null operands are),
+  // for more tokens than two tiles; few tokens are quicker with a wave to each row
+  const bool tiled = head_dim % 16 == 0 && head_dim <= 16 * kTiledThreads &&
+                     num_tokens > 2 * (kTiledThreads / (head_dim / 16)) && aligned16(packed) &&
+                     aligned16(q_weight) && aligned16(k_weight) && aligned16(cos_table) && aligned16(sin_table) &&
+                     aligned16(q_out) && aligned16(key_pool) && aligned16(value_pool);
+  if (tiled && (dtype == MS_F32 || dtype == MS_BF16)) {
+    if (dtype == MS_F32) {
+      launch_tiled<float>(packed, q_weight, k_weight, cos_table, sin_table, slot_mapping, q_out, key_pool,
+                          value_pool, num_tokens, num_q_heads, num_kv_heads, head_dim, block_size, eps, stream);
+    } else {
+      launch_tiled<ms::bf16>(packed, q_weight, k_weight, cos_table, sin_table, slot_mapping, q_out, key_pool,
+                             value_pool, num_tokens, num_q_heads, num_kv_heads, head_dim, block_size, eps, stream);
+    }
+    MS_CHECK_LAUNCH("qk_norm_rope_append");
+    return 0;
+  }
   int rc;
   if (dtype == MS_F32) {
     rc = launch<float>(packed, q_weight, k_weight, cos_table, sin_table, slot_mapping, q_out, key_pool, value_pool,

@@ -171,6 +171,54 @@ def test_qk_norm_rope_append(ops, dtype, heads, kv_heads, dim, block):
     assert torch.all(untouched(key_pool.cpu()) == 0) and torch.all(untouched(values) == 0)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,dim,block,start", [(4, 2, 128, 16, 5), (2, 1, 80, 8, 0), (3, 3, 16, 12, 7), (2, 2, 64, 4, 3), (1, 1, 512, 16, 9)])
+def test_append_of_a_run_of_tokens_beside_single_ones(ops, dtype, heads, kv_heads, dim, block, start):
+    """A portion of a prompt that starts in the middle of a page and runs over several
+    pages (handed out in reverse), behind three single tokens in pages of their own:
+    every key and value lands in its slot and nothing else is touched."""
+
+    from miniserve_amd.parts.rotary import inverse_frequencies
+
+    run, theta, eps = max(150, 2 * 256 * 16 // dim + 40), 1e4, 1e-6     # enough for the many-token kernel
+    run_pages = (start + run + block - 1) // block
+    pages = run_pages + 3
+    table = list(range(run_pages - 1, -1, -1))                                  # logical -> physical page
+    run_slots = [table[(start + i) // block] * block + (start + i) % block for i in range(run)]
+    single_slots = [(run_pages + i) * block + (3 * i + 1) % block for i in range(3)]
+    slots = torch.tensor(single_slots + run_slots, dtype=torch.int32, device=DEVICE)
+    n = len(slots)
+    positions = torch.tensor([900, 17, 4000] + list(range(start, start + run)), dtype=torch.int32, device=DEVICE)
+    packed = rand(n, (heads + 2 * kv_heads) * dim, seed=dim + block, dtype=dtype)
+    qw = (1 + 0.1 * rand(dim, seed=1)).to(dtype)
+    kw = (1 + 0.1 * rand(dim, seed=2)).to(dtype)
+    key_pool = torch.zeros(pages, kv_heads, block, dim, dtype=dtype, device=DEVICE)
+    value_pool = torch.zeros(pages, kv_heads, dim, block, dtype=dtype, device=DEVICE)
+    q = ops.qk_norm_rope_append(
+        packed, num_q_heads=heads, num_kv_heads=kv_heads, head_dim=dim, q_weight=qw, k_weight=kw, eps=eps,
+        rope=ops.rope_table(positions, inverse_frequencies(dim, theta).to(DEVICE)), slot_mapping=slots,
+        key_pool=key_pool, value_pool=value_pool,
+    )
+    rows = packed.cpu().double().view(n, heads + 2 * kv_heads, dim)
+    cos, sin = plain.rope_angles(positions.cpu().long(), dim, theta)
+
+    def prepare(x, weight):
+        normed = rmsnorm_reference(x, weight.cpu(), eps, dtype).double()
+        return plain.apply_rope(normed.transpose(0, 1), cos, sin).transpose(0, 1)
+
+    tol = tolerance(dtype, 1e-5, 1.6e-2)
+    torch.testing.assert_close(q.cpu().double(), prepare(rows[:, :heads], qw), atol=tol, rtol=tol)
+    page, offset = slots.cpu().long() // block, slots.cpu().long() % block
+    torch.testing.assert_close(key_pool.cpu().double()[page, :, offset], prepare(rows[:, heads : heads + kv_heads], kw),
+                               atol=tol, rtol=tol)
+    values = value_pool.cpu().double().transpose(2, 3)
+    assert torch.equal(values[page, :, offset], rows[:, heads + kv_heads :])
+    touched = torch.zeros(pages, block, dtype=torch.bool)
+    touched[page, offset] = True
+    untouched = lambda pool: pool.permute(0, 2, 1, 3)[~touched]
+    assert torch.all(untouched(key_pool.cpu()) == 0) and torch.all(untouched(values) == 0)
+
+
 def test_rotation_and_norm_alone(ops):
     """Without weights the kernel is the rotation alone; without frequencies the norm alone."""
 
