@@ -4,8 +4,8 @@
 
 A "step" is one decode step of the engine loop (schedule, the step function over
 the paged cache, sampling) with ``--batch`` live requests, each after a prompt of
-``--prompt-len`` random tokens.  The model has the layer sizes of Qwen3-0.6B with
-random weights.  One JSON line is printed: decoded tokens a second, the prefill
+``--prompt-len`` random tokens.  The model has the layer sizes of Qwen3-0.6B (or
+of ``--size``) with random weights.  One JSON line is printed: decoded tokens a second, the prefill
 rate of one 2,048-token prompt with its fraction of the bf16 MFMA peak, the
 fraction of the HBM peak that the decode step reaches, and decode rates at batch
 1 and 64.
@@ -28,11 +28,16 @@ if ROOT not in sys.path:
 HBM_GBPS = 8000.0
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}
 
-QWEN3_0_6B = dict(
-    hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16, num_key_value_heads=8,
-    head_dim=128, vocab_size=151936, max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1e6,
-    tie_word_embeddings=True,
-)
+# layer sizes of the Qwen3 dense models; the default run is the first
+_COMMON = dict(head_dim=128, vocab_size=151936, max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1e6)
+SIZES = {
+    "0.6B": dict(hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16,
+                 num_key_value_heads=8, tie_word_embeddings=True, **_COMMON),
+    "8B": dict(hidden_size=4096, intermediate_size=12288, num_hidden_layers=36, num_attention_heads=32,
+               num_key_value_heads=8, tie_word_embeddings=False, **_COMMON),
+    "32B": dict(hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64,
+                num_key_value_heads=8, tie_word_embeddings=False, **_COMMON),
+}
 
 
 def parse_args():
@@ -43,6 +48,7 @@ def parse_args():
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--prompt-len", type=int, default=2048)
     parser.add_argument("--context", type=int, default=4096)
+    parser.add_argument("--size", default="0.6B", choices=tuple(SIZES), help="layer sizes of this Qwen3 model")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--prefill-tokens", type=int, default=2048)
@@ -90,7 +96,7 @@ def main() -> int:
     from miniserve_amd.config import EngineConfig, Qwen3Config
     from miniserve_amd.engine import Engine, ModelRunner, SamplingParams, StepEntry
 
-    sizes = dict(QWEN3_0_6B)
+    sizes = dict(SIZES[args.size])
     full_layers = sizes["num_hidden_layers"]
     if args.layers is not None:
         sizes["num_hidden_layers"] = args.layers
@@ -167,7 +173,8 @@ def main() -> int:
             points[f"decode_b{batch}"] = round(rate, 1)
 
     line = {
-        "metric": "decode tok/s at batch 8 (Qwen3-0.6B sizes, 2,048-token prompts, paged cache)",
+        "metric": f"decode tok/s at batch {args.batch} (Qwen3-{args.size} sizes, {args.prompt_len:,}-token prompts, "
+                  "paged cache)",
         "value": round(value, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -180,7 +187,7 @@ def main() -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: random weights, uniform random token ids",
         "config": {
-            "model": "Qwen3-0.6B sizes",
+            "model": f"Qwen3-{args.size} sizes",
             "global_batch": args.batch,
             "seq_len": args.context,
             "prompt_len": args.prompt_len,
