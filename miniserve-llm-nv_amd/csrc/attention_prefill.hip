@@ -1,18 +1,20 @@
 // Paged causal attention for rows that bring runs of query tokens (prompts and
 // their portions), bfloat16 storage, matrix cores.
 //
-// A workgroup of 4 waves owns a tile of up to 64 consecutive query tokens of one
-// sequence and HB query heads that share a kv head; each wave owns 16 of the tokens:
-// 16 * HB columns.  The workgroup walks the keys 0 .. (its last token's position)
-// in pairs of tiles of 16; all threads load a pair together (16 bytes a thread,
-// three pairs in flight in registers) into one of two LDS buffers, and every wave
-// reads its matrix-core operands from there.  Each wave keeps for every column an
-// online softmax in 32-bit:
+// A workgroup owns a tile of up to 64 consecutive query tokens of one sequence and HB
+// query heads that share a kv head: 64 * HB columns, 32 to a wave (16 tokens of two
+// heads, or 32 tokens of one).  It walks the keys 0 .. (its last token's position) in
+// pairs of tiles of 16; its threads load a pair together (16 bytes a thread) into an
+// LDS buffer, and every wave reads its matrix-core operands from there.  With
+// 32x32x16 products
 //
-//   S^T[key, query] = K[key, :] . Q[query, :]     A = K tile, B = Q^T (16 queries of one head)
-//   P = exp(S * scale - m), masked to lo <= key <= position of the query
-//   O[query, d]    += P[query, keys] . V[keys, d]
+//   S^T[key, column]  = K[key, :] . Q[column, :]       A = 32 keys, B = Q^T
+//   P = exp(S * scale - m), masked to lo <= key <= position of the column's token
+//   O^T[d, column]   += V^T[d, keys] . P^T[keys, column]
 //
+// a column's scores, its running maximum and sum and its outputs all live in the two
+// lanes column and column + 32: the online softmax needs one exchange between the
+// halves of the wave a step, and rescaling and the final division are per lane.
 // Every key and value read from memory serves all 64 * HB columns.  The mask is by
 // absolute position, so a portion of a prompt sees the history in the cache and
 // itself (reference: miniserve/model/qwen3.py:237-249, where the scores of a chunk
@@ -24,125 +26,23 @@ namespace {
 using ms::bf16;
 using ms::bf16x4;
 using ms::bf16x8;
-using ms::floatx4;
+using ms::floatx16;
 using ms::kTileKeys;
-using ms::load_pair;
-using ms::TilePair;
 
-constexpr int kQueryTile = 16;        // query tokens of one wave
-constexpr int kBlockWaves = 4;        // waves of a workgroup: 64 query tokens share the keys and values in LDS
-constexpr int kBlockThreads = kBlockWaves * ms::kWave;
+constexpr int kTileTokens = 64;       // query tokens of a workgroup at most
+constexpr int kWaveColumns = 32;      // columns (token, head) of one wave
 
-template <int D, int HB>
-struct PrefillState {
-  floatx4 o[HB][D / 16];
-  float run_max[HB], run_sum[HB];   // of query column r (the same in all four lane groups)
-};
-
-// Softmax arithmetic runs in base 2: scores are multiplied by scale * log2(e) once
-// and exp2 is one instruction.  The running maximum of a column moves only when a
-// tile exceeds it by more than kMaxSlack (in base-2 units): weights may then be as
-// large as 2^kMaxSlack instead of 1, which 32-bit sums and bfloat16 weights hold
-// without loss, and the rescaling of the output tile - the most expensive vector
-// work of a step - is skipped for the steps in which no column's maximum moved.
+// Softmax arithmetic runs in base 2: the scale and log2(e) enter the exponent's
+// argument by one fused multiply-add and exp2 is one instruction.  The running
+// maximum of a column moves only when a step exceeds it by more than kMaxSlack (in
+// base-2 units): weights may then be as large as 2^kMaxSlack instead of 1, which
+// 32-bit sums and bfloat16 weights hold without loss, and the rescaling of the
+// output - the most expensive vector work of a step - is skipped for the steps in
+// which no column's maximum moved.
 constexpr float kMaxSlack = 6.0f;
 
-template <int D, int HB>
-__device__ __forceinline__ void consume_pair(PrefillState<D, HB>& st, TilePair<D>& pair,
-                                             const bf16x8 (&q_reg)[HB][TilePair<D>::KS], int tile, int lo, int pos,
-                                             int last_key, float scale_log2, int g, bool all_visible) {
-  constexpr int KS = TilePair<D>::KS, CS = TilePair<D>::CS;
-  const int key_a = tile * kTileKeys, key_b = key_a + kTileKeys;
-  // this lane: query column r (position pos, window start lo), keys key_a + 4 g + e and key_b + 4 g + e
-  bool ok_a[4], ok_b[4];
-  if (!all_visible) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int ka = key_a + 4 * g + e, kb = key_b + 4 * g + e;
-      ok_a[e] = ka >= lo && ka <= pos;
-      ok_b[e] = pair.has_b && kb >= lo && kb <= pos;
-    }
-  }
-  float alpha[HB];
-  bf16x8 p[HB];
-  bool moved = false;
-#pragma unroll
-  for (int hb = 0; hb < HB; ++hb) {
-    floatx4 s_a = {0.f, 0.f, 0.f, 0.f}, s_b = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      s_a = ms::mfma_16x16x32(pair.k_a[s], q_reg[hb][s], s_a);
-      s_b = ms::mfma_16x16x32(pair.k_b[s], q_reg[hb][s], s_b);
-    }
-    float tile_max = -INFINITY;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      s_a[e] *= scale_log2;
-      s_b[e] *= scale_log2;
-      if (!all_visible) {
-        s_a[e] = ok_a[e] ? s_a[e] : -INFINITY;
-        s_b[e] = ok_b[e] ? s_b[e] : -INFINITY;
-      }
-      tile_max = fmaxf(tile_max, fmaxf(s_a[e], s_b[e]));
-    }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, ms::kWave));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, ms::kWave));
-    // the maximum moves only when it is exceeded by more than the slack (or is still unset)
-    const bool move = tile_max > st.run_max[hb] + kMaxSlack;
-    const float new_max = move ? tile_max : st.run_max[hb];
-    // a column may have seen no key yet: keep everything at zero
-    const float safe_max = new_max == -INFINITY ? 0.f : new_max;
-    alpha[hb] = move ? ms::fast_exp2(st.run_max[hb] - safe_max) : 1.0f;
-    moved = moved || move;
-    float tile_sum = 0.f;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float pa = ms::fast_exp2(s_a[e] - safe_max);
-      const float pb = ms::fast_exp2(s_b[e] - safe_max);
-      tile_sum += pa + pb;
-      p[hb][e] = static_cast<__bf16>(pa);
-      p[hb][e + 4] = static_cast<__bf16>(pb);
-    }
-    tile_sum += __shfl_xor(tile_sum, 16, ms::kWave);
-    tile_sum += __shfl_xor(tile_sum, 32, ms::kWave);
-    st.run_sum[hb] = st.run_sum[hb] * alpha[hb] + tile_sum;
-    st.run_max[hb] = new_max;
-  }
-
-  // O's rows in this lane are the queries 4 g + e; their alpha lives in lane 4 g + e.
-  if (__any(moved)) {
-#pragma unroll
-    for (int hb = 0; hb < HB; ++hb) {
-      float alpha_row[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) alpha_row[e] = __shfl(alpha[hb], 4 * g + e, ms::kWave);
-#pragma unroll
-      for (int c = 0; c < CS; ++c)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) st.o[hb][c][e] *= alpha_row[e];
-    }
-  }
-  // A stale value (a slot beyond what the sequence has written) times a zero weight
-  // must not become NaN: such slots exist only in the pair that holds the last key.
-  const bool has_stale = key_b + kTileKeys - 1 > last_key;
-#pragma unroll
-  for (int c = 0; c < CS; ++c) {
-    bf16x4 va = pair.v_a[c], vb = pair.v_b[c];
-    if (has_stale) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (key_a + 4 * g + e > last_key) va[e] = static_cast<__bf16>(0.0f);
-        if (key_b + 4 * g + e > last_key) vb[e] = static_cast<__bf16>(0.0f);
-      }
-    }
-    const bf16x8 v = ms::concat(va, vb);
-#pragma unroll
-    for (int hb = 0; hb < HB; ++hb) st.o[hb][c] = ms::mfma_16x16x32(p[hb], v, st.o[hb][c]);
-  }
-}
-
-// Keys and values of one pair of tiles in LDS.  Rows are padded so that the 16 lanes
-// that read 16 different rows spread over the banks.
+// Keys and values of one pair of tiles in LDS.  Rows are padded so that lanes that
+// read different rows spread over the banks.
 template <int D>
 struct alignas(16) PairBuffer {
   static constexpr int kKeyRow = D + 8;      // elements; 16-byte aligned rows
@@ -152,108 +52,205 @@ struct alignas(16) PairBuffer {
 };
 
 // The share of one thread in the cooperative load of a pair: 16-byte chunks, the
-// same number for keys and for values.
-template <int D>
+// same number for keys and for values, tile by tile, so that every load has a base
+// that is the same in all lanes (a scalar register pair) and a 32-bit lane offset
+// that never changes.
+template <int D, int THREADS>
 struct StagedPair {
-  static constexpr int kChunks = 4 * D;                        // of keys; as many of values
-  static constexpr int kPerThread = (kChunks + kBlockThreads - 1) / kBlockThreads;
-  bf16x8 k[kPerThread], v[kPerThread];
+  static constexpr int kTileChunks = 2 * D;                    // of one tile's keys; as many of its values
+  static constexpr int kPerTile = (kTileChunks + THREADS - 1) / THREADS;
+  bf16x8 k[2][kPerTile], v[2][kPerTile];
 };
 
-template <int D>
-__device__ __forceinline__ void stage_load(StagedPair<D>& staged, int tile, int end_tile,
+// chunk of a tile -> element offsets in the cache (from the tile's first key, and from
+// the same offset of the page's value rows) and in the LDS buffer
+template <int D, int THREADS>
+struct ChunkPlace {
+  int key, part;     // keys: (key 0..15, 8 consecutive d)
+  int d, half;       // values: (column d, keys 8 half .. 8 half + 7)
+  __device__ __forceinline__ ChunkPlace(int thread, int j) {
+    // small heads have fewer chunks than threads: the surplus threads repeat the last chunk
+    const int chunk = min(thread + j * THREADS, StagedPair<D, THREADS>::kTileChunks - 1);
+    key = chunk / (D / 8);
+    part = chunk - key * (D / 8);
+    d = chunk >> 1;
+    half = chunk & 1;
+  }
+};
+
+template <int D, int THREADS>
+__device__ __forceinline__ void stage_load(StagedPair<D, THREADS>& staged, int thread, int tile, int end_tile,
                                            const int32_t* __restrict__ table, const bf16* __restrict__ key_pool,
                                            const bf16* __restrict__ value_pool, int num_kv_heads, int kv_head,
                                            int block_size) {
-  // No branch stands around a load: the counters that order the loads of the three
-  // register sets stay exact.  A pair past the end repeats the last one and a missing
-  // second tile repeats the first; what they hold lies beyond the last key and is masked.
+  // No branch stands around a load: the counters that order the loads stay exact.  A
+  // pair past the end repeats the last one and a missing second tile repeats the
+  // first; what they hold lies beyond the last key and is masked.
   tile = min(tile, end_tile - 1);
-  const bool has_b = tile + 1 < end_tile;
-  const int key_a = tile * kTileKeys, key_b = key_a + kTileKeys;
-  const int second_key = has_b ? key_b : key_a;
-  const int64_t page_a = table[key_a / block_size];
-  const int off_a = key_a % block_size;
-  const int64_t page_b = table[second_key / block_size];
-  const int off_b = second_key % block_size;
 #pragma unroll
-  for (int j = 0; j < StagedPair<D>::kPerThread; ++j) {
-    // small heads have fewer chunks than threads: the surplus threads repeat the last chunk
-    const int chunk = min(static_cast<int>(threadIdx.x) + j * kBlockThreads, StagedPair<D>::kChunks - 1);
-    {   // keys: chunk -> (key 0..31, 8 consecutive d)
-      const int key = chunk / (D / 8), part = chunk - key * (D / 8);
-      const bool second = key >= kTileKeys;
-      const int64_t page = second ? page_b : page_a;
-      const int offset = (second ? off_b : off_a) + (key & (kTileKeys - 1));
-      staged.k[j] = ms::load_bf16x8(key_pool + ((page * num_kv_heads + kv_head) * block_size + offset) * D + 8 * part);
-    }
-    {   // values: chunk -> (tile, column d, 8 consecutive keys)
-      const int tile_index = chunk / (2 * D), rest = chunk - tile_index * 2 * D;
-      const int d = rest >> 1, half = rest & 1;
-      const int64_t page = tile_index ? page_b : page_a;
-      const int offset = (tile_index ? off_b : off_a) + 8 * half;
-      staged.v[j] = ms::load_bf16x8(value_pool + ((page * num_kv_heads + kv_head) * D + d) * block_size + offset);
+  for (int side = 0; side < 2; ++side) {
+    const int first_key = (side == 1 && tile + 1 < end_tile ? tile + 1 : tile) * kTileKeys;
+    // the same in every lane: scalar arithmetic
+    const int64_t page = ms::uniform(table[first_key / block_size]);
+    const int offset = first_key % block_size;
+    const int64_t slab = page * num_kv_heads + kv_head;
+    const bf16* keys = key_pool + (slab * block_size + offset) * D;
+    const bf16* values = value_pool + slab * D * block_size + offset;
+#pragma unroll
+    for (int j = 0; j < StagedPair<D, THREADS>::kPerTile; ++j) {
+      const ChunkPlace<D, THREADS> place(thread, j);
+      staged.k[side][j] = ms::load_bf16x8(keys + static_cast<uint32_t>(place.key * D + 8 * place.part));
+      staged.v[side][j] = ms::load_bf16x8(values + static_cast<uint32_t>(place.d * block_size + 8 * place.half));
     }
   }
 }
 
-template <int D>
-__device__ __forceinline__ void stage_store(const StagedPair<D>& staged, PairBuffer<D>& buffer) {
+template <int D, int THREADS>
+__device__ __forceinline__ void stage_store(const StagedPair<D, THREADS>& staged, int thread, PairBuffer<D>& buffer) {
 #pragma unroll
-  for (int j = 0; j < StagedPair<D>::kPerThread; ++j) {
-    const int chunk = min(static_cast<int>(threadIdx.x) + j * kBlockThreads, StagedPair<D>::kChunks - 1);
-    const int key = chunk / (D / 8), part = chunk - key * (D / 8);
-    *reinterpret_cast<bf16x8*>(&buffer.k[key][8 * part]) = staged.k[j];
-    const int tile_index = chunk / (2 * D), rest = chunk - tile_index * 2 * D;
-    *reinterpret_cast<bf16x8*>(&buffer.v[tile_index][rest >> 1][8 * (rest & 1)]) = staged.v[j];
+  for (int side = 0; side < 2; ++side)
+#pragma unroll
+    for (int j = 0; j < StagedPair<D, THREADS>::kPerTile; ++j) {
+      const ChunkPlace<D, THREADS> place(thread, j);
+      *reinterpret_cast<bf16x8*>(&buffer.k[side * kTileKeys + place.key][8 * place.part]) = staged.k[side][j];
+      *reinterpret_cast<bf16x8*>(&buffer.v[side][place.d][8 * place.half]) = staged.v[side][j];
+    }
+}
+
+// What a wave keeps of its 32 columns: this lane holds column `lane & 31`; of the
+// 32 x 32 outputs of a product it holds rows 8 (v / 4) + 4 h + v % 4, h = lane / 32.
+template <int D>
+struct PrefillState {
+  static constexpr int CS = (D + 31) / 32;   // blocks of 32 rows of O^T
+  floatx16 o[CS];
+  float run_max;    // scaled by log2(e) * scale; the same in both lanes of a column
+  float run_sum;    // of this lane's keys only; the two lanes are added at the end
+};
+
+// One pair of key tiles (32 keys from `key0`) against the wave's 32 columns.
+template <int D, bool MASKED>
+__device__ __forceinline__ void consume_pair(PrefillState<D>& st, const PairBuffer<D>& buffer,
+                                             const bf16x8 (&q_reg)[D / 16], int key0, int lo, int pos, int last_key,
+                                             float scale_log2, int h, int column) {
+  constexpr int KS = D / 16, CS = PrefillState<D>::CS;
+  floatx16 s;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+  for (int step = 0; step < KS; ++step) {
+    const bf16x8 keys = *reinterpret_cast<const bf16x8*>(&buffer.k[column][16 * step + 8 * h]);
+    s = ms::mfma_32x32x16(keys, q_reg[step], s);
+  }
+  // register v: key0 + 8 (v / 4) + 4 h + v % 4
+  float tile_max = -INFINITY;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    if (MASKED) {
+      const int key = key0 + 8 * (v / 4) + 4 * h + (v % 4);
+      s[v] = (key >= lo && key <= pos) ? s[v] : -INFINITY;
+    }
+    tile_max = fmaxf(tile_max, s[v]);
+  }
+  tile_max = ms::max_xor32(tile_max) * scale_log2;
+  // the maximum moves only when it is exceeded by more than the slack (or is still unset)
+  const bool move = tile_max > st.run_max + kMaxSlack;
+  const float new_max = move ? tile_max : st.run_max;
+  // a column may have seen no key yet: keep everything at zero
+  const float safe_max = new_max == -INFINITY ? 0.f : new_max;
+  float tile_sum = 0.f;
+  bf16x8 p[2];
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const float weight = ms::fast_exp2(fmaf(s[v], scale_log2, -safe_max));
+    tile_sum += weight;
+    p[v / 8][v % 8] = static_cast<__bf16>(weight);
+  }
+  if (__any(move)) {
+    const float alpha = move ? ms::fast_exp2(st.run_max - safe_max) : 1.0f;
+    st.run_sum *= alpha;
+#pragma unroll
+    for (int c = 0; c < CS; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) st.o[c][v] *= alpha;
+  }
+  st.run_sum += tile_sum;
+  st.run_max = new_max;
+
+  // slot x of the contraction index of half j: key0 + 16 j + 8 (x / 4) + 4 h + x % 4,
+  // for P (registers 8 j + x above) and for V alike
+#pragma unroll
+  for (int c = 0; c < CS; ++c) {
+    const int d = (D % 32 == 0) ? 32 * c + column : min(32 * c + column, D - 1);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      bf16x4 near = *reinterpret_cast<const bf16x4*>(&buffer.v[j][d][4 * h]);
+      bf16x4 far = *reinterpret_cast<const bf16x4*>(&buffer.v[j][d][8 + 4 * h]);
+      if (MASKED) {
+        // A stale value (a slot beyond what the sequence has written) times a zero
+        // weight must not become NaN: such slots exist only in steps that are masked.
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (key0 + 16 * j + 4 * h + e > last_key) near[e] = static_cast<__bf16>(0.0f);
+          if (key0 + 16 * j + 8 + 4 * h + e > last_key) far[e] = static_cast<__bf16>(0.0f);
+        }
+      }
+      st.o[c] = ms::mfma_32x32x16(ms::concat(near, far), p[j], st.o[c]);
+    }
   }
 }
 
-// The pair's operands of this lane, read from LDS.
+// What the second half of a workgroup hands to the first at the end: every register
+// of the state, lane by lane.
 template <int D>
-__device__ __forceinline__ void read_pair(TilePair<D>& pair, const PairBuffer<D>& buffer, bool has_b, int g, int r) {
-  pair.has_b = has_b;
-#pragma unroll
-  for (int s = 0; s < TilePair<D>::KS; ++s) {
-    const int d0 = 32 * s + 8 * g;
-    if (d0 < D) {
-      pair.k_a[s] = *reinterpret_cast<const bf16x8*>(&buffer.k[r][d0]);
-      pair.k_b[s] = *reinterpret_cast<const bf16x8*>(&buffer.k[kTileKeys + r][d0]);
-    } else {
-      pair.k_a[s] = ms::zero_bf16x8();
-      pair.k_b[s] = ms::zero_bf16x8();
-    }
-  }
-#pragma unroll
-  for (int c = 0; c < TilePair<D>::CS; ++c) {
-    pair.v_a[c] = *reinterpret_cast<const bf16x4*>(&buffer.v[0][16 * c + r][4 * g]);
-    pair.v_b[c] = *reinterpret_cast<const bf16x4*>(&buffer.v[1][16 * c + r][4 * g]);
-  }
+struct MergeSlot {
+  float value[PrefillState<D>::CS * 16 + 2][ms::kWave];
+};
+
+constexpr int kMergeWaves = 4;   // slots of one round of the hand-over
+
+template <int D>
+constexpr size_t prefill_lds_bytes() {
+  return 4 * sizeof(PairBuffer<D>) > kMergeWaves * sizeof(MergeSlot<D>) ? 4 * sizeof(PairBuffer<D>)
+                                                                          : kMergeWaves * sizeof(MergeSlot<D>);
 }
 
 template <int D, int HB>
-__global__ __launch_bounds__(kBlockThreads) void attention_prefill_kernel(
+__global__ __launch_bounds__(256 * HB) MS_WAVES_PER_EU(2, 2) void attention_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ key_pool, const bf16* __restrict__ value_pool,
     const int32_t* __restrict__ block_table, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_token, const int32_t* __restrict__ tile_count,
     bf16* __restrict__ out, int num_q_heads, int num_kv_heads, int block_size, int max_blocks, float scale,
     int window) {
-  constexpr int KS = TilePair<D>::KS, CS = TilePair<D>::CS;
-  __shared__ PairBuffer<D> buffers[2];
+  // The workgroup is two halves of 2 HB waves.  Both hold the same 64 HB columns; the
+  // first takes the pairs of key tiles 0, 2, 4, ... of the tile's range and the second
+  // the pairs 1, 3, 5, ...: two waves on every SIMD, one in the matrix cores while the
+  // other is in its softmax, and half as many steps for the longest tile.  Each half
+  // loads its own pairs into its own LDS buffers; at the end the second hands its
+  // state to the first through LDS.
+  constexpr int HALF_THREADS = 128 * HB;
+  constexpr int HALF_WAVES = 2 * HB;
+  constexpr int KS = D / 16, CS = PrefillState<D>::CS;
+  __shared__ __align__(16) unsigned char lds[prefill_lds_bytes<D>()];
+  PairBuffer<D>* buffers = reinterpret_cast<PairBuffer<D>*>(lds);        // [parity][half]
+  MergeSlot<D>* slots = reinterpret_cast<MergeSlot<D>*>(lds);
 
   const int lane = threadIdx.x & 63;
-  const int wave = ms::uniform(threadIdx.x >> 6);   // the same in all lanes: kept in a scalar register
-  const int g = lane >> 4;
-  const int r = lane & 15;
+  const int wave_of_group = ms::uniform(threadIdx.x >> 6);   // the same in all lanes: kept in a scalar register
+  const int half_id = wave_of_group / HALF_WAVES;
+  const int wave = wave_of_group - half_id * HALF_WAVES;
+  const int thread = threadIdx.x - half_id * HALF_THREADS;
+  const int h = lane >> 5;
+  const int column = lane & 31;
 
-  const int tile_index = blockIdx.x;
+  // long tiles (late in their sequences) first
+  const int tile_index = gridDim.x - 1 - blockIdx.x;
   const int group = num_q_heads / num_kv_heads;
   const int head_blocks = (group + HB - 1) / HB;
   const int kv_head = blockIdx.y / head_blocks;
   const int head0 = kv_head * group + (blockIdx.y - kv_head * head_blocks) * HB;
   const int heads_here = min(HB, kv_head * group + group - head0);
 
-  // The workgroup's tile: up to 64 consecutive tokens of one sequence; wave w owns tokens 16 w .. 16 w + 15.
+  // The workgroup's tile: up to 64 consecutive tokens of one sequence.
   const int token0 = tile_token[tile_index];
   const int count = tile_count[tile_index];
   const int32_t* table = block_table + static_cast<int64_t>(tile_seq[tile_index]) * max_blocks;
@@ -263,82 +260,111 @@ __global__ __launch_bounds__(kBlockThreads) void attention_prefill_kernel(
   const int t0 = first_lo / kTileKeys;
   const int t1 = last_key / kTileKeys + 1;
 
-  const int my_count = max(0, min(kQueryTile, count - kQueryTile * wave));
-  // query column r of this lane; a column past the wave's tokens repeats the last one and is not stored
-  const int64_t my_token = token0 + (my_count > 0 ? kQueryTile * wave + min(r, my_count - 1) : 0);
+  // The wave's columns: with one head 32 tokens, else 16 tokens of two heads.
+  const int wave_token = HB == 1 ? kWaveColumns * wave : 16 * wave;
+  const int wave_span = HB == 1 ? kWaveColumns : 16;
+  const int my_head = HB == 1 ? 0 : (column >> 4);
+  const int my_local = HB == 1 ? column : (column & 15);
+  const int my_count = max(0, min(wave_span, count - wave_token));
+  // a column past the wave's tokens repeats the last one and is not stored
+  const int64_t my_token = token0 + (my_count > 0 ? wave_token + min(my_local, my_count - 1) : 0);
+  const bool head_live = my_head < heads_here;
   const int pos = positions[my_token];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int wave_last_key = my_count > 0 ? first_pos + kQueryTile * wave + my_count - 1 : -1;
-  const int wave_first_pos = first_pos + kQueryTile * wave;
+  const int wave_first_pos = first_pos + wave_token;
+  const int wave_last_key = my_count > 0 ? wave_first_pos + my_count - 1 : -1;
   const int wave_first_lo = (window > 0 && wave_first_pos - window + 1 > 0) ? wave_first_pos - window + 1 : 0;
   const int wave_last_lo = (window > 0 && wave_last_key - window + 1 > 0) ? wave_last_key - window + 1 : 0;
   const float scale_log2 = scale * 1.4426950408889634f;
 
-  bf16x8 q_reg[HB][KS];
+  bf16x8 q_reg[KS];
 #pragma unroll
-  for (int hb = 0; hb < HB; ++hb)
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int d0 = 32 * s + 8 * g;
-      q_reg[hb][s] = (hb < heads_here && d0 < D) ? ms::load_bf16x8(q + (my_token * num_q_heads + head0 + hb) * D + d0)
-                                                  : ms::zero_bf16x8();
-    }
+  for (int step = 0; step < KS; ++step)
+    q_reg[step] = head_live ? ms::load_bf16x8(q + (my_token * num_q_heads + head0 + my_head) * D + 16 * step + 8 * h)
+                            : ms::zero_bf16x8();
 
-  PrefillState<D, HB> st;
+  PrefillState<D> st;
 #pragma unroll
-  for (int hb = 0; hb < HB; ++hb) {
+  for (int c = 0; c < CS; ++c)
 #pragma unroll
-    for (int c = 0; c < CS; ++c) st.o[hb][c] = floatx4{0.f, 0.f, 0.f, 0.f};
-    st.run_max[hb] = -INFINITY;
-    st.run_sum[hb] = 0.f;
-  }
+    for (int v = 0; v < 16; ++v) st.o[c][v] = 0.f;
+  st.run_max = -INFINITY;
+  st.run_sum = 0.f;
 
-  // Three pairs in flight in registers, two buffers in LDS: the loads of pair i + 3
-  // are issued before pair i is consumed.  The loop is unrolled by hand over the three
-  // register sets: a copy from one set to another would have to wait for its loads.
-  StagedPair<D> ring0, ring1, ring2;
-  stage_load<D>(ring0, t0, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size);
-  stage_load<D>(ring1, t0 + 2, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size);
-  stage_load<D>(ring2, t0 + 4, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size);
+  // One pair in flight in registers, two buffers in LDS for each half: the loads of
+  // the half's next pair are issued before the current one is consumed.  No branch
+  // stands between a load and its use; both halves make the same number of rounds.
+  StagedPair<D, HALF_THREADS> staged;
+  stage_load<D, HALF_THREADS>(staged, thread, t0 + 2 * half_id, t1, table, key_pool, value_pool, num_kv_heads, kv_head,
+                              block_size);
   int parity = 0;
-  auto step = [&](StagedPair<D>& staged, int t) {
-    PairBuffer<D>& buffer = buffers[parity];
-    stage_store<D>(staged, buffer);
-    stage_load<D>(staged, t + 6, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size);
-    __syncthreads();    // the pair is in LDS; every wave is done with the other buffer's previous content
+  for (int round_tile = t0; round_tile < t1; round_tile += 4) {
+    const int t = round_tile + 2 * half_id;
+    PairBuffer<D>& buffer = buffers[2 * parity + half_id];
+    stage_store<D, HALF_THREADS>(staged, thread, buffer);
+    stage_load<D, HALF_THREADS>(staged, thread, t + 4, t1, table, key_pool, value_pool, num_kv_heads, kv_head,
+                                block_size);
+    __syncthreads();    // the pair is in LDS; every wave is done with the other buffers' previous content
     if (t < t1 && t * kTileKeys <= wave_last_key && (t + 2) * kTileKeys > wave_first_lo) {
-      TilePair<D> pair;
-      read_pair<D>(pair, buffer, t + 1 < t1, g, r);
-      // every key of the pair visible to every query of the wave: no masks
+      // every key of the pair visible to every column of the wave: no masks
       const bool all_visible = (t + 2) * kTileKeys - 1 <= wave_first_pos && t * kTileKeys >= wave_last_lo;
-      consume_pair<D, HB>(st, pair, q_reg, t, lo, pos, last_key, scale_log2, g, all_visible);
+      if (all_visible) {
+        consume_pair<D, false>(st, buffer, q_reg, t * kTileKeys, lo, pos, last_key, scale_log2, h, column);
+      } else {
+        consume_pair<D, true>(st, buffer, q_reg, t * kTileKeys, lo, pos, last_key, scale_log2, h, column);
+      }
     }
     parity ^= 1;
-  };
-  // Straight-line body (three steps, no exit between them): steps past the end load
-  // and store a repeated pair and consume nothing.
-  for (int t = t0; t < t1; t += 6) {
-    step(ring0, t);
-    step(ring1, t + 2);
-    step(ring2, t + 4);
   }
 
-  // this lane: output rows = queries 4 g + e, column d = 16 c + r; the row's sum lives in lane 4 g + e
+  // The second half hands over; the two states of a column are joined as two steps
+  // of the online softmax are.
+#pragma unroll 1
+  for (int first_wave = 0; first_wave < HALF_WAVES; first_wave += kMergeWaves) {
+    __syncthreads();    // everybody is done with what the memory held before
+    const bool in_round = wave >= first_wave && wave < first_wave + kMergeWaves;
+    MergeSlot<D>& slot = slots[wave - first_wave];
+    if (in_round && half_id == 1) {
 #pragma unroll
-  for (int hb = 0; hb < HB; ++hb) {
-    float inv_row[4];
+      for (int c = 0; c < CS; ++c)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) inv_row[e] = 1.0f / __shfl(st.run_sum[hb], 4 * g + e, ms::kWave);
-    if (hb >= heads_here) continue;
+        for (int v = 0; v < 16; ++v) slot.value[16 * c + v][lane] = st.o[c][v];
+      slot.value[16 * CS][lane] = st.run_max;
+      slot.value[16 * CS + 1][lane] = st.run_sum;
+    }
+    __syncthreads();
+    if (in_round && half_id == 0) {
+      const float other_max = slot.value[16 * CS][lane];
+      const float joint = fmaxf(st.run_max, other_max);
+      // a half may have seen no key of a column: its share is zero
+      const float mine = st.run_max == -INFINITY ? 0.f : ms::fast_exp2(st.run_max - joint);
+      const float theirs = other_max == -INFINITY ? 0.f : ms::fast_exp2(other_max - joint);
+      st.run_sum = st.run_sum * mine + slot.value[16 * CS + 1][lane] * theirs;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int row = 4 * g + e;
-      if (row >= my_count) continue;
-      bf16* dst = out + ((static_cast<int64_t>(token0) + kQueryTile * wave + row) * num_q_heads + head0 + hb) * D;
+      for (int c = 0; c < CS; ++c)
 #pragma unroll
-      for (int c = 0; c < CS; ++c) dst[16 * c + r] = ms::from_float<bf16>(st.o[hb][c][e] * inv_row[e]);
+        for (int v = 0; v < 16; ++v) st.o[c][v] = st.o[c][v] * mine + slot.value[16 * c + v][lane] * theirs;
     }
   }
+  if (half_id == 1) return;
+
+  // this lane: column's rows d = 32 c + 8 (v / 4) + 4 h + v % 4; its sum is shared with lane + 32
+  const float total = st.run_sum + __shfl_xor(st.run_sum, 32, ms::kWave);
+  const float inv = 1.0f / total;
+  if (!head_live || my_local >= my_count) return;
+  bf16* dst = out + (my_token * num_q_heads + head0 + my_head) * D;
+#pragma unroll
+  for (int c = 0; c < CS; ++c)
+#pragma unroll
+    for (int quad = 0; quad < 4; ++quad) {
+      const int d = 32 * c + 8 * quad + 4 * h;
+      if (D % 32 != 0 && d >= D) continue;
+      const uint32_t low = static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad] * inv)) |
+                           (static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 1] * inv)) << 16);
+      const uint32_t high = static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 2] * inv)) |
+                            (static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 3] * inv)) << 16);
+      *reinterpret_cast<uint2*>(dst + d) = make_uint2(low, high);
+    }
 }
 
 template <int D, int HB>
@@ -348,7 +374,7 @@ void launch_prefill(const void* q, const void* key_pool, const void* value_pool,
                     float scale, int window, hipStream_t stream) {
   const int head_blocks = (num_q_heads / num_kv_heads + HB - 1) / HB;
   const dim3 grid(num_tiles, num_kv_heads * head_blocks);
-  hipLaunchKernelGGL((attention_prefill_kernel<D, HB>), grid, dim3(kBlockThreads), 0, stream, static_cast<const bf16*>(q),
+  hipLaunchKernelGGL((attention_prefill_kernel<D, HB>), grid, dim3(256 * HB), 0, stream, static_cast<const bf16*>(q),
                      static_cast<const bf16*>(key_pool), static_cast<const bf16*>(value_pool),
                      static_cast<const int32_t*>(block_table), static_cast<const int32_t*>(positions),
                      static_cast<const int32_t*>(tile_seq), static_cast<const int32_t*>(tile_token),
@@ -365,11 +391,8 @@ void launch_prefill_heads(int hb, const void* q, const void* key_pool, const voi
   if (hb == 1) {
     launch_prefill<D, 1>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
                          num_tiles, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, stream);
-  } else if (hb == 2) {
-    launch_prefill<D, 2>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
-                         num_tiles, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, stream);
   } else {
-    launch_prefill<D, 4>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
+    launch_prefill<D, 2>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
                          num_tiles, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, stream);
   }
 }
@@ -401,7 +424,7 @@ extern "C" int ms_attention_prefill(const void* q, const void* key_pool, const v
              head_dim, block_size);
   MS_REQUIRE(max_blocks > 0 && window >= 0, "attention_prefill: bad table width or window");
   const int group = num_q_heads / num_kv_heads;
-  const int hb = group >= 4 ? 4 : (group >= 2 ? 2 : 1);   // query heads of one workgroup
+  const int hb = group >= 2 ? 2 : 1;   // query heads of one workgroup
   MS_REQUIRE(num_kv_heads * ((group + hb - 1) / hb) <= 65535, "attention_prefill: too many heads");
 #define MS_PREFILL_CASE(DIM)                                                                                       \
   case DIM:                                                                                                        \
