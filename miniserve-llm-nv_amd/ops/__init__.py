@@ -56,7 +56,15 @@ def _ptr(tensor: torch.Tensor | None) -> int | None:
     return None if tensor is None else tensor.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """The current stream of the current device as a raw handle (the short way where
+    torch offers it: this is called once per kernel)."""
+
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -311,6 +319,39 @@ _EPILOGUE_BF16, _EPILOGUE_F32, _EPILOGUE_ADD_F32, _EPILOGUE_SILU_MUL = 0, 1, 2, 
 SKINNY_MAX_ROWS = 16
 
 
+_GEMM_WORKSPACE_BYTES = 64 << 20
+_gemm_workspaces: dict[int, torch.Tensor] = {}
+_gemm_library_opened = False
+
+
+def _loaded_hipblaslt() -> str:
+    """Path of the hipBLASLt that this process has loaded (torch's): the product for
+    many rows binds to that copy, not to a second one."""
+
+    with open("/proc/self/maps") as maps:
+        for line in maps:
+            path = line.rsplit(" ", 1)[-1].strip()
+            if "libhipblaslt" in path.rsplit("/", 1)[-1]:
+                return path
+    raise KernelError("no hipBLASLt is loaded in this process (torch on ROCm brings it).")
+
+
+def _library_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
+    """``out (+)= x @ weight^T`` through hipBLASLt; bfloat16 in, bfloat16 or float32 out."""
+
+    global _gemm_library_opened
+    if not _gemm_library_opened:
+        call("ms_gemm_library_open", _loaded_hipblaslt().encode())
+        _gemm_library_opened = True
+    index = x.device.index if x.device.index is not None else torch.cuda.current_device()
+    workspace = _gemm_workspaces.get(index)
+    if workspace is None:
+        workspace = _gemm_workspaces[index] = torch.empty(_GEMM_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
+    m, k = x.shape
+    call("ms_gemm_library", _ptr(x), _ptr(weight), _ptr(out), m, weight.shape[0], k, int(out.dtype == torch.float32),
+         int(accumulate), _ptr(workspace), _GEMM_WORKSPACE_BYTES, _stream())
+
+
 def _use_skinny(m: int, n: int, k: int, epilogue: int) -> bool:
     return m <= SKINNY_MAX_ROWS and bool(load().ms_gemm_skinny_supported(m, n, k, epilogue))
 
@@ -335,7 +376,7 @@ def linear(
     float32: this library's FMA kernel (true 32-bit; row results do not depend on
     M).  bfloat16 with at most ``SKINNY_MAX_ROWS`` rows: this library's matrix-core
     kernel that streams the weights once; more rows: the library matrix product
-    (hipBLASLt through torch), both with 32-bit accumulation.  ``accumulate_into`` (float32
+    (hipBLASLt, the copy that torch has loaded), both with 32-bit accumulation.  ``accumulate_into`` (float32
     ``[M, N]``) receives ``+=`` and is returned; ``out_float32`` returns the
     32-bit sums without a rounding to bfloat16 in between."""
 
@@ -359,19 +400,19 @@ def linear(
         out = torch.empty((m, n), dtype=torch.float32 if out_float32 else torch.bfloat16, device=x.device)
         _skinny(x, weight, _EPILOGUE_F32 if out_float32 else _EPILOGUE_BF16, out)
         return out
-    out = torch.mm(x, weight.t())
     if accumulate_into is not None:
-        residual_add(accumulate_into, out)
+        _library_product(x, weight, accumulate_into, True)
         return accumulate_into
-    return out.float() if out_float32 else out
+    out = torch.empty((m, n), dtype=torch.float32 if out_float32 else torch.bfloat16, device=x.device)
+    _library_product(x, weight, out, False)
+    return out
 
 
 def can_accumulate(rows: int, weight: torch.Tensor) -> bool:
     """Whether ``linear(..., accumulate_into=...)`` adds in the product's own epilogue
     (else it would cost a kernel more than handing the sum to the next norm)."""
 
-    n, k = weight.shape
-    return weight.dtype == torch.float32 or _use_skinny(rows, n, k, _EPILOGUE_ADD_F32)
+    return weight.dtype in (torch.float32, torch.bfloat16)
 
 
 def can_fuse_norm(rows: int, weight: torch.Tensor, *, gated: bool = False) -> bool:

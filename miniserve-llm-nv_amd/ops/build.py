@@ -122,7 +122,7 @@ def build(*, force: bool = True, jobs: int | None = None) -> Path:
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objects = list(pool.map(compile_one, files))
     partial = target.with_suffix(f".tmp{os.getpid()}")
-    command = [hipcc, f"--offload-arch={OFFLOAD_ARCH}", "-shared", "-fPIC", "-o", str(partial), *map(str, objects)]
+    command = [hipcc, f"--offload-arch={OFFLOAD_ARCH}", "-shared", "-fPIC", "-o", str(partial), *map(str, objects), "-ldl"]
     result = subprocess.run(command, capture_output=True, text=True)
     if result.returncode != 0:
         raise RuntimeError(f"hipcc failed to link {LIBRARY_NAME}:\n{result.stderr}")

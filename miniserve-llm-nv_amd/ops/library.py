@@ -9,7 +9,7 @@ from __future__ import annotations
 import ctypes
 import sys
 import threading
-from ctypes import c_char_p, c_float, c_int, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
 
 from . import build as _build
 
@@ -36,6 +36,8 @@ _SIGNATURES: dict[str, list] = {
     "ms_gemm_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
     "ms_gemm_skinny_supported": [_I, _I, _I, _I],
     "ms_gemm_skinny_normed": [_P, _P, _F, _P, _P, _I, _I, _I, _I, _P],
+    "ms_gemm_library_open": [c_char_p],
+    "ms_gemm_library": [_P, _P, _P, _I, _I, _I, _I, _I, _P, c_size_t, _P],
     "ms_silu_mul": [_P, _P, _I, _I, _I, _P],
     "ms_sample_rows": [_P, _P, _P, _P, _P, _P, _I, _I, _P],
     "ms_argmax_rows": [_P, _P, _P, _P, _I, _I, _I, _P],
