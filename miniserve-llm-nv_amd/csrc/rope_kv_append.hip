@@ -154,11 +154,6 @@ __device__ __forceinline__ void store8(ms::bf16* dst, const float in[8]) {
   *reinterpret_cast<uint4*>(dst) = make_uint4(words[0], words[1], words[2], words[3]);
 }
 
-__device__ __forceinline__ void store8(float* dst, const float in[8]) {
-  *reinterpret_cast<float4*>(dst) = make_float4(in[0], in[1], in[2], in[3]);
-  *reinterpret_cast<float4*>(dst + 4) = make_float4(in[4], in[5], in[6], in[7]);
-}
-
 template <typename T>
 __global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kernel(
     const T* __restrict__ packed, const T* __restrict__ q_weight, const T* __restrict__ k_weight,
@@ -354,21 +349,18 @@ extern "C" int ms_qk_norm_rope_append(const void* packed, const void* q_weight, 
   }
   MS_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "qk_norm_rope_append: rotation needs both tables");
   MS_REQUIRE(num_q_heads + 2 * num_kv_heads <= 65535, "qk_norm_rope_append: too many heads");
-  // 16 bytes a lane where the head size is a multiple of 16 and every operand is
-  // aligned to 16 bytes (null operands are),
-  // for more tokens than two tiles; few tokens are quicker with a wave to each row
-  const bool tiled = head_dim % 16 == 0 && head_dim <= 16 * kTiledThreads &&
+  // bfloat16, 16 bytes a lane, where the head size is a multiple of 16 and every operand
+  // is aligned to 16 bytes (null operands are), for more tokens than two tiles; few
+  // tokens are quicker with a wave to each row.  32-bit storage always takes the wave
+  // to each row: the order of its sums never depends on the number of tokens, so a
+  // position's result is the same to the bit however the tokens are cut into steps.
+  const bool tiled = dtype == MS_BF16 && head_dim % 16 == 0 && head_dim <= 16 * kTiledThreads &&
                      num_tokens > 2 * (kTiledThreads / (head_dim / 16)) && aligned16(packed) &&
                      aligned16(q_weight) && aligned16(k_weight) && aligned16(cos_table) && aligned16(sin_table) &&
                      aligned16(q_out) && aligned16(key_pool) && aligned16(value_pool);
-  if (tiled && (dtype == MS_F32 || dtype == MS_BF16)) {
-    if (dtype == MS_F32) {
-      launch_tiled<float>(packed, q_weight, k_weight, cos_table, sin_table, slot_mapping, q_out, key_pool,
-                          value_pool, num_tokens, num_q_heads, num_kv_heads, head_dim, block_size, eps, stream);
-    } else {
-      launch_tiled<ms::bf16>(packed, q_weight, k_weight, cos_table, sin_table, slot_mapping, q_out, key_pool,
-                             value_pool, num_tokens, num_q_heads, num_kv_heads, head_dim, block_size, eps, stream);
-    }
+  if (tiled) {
+    launch_tiled<ms::bf16>(packed, q_weight, k_weight, cos_table, sin_table, slot_mapping, q_out, key_pool,
+                           value_pool, num_tokens, num_q_heads, num_kv_heads, head_dim, block_size, eps, stream);
     MS_CHECK_LAUNCH("qk_norm_rope_append");
     return 0;
   }

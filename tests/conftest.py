@@ -30,8 +30,8 @@ def pytest_collection_modifyitems(config, items):
 
 @pytest.fixture(scope="session")
 def model_folders(tmp_path_factory):
-    """Model folders of the two tiny configurations, random weights stored in
-    float32, in a temporary place: ``{"a": (folder, block_size), "b": ...}``."""
+    """Model folders of the tiny configurations, random weights stored in
+    float32, in a temporary place: ``{"a": (folder, block_size), "b": ..., "c": ...}``."""
 
     from helpers import TINY, make_model_folder
 

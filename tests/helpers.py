@@ -1,4 +1,4 @@
-"""Shared test material: the two tiny configurations, model folders with random
+"""Shared test material: the tiny configurations, model folders with random
 weights in a temporary place, and replay shapes."""
 
 from __future__ import annotations
@@ -64,7 +64,33 @@ def tiny_b() -> dict:
     }
 
 
-TINY = {"a": (tiny_a, 16), "b": (tiny_b, 8)}
+def tiny_c() -> dict:
+    """A third one with wider heads and larger pages, and a group of three query heads
+    to a kv head: 2 layers, hidden 80,
+    6 q heads, 2 kv heads (group 3), head 64, inter 176, vocab 300, theta 5e5, eps
+    1e-6, untied head; pages of 32."""
+
+    return {
+        "architectures": ["Qwen3ForCausalLM"],
+        "model_type": "qwen3",
+        "hidden_size": 80,
+        "intermediate_size": 176,
+        "num_hidden_layers": 2,
+        "num_attention_heads": 6,
+        "num_key_value_heads": 2,
+        "head_dim": 64,
+        "vocab_size": 300,
+        "max_position_embeddings": 1024,
+        "rms_norm_eps": 1e-6,
+        "rope_theta": 500000.0,
+        "tie_word_embeddings": False,
+        "hidden_act": "silu",
+        "attention_bias": False,
+        "attention_dropout": 0.0,
+    }
+
+
+TINY = {"a": (tiny_a, 16), "b": (tiny_b, 8), "c": (tiny_c, 32)}
 
 
 def make_model_folder(folder: Path, config_dict: dict, seed: int, store_dtype: str = "float32") -> Path:

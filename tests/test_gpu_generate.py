@@ -57,6 +57,30 @@ def test_greedy_generation_tiny_a(dtype, model_folders):
     assert cache.live_requests() == () and cache.capacity().free_blocks == (16,)
 
 
+def test_greedy_generation_with_wide_heads_through_recorded_steps(model_folders):
+    """Tiny C has heads of 64 and pages of 32: in bfloat16 every matrix-core kernel
+    serves it, and its decode steps are replayed as recorded graphs.  Prompts of
+    changing length so that batches of 1 to 4 are decoded."""
+
+    from miniserve_amd.engine import SamplingParams
+    from miniserve_amd.entrypoint import LLM
+
+    folder, block = model_folders["c"]
+    config, weights = read_config(folder), rounded(read_weights(folder), "bfloat16")
+    prompts = [random_tokens(n, config["vocab_size"], 400 + n) for n in (3, 40, 65, 131)]
+    llm = LLM(str(folder), dtype="bfloat16", kv_block_size=block, num_kv_blocks=24, max_num_seqs=4)
+    assert llm.runner.engine_config.decode_graphs
+    limits = [SamplingParams(max_new_tokens=n) for n in (40, 9, 33, 20)]
+    got = llm.generate(prompts, limits)
+    assert [len(tokens) for tokens in got] == [40, 9, 33, 20]
+    for tokens, prompt in zip(got, prompts):
+        check_greedy(tokens, prompt, weights, config, "bfloat16")
+    eager = LLM(str(folder), dtype="bfloat16", kv_block_size=block, num_kv_blocks=24, max_num_seqs=4, decode_graphs=False)
+    for tokens, prompt in zip(eager.generate(prompts, limits), prompts):     # the same steps, launched one by one
+        check_greedy(tokens, prompt, weights, config, "bfloat16")
+    assert llm.runner.cache.live_requests() == ()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_chunked_prefill_mixed_with_decode_tiny_b(dtype, model_folders):
     """BASELINE configuration Tiny B: prompts of 1, 9, 24 and 40 tokens, portions of

@@ -1,7 +1,7 @@
 """Trace replay on the GPU against the plain implementation: each request alone and
 whole; most of it in one step and the last 32 tokens one by one; in portions of
 changing size; mixed with other requests on so few pages that they are used
-again - in 32-bit and in bfloat16, for both tiny configurations."""
+again - in 32-bit and in bfloat16, for every tiny configuration."""
 
 from __future__ import annotations
 
@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 # rounding of a few hundred float32 operations.  bfloat16: activations carry 8
 # bits, the logits themselves are rounded to bfloat16 (2^-9 relative).
 TOLERANCE = {"float32": 2e-5, "bfloat16": 2.5e-2}
-LENGTHS = {"a": (45, 70, 100, 33, 18, 64, 81), "b": (41, 96, 64, 57, 9, 80)}
+LENGTHS = {"a": (45, 70, 100, 33, 18, 64, 81), "b": (41, 96, 64, 57, 9, 80), "c": (150, 37, 66, 90, 129, 40)}
 
 
 def reference_weights(weights, dtype):
@@ -85,7 +85,7 @@ def run_and_compare(runner, steps, requests, logits, vocab, tolerance, tmp_path)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "c"])
 def test_replay_shapes(name, dtype, model_folders, oracle, tmp_path):
     folder, block_size = model_folders[name]
     requests, logits, config = oracle(name, dtype)
