@@ -8,6 +8,8 @@ where this runs one for all).
 
 from __future__ import annotations
 
+import gc
+import weakref
 from pathlib import Path
 from typing import Sequence
 
@@ -40,7 +42,9 @@ class DecodeGraph:
 
     def __init__(self, runner: "ModelRunner", batch: int) -> None:
         self.batch = batch
-        self.runner = runner
+        # no strong reference back: a runner that is dropped goes at once, with its graphs,
+        # and not at some later collection of cycles
+        self._runner = weakref.ref(runner)
         groups = len(runner.cache.layout.groups)
         width = runner.max_blocks_per_seq
         sizes = [("token_ids", batch), ("positions", batch), ("seq_of_token", batch), ("query_start", batch + 1),
@@ -98,9 +102,10 @@ class DecodeGraph:
         put("context_lens", [meta.after for meta in metas])
         put("state_slots", [meta.state_slot for meta in metas])
         put("logit_rows", range(batch))
-        block_size = self.runner.block_size
-        for group in range(len(self.runner.cache.layout.groups)):
-            pool_pages = self.runner.cache.num_blocks[group]
+        runner = self._runner()
+        block_size = runner.block_size
+        for group in range(len(runner.cache.layout.groups)):
+            pool_pages = runner.cache.num_blocks[group]
             slots = []
             start, _ = offsets[f"table{group}"]
             for row, meta in enumerate(metas):
@@ -120,16 +125,27 @@ class DecodeGraph:
 
         self._fill(entries, reservation)
         self.meta.copy_(self.host, non_blocking=True)
-        model, views = self.runner.model, self.runner._call_views
+        runner = self._runner()
+        model, views = runner.model, runner._call_views
         if self.graph is None:
             # Once eagerly, so that libraries set themselves up outside the recording;
             # running the same step twice writes the same cache slots twice.
             model.forward(self.ctx, views, self.rows)
-            torch.cuda.synchronize(self.runner.device)
+            torch.cuda.synchronize(runner.device)
             self.ctx.scratch.clear()        # what the step shares between layers is made again inside the recording
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self.runner._graph_pool):
-                self.logits = model.forward(self.ctx, views, self.rows)
+            # No collection of cycles while the stream records: it may free what earlier
+            # owners left behind (pinned memory, other graphs), and a free is not allowed
+            # inside a recording - the process would abort.
+            collecting = gc.isenabled()
+            gc.collect()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph, pool=runner._graph_pool):
+                    self.logits = model.forward(self.ctx, views, self.rows)
+            finally:
+                if collecting:
+                    gc.enable()
             self.graph = graph
         self.graph.replay()
         self.replays += 1

@@ -279,3 +279,56 @@ def test_decode_graphs_replay_like_eager_steps(dtype, model_folders):
     both({"b": 1})
     assert runners[0].graph_steps == 33 and runners[1].graph_steps == 0
     assert sorted(runners[0]._decode_graphs) == [1, 2, 3, 4]
+
+
+def test_a_dropped_runner_is_freed_at_once_and_recording_survives_a_collection(model_folders):
+    """A runner's recorded steps hold no reference back to it: dropping the runner frees
+    it, its graphs and its pinned memory without waiting for a collection of cycles -
+    which, falling into a later recording, would free them there and abort the process.
+    And a recording collects what garbage there is before it starts and keeps the
+    collector off while the stream records."""
+
+    import gc
+    import weakref
+
+    from miniserve_amd.config import EngineConfig
+    from miniserve_amd.engine import ModelRunner, StepEntry
+
+    folder, block = model_folders["a"]
+    config = read_config(folder)
+
+    def make():
+        return ModelRunner.from_folder(folder, EngineConfig(dtype="bfloat16", kv_block_size=block, num_kv_blocks=16, max_num_seqs=2))
+
+    def decode_once(runner):
+        runner.admit("x")
+        runner.step([StepEntry("x", tuple(random_tokens(5, config["vocab_size"], 1)), ())])
+        return runner.step([StepEntry("x", (3,), (0,))]).clone()      # recorded, then replayed
+
+    first = make()
+    expected = decode_once(first)
+    assert first.graph_steps == 1
+    gone = weakref.ref(first)
+    graph_gone = weakref.ref(first._decode_graphs[1])
+    del first
+    assert gone() is None and graph_gone() is None
+
+    # cyclic garbage that owns pinned and device memory, left for the collector
+    class Knot:
+        def __init__(self):
+            self.me = self
+            self.pinned = torch.zeros(1024).pin_memory()
+            self.device = torch.zeros(1024, device=DEVICE)
+
+    was_enabled = gc.isenabled()
+    gc.collect()
+    gc.disable()
+    try:
+        knot = weakref.ref(Knot())
+        gc.enable()                                   # the collector may run from here on
+        second = make()
+        got = decode_once(second)                     # records a graph with the knot lying about
+    finally:
+        gc.enable() if was_enabled else gc.disable()
+    assert knot() is None and gc.isenabled() == was_enabled
+    assert torch.equal(got, expected)
