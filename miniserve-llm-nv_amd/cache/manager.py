@@ -233,13 +233,19 @@ class CacheManager:
                     missing = table.required_blocks(item.end) - len(table.physical_block_ids)
                     new_pages = allocator.allocate(max(missing, 0))
                     taken.append((index, new_pages))
-                    tentative = table.physical_block_ids + new_pages
-                    slots = []
-                    for position in range(item.start, item.end):
-                        logical, offset = divmod(position, self.block_size)
-                        slots.append(tentative[logical] * self.block_size + offset)
-                    meta.block_tables.append(tuple(tentative))
-                    meta.slot_mappings.append(tuple(slots))
+                    # without a new page the step reads the table's own snapshot, made once per change
+                    tentative = tuple(table.physical_block_ids + new_pages) if new_pages else table.snapshot()
+                    block_size = self.block_size
+                    if item.end == item.start + 1:
+                        logical, offset = divmod(item.start, block_size)
+                        slots = (tentative[logical] * block_size + offset,)
+                    else:
+                        slots = tuple(
+                            tentative[position // block_size] * block_size + position % block_size
+                            for position in range(item.start, item.end)
+                        )
+                    meta.block_tables.append(tentative)
+                    meta.slot_mappings.append(slots)
                     meta.new_pages.append(new_pages)
                 reservation.sequences.append(meta)
         except OutOfPagesError:
@@ -296,7 +302,7 @@ class CacheManager:
             free_slots=len(self._free_slots),
             total_slots=self.max_num_seqs,
             held_blocks={
-                request_id: tuple(len(table.live_pages()) for table in live.tables)
+                request_id: tuple(table.live_count() for table in live.tables)
                 for request_id, live in self._live.items()
             },
         )

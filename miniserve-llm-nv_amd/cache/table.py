@@ -18,6 +18,7 @@ class BlockTable:
     block_size: int
     physical_block_ids: list[int] = field(default_factory=list)
     first_live: int = 0          # logical index of the first page still held
+    _snapshot: tuple[int, ...] | None = field(default=None, repr=False, compare=False)   # kept until the table changes
 
     def __post_init__(self) -> None:
         if not _is_int(self.block_size) or self.block_size <= 0:
@@ -33,11 +34,14 @@ class BlockTable:
         return (token_count + self.block_size - 1) // self.block_size
 
     def append_blocks(self, block_ids: list[int]) -> None:
+        if isinstance(block_ids, list) and not block_ids:
+            return               # most steps of a decoding request bring no new page
         if not isinstance(block_ids, list) or any(not _is_int(page) or page < 0 for page in block_ids):
             raise ValueError("Appended physical block IDs must be a list of non-negative integers.")
         if len(block_ids) != len(set(block_ids)) or set(block_ids) & set(self.live_pages()):
             raise ValueError("Appended physical block IDs must be unique.")
         self.physical_block_ids.extend(block_ids)
+        self._snapshot = None
 
     def resolve(self, token_position: int) -> tuple[int, int, int]:
         """``(logical page, physical page, offset)`` of a position."""
@@ -59,6 +63,9 @@ class BlockTable:
     def live_pages(self) -> list[int]:
         return self.physical_block_ids[self.first_live :]
 
+    def live_count(self) -> int:
+        return len(self.physical_block_ids) - self.first_live
+
     def give_back_before(self, token_position: int) -> list[int]:
         """Pages whose every position is below ``token_position`` leave the table."""
 
@@ -68,7 +75,13 @@ class BlockTable:
             returned.append(self.physical_block_ids[logical])
             self.physical_block_ids[logical] = RETURNED
         self.first_live = max(self.first_live, limit)
+        if returned:
+            self._snapshot = None
         return returned
 
     def snapshot(self) -> tuple[int, ...]:
-        return tuple(self.physical_block_ids)
+        """The table as a tuple; the same object until the table changes."""
+
+        if self._snapshot is None:
+            self._snapshot = tuple(self.physical_block_ids)
+        return self._snapshot

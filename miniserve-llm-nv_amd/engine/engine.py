@@ -141,7 +141,7 @@ class Engine:
             if state.status is RequestStatus.WAITING:
                 self.runner.admit(item.request_id)
                 state.begin_prefill()
-            tokens = state.all_tokens[item.token_start : item.token_end]
+            tokens = state.tokens_between(item.token_start, item.token_end)
             final = item.token_end == state.prefill_target
             entries.append(StepEntry(item.request_id, tuple(tokens), (len(tokens) - 1,) if final else ()))
             if final:

@@ -83,6 +83,9 @@ class DecodeGraph:
             decode_prefix=batch,
         )
         self.rows = view("logit_rows")
+        # the table object that each row of the host buffer was last filled from: a request's
+        # table is the same object until it gets a page, so most steps rewrite no row
+        self._row_tables: list[list[object]] = [[None] * batch for _ in range(groups)]
         self.graph: torch.cuda.CUDAGraph | None = None
         self.logits: torch.Tensor | None = None
         self.replays = 0
@@ -115,8 +118,10 @@ class DecodeGraph:
                 if not 0 <= page < pool_pages or slot != page * block_size + meta.before % block_size:
                     raise RuntimeError(f"request {meta.request_id!r}: slot {slot} disagrees with its block table.")
                 slots.append(slot)
-                # a page that was given back is never read; 0 keeps the entry inside the pool
-                host[start + row * width : start + row * width + len(table)] = [p if p >= 0 else 0 for p in table]
+                if self._row_tables[group][row] is not table:
+                    # a page that was given back is never read; 0 keeps the entry inside the pool
+                    host[start + row * width : start + row * width + len(table)] = [p if p >= 0 else 0 for p in table]
+                    self._row_tables[group][row] = table
             put(f"slots{group}", slots)
 
     def run(self, entries: Sequence[StepEntry], reservation) -> torch.Tensor:

@@ -79,6 +79,22 @@ class SequenceState:
     def all_tokens(self) -> tuple[int, ...]:
         return self.prompt_token_ids + tuple(self.generated_token_ids)
 
+    def token_at(self, index: int) -> int:
+        """``all_tokens[index]`` without building the whole tuple (this is asked every step)."""
+
+        prompt = len(self.prompt_token_ids)
+        return self.prompt_token_ids[index] if index < prompt else self.generated_token_ids[index - prompt]
+
+    def tokens_between(self, start: int, end: int) -> tuple[int, ...]:
+        """``all_tokens[start:end]``."""
+
+        prompt = len(self.prompt_token_ids)
+        if end <= prompt:
+            return self.prompt_token_ids[start:end]
+        if start >= prompt:
+            return tuple(self.generated_token_ids[start - prompt : end - prompt])
+        return self.prompt_token_ids[start:] + tuple(self.generated_token_ids[: end - prompt])
+
     @property
     def total_tokens(self) -> int:
         return len(self.prompt_token_ids) + len(self.generated_token_ids)
@@ -96,7 +112,7 @@ class SequenceState:
             max_new_tokens=self.sampling_params.max_new_tokens,
             arrival_ns=self.arrival_ns,
             next_input_token_id=(
-                self.all_tokens[self.computed_tokens] if self.status is RequestStatus.DECODING else None
+                self.token_at(self.computed_tokens) if self.status is RequestStatus.DECODING else None
             ),
             num_preemptions=self.num_preemptions,
         )
@@ -125,7 +141,7 @@ class SequenceState:
         self.computed_tokens += 1
 
     def append_sampled_token(self, token_id: int) -> None:
-        if self.status not in {RequestStatus.PREFILLING, RequestStatus.DECODING}:
+        if self.status is not RequestStatus.PREFILLING and self.status is not RequestStatus.DECODING:
             raise RuntimeError("A token can only be sampled after model execution.")
         if self.computed_tokens != self.total_tokens:
             raise RuntimeError("All current tokens must be computed before sampling the next token.")
@@ -195,15 +211,16 @@ class SequenceState:
             raise AssertionError("computed_tokens is outside all_tokens.")
         if len(self.generated_token_ids) > self.sampling_params.max_new_tokens:
             raise AssertionError("generated tokens exceed max_new_tokens.")
-        if self.status in {RequestStatus.WAITING, RequestStatus.PREFILLING}:
+        status = self.status          # identity tests: hashing an enum member costs a Python call
+        if status is RequestStatus.WAITING or status is RequestStatus.PREFILLING:
             if self.computed_tokens != self.prefill_cursor or self.prefill_target != self.total_tokens:
                 raise AssertionError("WAITING/PREFILLING only advances the prefill of all current tokens.")
-            if self.status is RequestStatus.WAITING and self.computed_tokens != 0:
+            if status is RequestStatus.WAITING and self.computed_tokens != 0:
                 raise AssertionError("WAITING holds no computed tokens.")
-        elif self.status in {RequestStatus.DECODING, RequestStatus.FINISHED}:
+        elif status is RequestStatus.DECODING or status is RequestStatus.FINISHED:
             if not self.generated_token_ids or self.computed_tokens != self.total_tokens - 1:
                 raise AssertionError("Decode/finish must retain one sampled, uncomputed token.")
-        if self.status is RequestStatus.FINISHED and self.finish_reason not in {"stop", "length"}:
+        if status is RequestStatus.FINISHED and self.finish_reason not in {"stop", "length"}:
             raise AssertionError("FINISHED state requires a normal finish reason.")
-        if self.status is RequestStatus.FAILED and (self.finish_reason != "error" or not self.error_message):
+        if status is RequestStatus.FAILED and (self.finish_reason != "error" or not self.error_message):
             raise AssertionError("FAILED state requires a separate diagnostic message.")
