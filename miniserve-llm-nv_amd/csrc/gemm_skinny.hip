@@ -27,7 +27,6 @@ using ms::floatx4;
 
 constexpr int kWavesPerGroup = 8;
 constexpr int kGroupThreads = kWavesPerGroup * ms::kWave;
-constexpr int kUnroll = 4;   // k-steps whose loads are issued together
 
 enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAddF32 = 2, kSiluMul = 3 };
 
@@ -39,7 +38,8 @@ enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAddF32 = 2, kSiluMul = 3 }
 // sums them in the same fixed order.  (The separate norm kernel rounds the
 // normalised value before the multiply by the weight, as the reference does; here
 // the one rounding is of w_norm * h.  Both carry 8 significant bits.)
-template <int MB, int RB, bool NORM>
+// UNROLL: k-steps whose loads are issued together (more for long rows: more bytes in flight)
+template <int MB, int RB, bool NORM, int UNROLL>
 __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                     const float* __restrict__ h,
                                                                     const bf16* __restrict__ norm_weight, float eps,
@@ -98,10 +98,10 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
   float square_sum = 0.f;
 
   const int steps = (k + 31) / 32;
-  for (int base = wave; base < steps; base += kWavesPerGroup * kUnroll) {
-    bf16x8 a[kUnroll][RB], b[kUnroll][MB];
+  for (int base = wave; base < steps; base += kWavesPerGroup * UNROLL) {
+    bf16x8 a[UNROLL][RB], b[UNROLL][MB];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < UNROLL; ++u) {
       const int k0 = 32 * (base + u * kWavesPerGroup) + 8 * g;
       const bool live = k0 < k;      // k is a multiple of 8
 #pragma unroll
@@ -127,7 +127,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
       }
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
+    for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
@@ -194,10 +194,18 @@ void launch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, 
   const int rows = epilogue == kSiluMul ? n / 2 : n;
   const int blocks_per_group = epilogue == kSiluMul ? RB / 2 : RB;
   const int groups = (rows + 16 * blocks_per_group - 1) / (16 * blocks_per_group);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM>), dim3(groups), dim3(kGroupThreads), 0, stream,
-                     static_cast<const bf16*>(x), static_cast<const float*>(h),
-                     static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
-                     static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue);
+  // rows of 2048 elements and more: eight k-steps in flight a wave (where the registers allow it)
+  if (k >= 2048 && MB * RB <= 2) {
+    hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 8>), dim3(groups), dim3(kGroupThreads), 0, stream,
+                       static_cast<const bf16*>(x), static_cast<const float*>(h),
+                       static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
+                       static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue);
+  } else {
+    hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 4>), dim3(groups), dim3(kGroupThreads), 0, stream,
+                       static_cast<const bf16*>(x), static_cast<const float*>(h),
+                       static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
+                       static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue);
+  }
 }
 
 }  // namespace
