@@ -7,8 +7,8 @@ the paged cache, sampling) with ``--batch`` live requests, each after a prompt o
 ``--prompt-len`` random tokens.  The model has the layer sizes of Qwen3-0.6B (or
 of ``--size``) with random weights.  One JSON line is printed: decoded tokens a second, the prefill
 rate of one 2,048-token prompt with its fraction of the bf16 MFMA peak, the
-fraction of the HBM peak that the decode step reaches, and decode rates at batch
-1 and 64.
+fraction of the HBM peak that the decode step reaches, decode rates at batch 1 and
+64, and what the card reaches on a plain device copy and a large library product.
 """
 
 from __future__ import annotations
@@ -166,6 +166,28 @@ def main() -> int:
     del runner
     torch.cuda.empty_cache()
 
+    # ---- what this card reaches on plain work: a device copy and a large library product ----
+    from miniserve_amd import ops
+
+    def rate(function, repeats=5):
+        function()
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        for _ in range(repeats):
+            function()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - begin) / repeats
+
+    source = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+    target = torch.empty_like(source)
+    copy_gbps = 2 * source.numel() / rate(lambda: target.copy_(source)) / 1e9       # bytes read and written
+    del source, target
+    a = torch.randn(8192, 8192, device=device, dtype=torch.bfloat16)
+    b = torch.randn(8192, 8192, device=device, dtype=torch.bfloat16)
+    gemm_tflops = 2 * 8192**3 / rate(lambda: ops.linear(a, b)) / 1e12
+    del a, b
+    torch.cuda.empty_cache()
+
     points = {}
     if not args.no_points:
         for batch in (1, 64):
@@ -218,6 +240,7 @@ def main() -> int:
             "frac": round(achieved / HBM_GBPS, 5),
         },
         "points": points,
+        "measured": {"copy_GBps": round(copy_gbps, 1), "library_gemm_8192_TFLOPs": round(gemm_tflops, 1)},
     }
     print(json.dumps(line))
     return 0

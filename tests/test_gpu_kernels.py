@@ -564,6 +564,51 @@ def test_product_beyond_64_rows_uses_the_library(ops):
     torch.testing.assert_close(ops.linear_silu_mul(x, w[:32].contiguous()), ops.silu_mul(ops.linear(x, w[:32].contiguous())))
 
 
+@pytest.mark.parametrize("m,n,k", [(17, 509, 96), (65, 33, 60), (300, 1024, 200), (2048, 4096, 1024), (129, 300, 80)])
+def test_library_product_for_many_rows(ops, m, n, k):
+    """Beyond 16 rows the product goes to hipBLASLt, bound at run time to the copy the
+    process has: bfloat16 out, 32-bit out, and += into a 32-bit tensor; sizes off every
+    grid; the same shape again takes the kept plan."""
+
+    x, w = rand(m, k, seed=m, dtype=torch.bfloat16), rand(n, k, seed=n, dtype=torch.bfloat16, scale=0.1)
+    exact = x.cpu().double() @ w.cpu().double().T
+    scale = float(exact.abs().max())
+    for _ in range(2):
+        torch.testing.assert_close(ops.linear(x, w).cpu().double(), exact, atol=scale * 2**-8, rtol=2**-7)
+        wide = ops.linear(x, w, out_float32=True)
+        assert wide.dtype == torch.float32
+        torch.testing.assert_close(wide.cpu().double(), exact, atol=scale * 1e-5, rtol=1e-5)
+        base = rand(m, n, seed=5)
+        total = base.clone()
+        assert ops.linear(x, w, accumulate_into=total) is total
+        torch.testing.assert_close(total.cpu().double(), base.cpu().double() + exact, atol=scale * 1e-5, rtol=1e-5)
+    from miniserve_amd.ops import KernelError
+
+    assert ops.can_accumulate(m, w)
+    with pytest.raises(KernelError, match="must have shape"):
+        ops.linear(x, w, accumulate_into=torch.zeros(m, n + 1, device=DEVICE))
+
+
+def test_library_product_inside_a_recorded_graph(ops):
+    """Replayed several times with eager work between the replays; every replay gives
+    what the eager call gives for the inputs of that moment."""
+
+    x = rand(64, 256, seed=1, dtype=torch.bfloat16)
+    w = rand(512, 256, seed=2, dtype=torch.bfloat16, scale=0.1)
+    ops.linear(x, w)                                        # plan and workspace exist before the recording
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = ops.linear(x, w, out_float32=True)
+    for round_index in range(4):
+        x.copy_(rand(64, 256, seed=10 + round_index, dtype=torch.bfloat16))
+        graph.replay()
+        torch.cuda.synchronize()
+        expected = ops.linear(x, w, out_float32=True)       # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(out, expected)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rows,inter", [(1, 1), (3, 63), (5, 200), (64, 3072), (2, 1031)])
 def test_silu_mul(ops, dtype, rows, inter):
