@@ -45,7 +45,9 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
                                                                     const bf16* __restrict__ norm_weight, float eps,
                                                                     const bf16* __restrict__ w, bf16* out_bf16,
                                                                     float* out_f32, int m, int n, int k,
-                                                                    int epilogue) {
+                                                                    int epilogue, int rows) {
+  // rows: how many of the 16 rows of a block are this workgroup's (16, or 8 or 4 for a
+  // matrix of few rows, so that there are workgroups enough to fill the chip)
   __shared__ float c_s[kWavesPerGroup][RB * MB][16][16];
   __shared__ float square_s[kWavesPerGroup][16];
 
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
       const int pair = rb % (RB / 2 > 0 ? RB / 2 : 1);
       row_start[rb] = (blockIdx.x * (RB / 2 > 0 ? RB / 2 : 1) + pair) * 16 + (rb >= RB / 2 ? half : 0);
     } else {
-      row_start[rb] = (blockIdx.x * RB + rb) * 16;
+      row_start[rb] = (blockIdx.x * RB + rb) * rows;
     }
   }
   const int row_limit = epilogue == kSiluMul ? half : n;   // rows of one half for the gated form
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
       const int k0 = 32 * (base + u * kWavesPerGroup) + 8 * g;
       const bool live = k0 < k;      // k is a multiple of 8
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) a[u][rb] = live ? ms::load_bf16x8(w_row[rb] + k0) : ms::zero_bf16x8();
+      for (int rb = 0; rb < RB; ++rb) a[u][rb] = (live && r < rows) ? ms::load_bf16x8(w_row[rb] + k0) : ms::zero_bf16x8();
       if (NORM) {
         bf16x8 made = ms::zero_bf16x8();
         if (live && x_live[0]) {
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     const int rb = tile / MB, mb = tile - rb * MB;
     const int row_m = 16 * mb + m_local;
     const int col_n = row_start[rb] + n_local;
-    if (row_m >= m || col_n >= row_limit) continue;
+    if (row_m >= m || col_n >= row_limit || n_local >= rows) continue;
     float sum = 0.f;
 #pragma unroll
     for (int wv = 0; wv < kWavesPerGroup; ++wv) sum += c_s[wv][tile][m_local][n_local];
@@ -191,20 +193,26 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
 template <int MB, int RB, bool NORM = false>
 void launch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, int n, int k, int epilogue,
             hipStream_t stream, const void* h = nullptr, const void* norm_weight = nullptr, float eps = 0.f) {
-  const int rows = epilogue == kSiluMul ? n / 2 : n;
+  const int out_rows = epilogue == kSiluMul ? n / 2 : n;
   const int blocks_per_group = epilogue == kSiluMul ? RB / 2 : RB;
-  const int groups = (rows + 16 * blocks_per_group - 1) / (16 * blocks_per_group);
+  // A matrix of few rows gives 8 or 4 rows instead of 16 to a workgroup: one workgroup
+  // streams less, and there are 256 compute units to feed.
+  int rows = 16;
+  if (RB == 1 && epilogue != kSiluMul) {
+    while (rows > 4 && (out_rows + rows - 1) / rows < 256) rows /= 2;
+  }
+  const int groups = (out_rows + rows * blocks_per_group - 1) / (rows * blocks_per_group);
   // rows of 2048 elements and more: eight k-steps in flight a wave (where the registers allow it)
   if (k >= 2048 && MB * RB <= 2) {
     hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 8>), dim3(groups), dim3(kGroupThreads), 0, stream,
                        static_cast<const bf16*>(x), static_cast<const float*>(h),
                        static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
-                       static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue);
+                       static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue, rows);
   } else {
     hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 4>), dim3(groups), dim3(kGroupThreads), 0, stream,
                        static_cast<const bf16*>(x), static_cast<const float*>(h),
                        static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
-                       static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue);
+                       static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue, rows);
   }
 }
 
