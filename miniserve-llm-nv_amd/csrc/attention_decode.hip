@@ -264,6 +264,16 @@ __global__ void attention_merge_splits_kernel(const float* __restrict__ partial_
                                               int head_dim, int num_splits) {
   __shared__ float weight_s[ms::kWave];
   const int64_t row = blockIdx.x;
+  // the first partial outputs of this thread's column are on their way while the first
+  // wave makes the weights
+  constexpr int kAhead = 16;
+  const int d0 = threadIdx.x;
+  float ahead[kAhead];
+  if (d0 < head_dim) {
+    const float* column = partial_o + row * num_splits * head_dim + d0;
+#pragma unroll
+    for (int s = 0; s < kAhead; ++s) ahead[s] = s < num_splits ? column[static_cast<int64_t>(s) * head_dim] : 0.f;
+  }
   if (threadIdx.x < ms::kWave) {
     const int s = threadIdx.x;
     const bool live = s < num_splits;
@@ -275,11 +285,17 @@ __global__ void attention_merge_splits_kernel(const float* __restrict__ partial_
     weight_s[s] = f / total;
   }
   __syncthreads();
-  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+  for (int d = d0; d < head_dim; d += blockDim.x) {
     const float* column = partial_o + row * num_splits * head_dim + d;
     float acc = 0.f;
+    if (d == d0) {
+#pragma unroll
+      for (int s = 0; s < kAhead; ++s) acc = fmaf(s < num_splits ? weight_s[s] : 0.f, ahead[s], acc);
+      for (int s = kAhead; s < num_splits; ++s) acc = fmaf(weight_s[s], column[static_cast<int64_t>(s) * head_dim], acc);
+    } else {
 #pragma unroll 8
-    for (int s = 0; s < num_splits; ++s) acc = fmaf(weight_s[s], column[static_cast<int64_t>(s) * head_dim], acc);
+      for (int s = 0; s < num_splits; ++s) acc = fmaf(weight_s[s], column[static_cast<int64_t>(s) * head_dim], acc);
+    }
     out[row * head_dim + d] = ms::from_float<bf16>(acc);
   }
 }

@@ -55,45 +55,56 @@ __global__ void qk_norm_rope_append_kernel(const T* __restrict__ packed, const T
     }
   }
 
+  // Everything the row needs is asked for at once (the row, the norm's weight, the
+  // angles): one round trip to memory, not three behind one another.
+  const T* weight = is_q ? q_weight : (is_k ? k_weight : nullptr);
+  const bool rotate = cos_table != nullptr && (is_q || is_k);
   float lo[kMaxPairsPerLane], hi[kMaxPairsPerLane];
-  float partial = 0.f;
+  float w_lo[kMaxPairsPerLane], w_hi[kMaxPairsPerLane], cs[kMaxPairsPerLane], sn[kMaxPairsPerLane];
 #pragma unroll
   for (int c = 0; c < kMaxPairsPerLane; ++c) {
     const int i = lane + c * ms::kWave;
     lo[c] = hi[c] = 0.f;
+    w_lo[c] = w_hi[c] = cs[c] = 1.f;
+    sn[c] = 0.f;
     if (i < half) {
       lo[c] = ms::to_float(row[i]);
       hi[c] = ms::to_float(row[i + half]);
-      partial = fmaf(lo[c], lo[c], partial);
-      partial = fmaf(hi[c], hi[c], partial);
-    }
-  }
-
-  const T* weight = is_q ? q_weight : (is_k ? k_weight : nullptr);
-  if (weight) {
-    const float total = ms::wave_sum(partial);
-    const float inv = 1.0f / sqrtf(total / static_cast<float>(head_dim) + eps);
-#pragma unroll
-    for (int c = 0; c < kMaxPairsPerLane; ++c) {
-      const int i = lane + c * ms::kWave;
-      if (i < half) {
-        lo[c] = ms::round_to<T>(ms::to_float(weight[i]) * ms::round_to<T>(lo[c] * inv));
-        hi[c] = ms::round_to<T>(ms::to_float(weight[i + half]) * ms::round_to<T>(hi[c] * inv));
+      if (weight) {
+        w_lo[c] = ms::to_float(weight[i]);
+        w_hi[c] = ms::to_float(weight[i + half]);
+      }
+      if (rotate) {
+        cs[c] = cos_table[token * half + i];
+        sn[c] = sin_table[token * half + i];
       }
     }
   }
 
-  const bool rotate = cos_table != nullptr && (is_q || is_k);
+  if (weight) {
+    float partial = 0.f;
+#pragma unroll
+    for (int c = 0; c < kMaxPairsPerLane; ++c) {
+      partial = fmaf(lo[c], lo[c], partial);
+      partial = fmaf(hi[c], hi[c], partial);
+    }
+    const float total = ms::wave_sum(partial);
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(head_dim) + eps);
+#pragma unroll
+    for (int c = 0; c < kMaxPairsPerLane; ++c) {
+      lo[c] = ms::round_to<T>(w_lo[c] * ms::round_to<T>(lo[c] * inv));
+      hi[c] = ms::round_to<T>(w_hi[c] * ms::round_to<T>(hi[c] * inv));
+    }
+  }
+
 #pragma unroll
   for (int c = 0; c < kMaxPairsPerLane; ++c) {
     const int i = lane + c * ms::kWave;
     if (i < half) {
       float a = lo[c], b = hi[c];
       if (rotate) {
-        const float cs = cos_table[token * half + i];
-        const float sn = sin_table[token * half + i];
-        const float ra = a * cs - b * sn;
-        const float rb = b * cs + a * sn;
+        const float ra = a * cs[c] - b * sn[c];
+        const float rb = b * cs[c] + a * sn[c];
         a = ra;
         b = rb;
       }
