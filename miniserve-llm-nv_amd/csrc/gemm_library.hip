@@ -47,6 +47,46 @@ std::map<int, hipblasLtHandle_t> g_handles;                             // by de
 std::map<std::tuple<int, int, int, int, int>, Plan> g_plans;            // (device, m, n, k, out is float)
 constexpr size_t kMaxPlans = 4096;
 
+constexpr int kCandidates = 8;
+constexpr int kTuneFromRows = 256;
+
+// Index of the candidate that runs this product fastest (two timed runs after a first
+// one).  The output goes to memory of its own, so that `out` is written once, by the call.
+int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const hipblasLtMatmulHeuristicResult_t* candidates,
+                      int count, const void* x, const void* w, int m, int n, int out_float, void* workspace,
+                      size_t workspace_bytes, hipStream_t stream) {
+  void* scratch = nullptr;
+  const size_t bytes = static_cast<size_t>(m) * n * (out_float ? 4 : 2);
+  if (hipMalloc(&scratch, bytes) != hipSuccess) return 0;
+  hipEvent_t begin = nullptr, end = nullptr;
+  int best = 0;
+  if (hipEventCreate(&begin) == hipSuccess && hipEventCreate(&end) == hipSuccess) {
+    const float alpha = 1.0f, beta = 0.0f;
+    float best_ms = 0.f;
+    for (int i = 0; i < count; ++i) {
+      if (candidates[i].state != HIPBLAS_STATUS_SUCCESS || candidates[i].workspaceSize > workspace_bytes) continue;
+      bool ok = true;
+      float ms = 0.f;
+      for (int run = 0; run < 3 && ok; ++run) {
+        if (run == 1) ok = hipEventRecord(begin, stream) == hipSuccess;
+        ok = ok && g_api.matmul(handle, plan.desc, &alpha, w, plan.a, x, plan.b, &beta, scratch, plan.c, scratch, plan.c,
+                                &candidates[i].algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
+      }
+      ok = ok && hipEventRecord(end, stream) == hipSuccess && hipEventSynchronize(end) == hipSuccess &&
+           hipEventElapsedTime(&ms, begin, end) == hipSuccess;
+      if (ok && (best_ms == 0.f || ms < best_ms)) {
+        best_ms = ms;
+        best = i;
+      }
+    }
+  }
+  if (begin) hipEventDestroy(begin);
+  if (end) hipEventDestroy(end);
+  hipStreamSynchronize(stream);
+  hipFree(scratch);
+  return best;
+}
+
 template <typename F>
 bool resolve(F& slot, const char* name) {
   slot = reinterpret_cast<F>(dlsym(g_api.library, name));
@@ -115,14 +155,22 @@ extern "C" int ms_gemm_library(const void* x, const void* w, void* out, int m, i
     MS_REQUIRE(g_api.pref_create(&preference) == HIPBLAS_STATUS_SUCCESS, "gemm_library: no preference object");
     const uint64_t limit = workspace_bytes;
     g_api.pref_set(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit));
-    hipblasLtMatmulHeuristicResult_t result[1];
+    hipblasLtMatmulHeuristicResult_t result[kCandidates];
     int returned = 0;
     const hipblasStatus_t status =
-        g_api.heuristic(handle, plan.desc, plan.a, plan.b, plan.c, plan.c, preference, 1, result, &returned);
+        g_api.heuristic(handle, plan.desc, plan.a, plan.b, plan.c, plan.c, preference, kCandidates, result, &returned);
     g_api.pref_destroy(preference);
     MS_REQUIRE(status == HIPBLAS_STATUS_SUCCESS && returned > 0, "gemm_library: no algorithm for %d x %d x %d", m, n, k);
-    plan.algo = result[0].algo;
-    plan.workspace = result[0].workspaceSize;
+    int best = 0;
+    // Many rows: the library's first choice is not always its fastest.  The candidates
+    // are timed once, on scratch output, unless the stream is recording (no waiting there).
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (m >= kTuneFromRows && returned > 1 && hipStreamIsCapturing(stream, &capture) == hipSuccess &&
+        capture == hipStreamCaptureStatusNone) {
+      best = fastest_candidate(handle, plan, result, returned, x, w, m, n, out_float, workspace, workspace_bytes, stream);
+    }
+    plan.algo = result[best].algo;
+    plan.workspace = result[best].workspaceSize;
     found = g_plans.emplace(key, plan).first;
   }
   const Plan& plan = found->second;

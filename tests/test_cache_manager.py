@@ -121,6 +121,36 @@ def test_window_table_gives_pages_back():
     assert table.slot(16) == 9 * 4
 
 
+def test_the_snapshot_is_one_object_until_the_table_changes():
+    table = BlockTable(4, [3, 5])
+    first = table.snapshot()
+    assert first == (3, 5) and table.snapshot() is first
+    table.append_blocks([])
+    assert table.snapshot() is first and table.live_count() == 2
+    table.append_blocks([7])
+    assert table.snapshot() == (3, 5, 7) and table.snapshot() is not first
+    kept = table.snapshot()
+    assert table.give_back_before(3) == [] and table.snapshot() is kept
+    assert table.give_back_before(4) == [3] and table.snapshot() == (RETURNED, 5, 7) and table.live_count() == 2
+
+
+def test_a_step_without_a_new_page_shares_the_table_snapshot():
+    m = manager()
+    m.admit("r")
+    m.commit_step(m.prepare_step([StepItem("r", 0, 5)]))
+    one = m.prepare_step([StepItem("r", 5, 6)])
+    table = one.sequences[0].block_tables[0]
+    assert one.sequences[0].new_pages[0] == [] and one.sequences[0].slot_mappings[0] == (table[1] * 4 + 1,)
+    m.commit_step(one)
+    two = m.prepare_step([StepItem("r", 6, 7)])
+    assert two.sequences[0].block_tables[0] is table          # nothing changed: the same object
+    m.commit_step(two)
+    three = m.prepare_step([StepItem("r", 7, 9)])              # crosses into a third page
+    assert len(three.sequences[0].new_pages[0]) == 1 and len(three.sequences[0].block_tables[0]) == 3
+    m.abort_step(three)
+    assert m.prepare_step([StepItem("r", 7, 8)]).sequences[0].block_tables[0] is table
+
+
 # ---- the manager ------------------------------------------------------------------------
 
 def test_ten_tokens_take_three_pages_and_abort_restores():

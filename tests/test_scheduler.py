@@ -67,6 +67,22 @@ def test_prefill_and_decode_preserve_pending_token_invariant():
     assert state.status is RequestStatus.FINISHED and state.computed_tokens == state.total_tokens - 1
 
 
+def test_tokens_are_read_without_building_the_whole_sequence():
+    state = SequenceState.from_request(request(max_new_tokens=4))
+    state.begin_prefill()
+    state.commit_prefill(3)
+    for token in (42, 43):
+        state.append_sampled_token(token)
+        state.mark_decode_input_computed()
+    state.append_sampled_token(44)
+    everything = state.all_tokens
+    assert everything == (10, 20, 30, 42, 43, 44)
+    assert [state.token_at(i) for i in range(6)] == list(everything)
+    for start in range(6):
+        for end in range(start + 1, 7):
+            assert state.tokens_between(start, end) == everything[start:end]
+
+
 def test_stop_token_finishes_without_being_run():
     # reference: tests/unit/test_sequence_state.py:74-82
     state = SequenceState.from_request(request(max_new_tokens=4, stop=(99,)))
