@@ -524,7 +524,7 @@ def test_linear_bfloat16_and_fused_projection_rows(ops):
 
 
 @pytest.mark.parametrize("m", [1, 8, 15, 16, 17, 33, 64])
-@pytest.mark.parametrize("n,k", [(16, 32), (509, 96), (100, 200), (4096, 1024), (1024, 3072), (72, 2056), (40000, 64)])
+@pytest.mark.parametrize("n,k", [(16, 32), (509, 96), (100, 200), (4096, 1024), (1024, 3072), (72, 2056), (40, 4104), (40000, 64)])
 def test_skinny_product_for_few_rows(ops, m, n, k, monkeypatch):
     """The matrix-core product that decoding uses (at most 64 rows), with its four
     epilogues, against float64; sizes off the tile grid in every dimension."""
@@ -740,7 +740,7 @@ def test_sampler_stages_without_advancing_the_stream(ops):
 
 
 @pytest.mark.parametrize("m", [1, 7, 16])
-@pytest.mark.parametrize("n,k", [(48, 64), (512, 96), (4096, 1024), (200, 200), (96, 2056)])
+@pytest.mark.parametrize("n,k", [(48, 64), (512, 96), (4096, 1024), (200, 200), (96, 2056), (64, 4104)])
 def test_product_with_the_norm_as_its_prologue(ops, m, n, k):
     """RMSNorm of the 32-bit residual stream fused into the few-rows product equals the
     norm kernel followed by the product, also with the gated activation behind it."""
