@@ -10,12 +10,13 @@ import time
 from dataclasses import dataclass
 from typing import Callable, Sequence
 
+from ..cache import OutOfPagesError
 from ..sampling import Sampler
 from .batch import StepEntry
 from .plan import ExecutionPlan
 from .request import Request, SamplingParams
 from .scheduler import Scheduler
-from .sequence import TERMINAL, RequestStatus, SequenceState
+from .sequence import TERMINAL, RequestStatus, SequenceState, SequenceView
 
 
 @dataclass(frozen=True)
@@ -35,6 +36,13 @@ class GenerationResult:
     token_ids: tuple[int, ...]
     finish_reason: str | None
     num_preemptions: int = 0
+
+
+@dataclass(frozen=True)
+class _StepAhead:
+    version: int            # of the engine's request set when the step was planned
+    plan: ExecutionPlan
+    prepared: object        # the runner's handle: an open cache transaction
 
 
 class Engine:
@@ -62,6 +70,8 @@ class Engine:
         self._sequences: dict[str, SequenceState] = {}
         self._results: dict[str, GenerationResult] = {}
         self.last_plan: ExecutionPlan | None = None
+        self._version = 0                       # goes up when requests are added or cancelled
+        self._ahead: _StepAhead | None = None
         self.counters = {"steps": 0, "prefill_tokens": 0, "decode_tokens": 0, "preemptions": 0, "empty_plans": 0}
 
     # ---- admission --------------------------------------------------------------------
@@ -109,19 +119,31 @@ class Engine:
                 "enable chunked prefill."
             )
         self._sequences[request_id] = SequenceState.from_request(request)
+        self._version += 1
 
     def cancel(self, request_id: str) -> None:
         state = self._sequences[request_id]
+        self._version += 1
+        self._drop_prepared_step()
         state.cancel()
         self._finalize(state)
+
+    def _drop_prepared_step(self) -> None:
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None:
+            self.runner.discard(ahead.prepared)
 
     def has_unfinished(self) -> bool:
         return bool(self._sequences)
 
     # ---- one step ---------------------------------------------------------------------
     def step(self) -> list[StepOutput]:
-        views = [state.snapshot() for state in self._sequences.values()]
-        plan = self.scheduler.schedule(views, self.runner.cache.capacity())
+        ahead = self._take_prepared_step()
+        if ahead is not None:
+            plan = ahead.plan
+        else:
+            views = [state.snapshot() for state in self._sequences.values()]
+            plan = self.scheduler.schedule(views, self.runner.cache.capacity())
         self.last_plan = plan
         for request_id in plan.preempted:
             self.runner.release(request_id)
@@ -134,8 +156,10 @@ class Engine:
         entries: list[StepEntry] = []
         sampled: list[SequenceState] = []
         for item in plan.decode_items:
-            entries.append(StepEntry(item.request_id, (item.input_token_id,), (0,)))
-            sampled.append(self._sequences[item.request_id])
+            state = self._sequences[item.request_id]
+            # (a step planned ahead did not know the token yet)
+            entries.append(StepEntry(item.request_id, (state.token_at(state.computed_tokens),), (0,)))
+            sampled.append(state)
         for item in plan.prefill_items:
             state = self._sequences[item.request_id]
             if state.status is RequestStatus.WAITING:
@@ -147,13 +171,26 @@ class Engine:
             if final:
                 sampled.append(state)
 
+        next_ahead = None
         try:
-            logits = self.runner.step(entries)
+            if ahead is not None:
+                logits = self.runner.step(entries, prepared=ahead.prepared)
+            else:
+                logits = self.runner.step(entries)
             staged = ()
             if sampled:
-                staged = self.sampler.stage(logits, [(s.request_id, s.sampling_params) for s in sampled])
+                requests = [(s.request_id, s.sampling_params) for s in sampled]
+                if hasattr(self.sampler, "launch"):
+                    launched = self.sampler.launch(logits, requests)
+                    # while the GPU runs the step: the next one, if it can be foreseen
+                    next_ahead = self._prepare_step_ahead(plan, sampled)
+                    staged = self.sampler.finish(launched)
+                else:
+                    staged = self.sampler.stage(logits, requests)
         except Exception as exc:
             # the step left no trace in the cache; its requests fail (reference: core.py:396-406)
+            if next_ahead is not None:
+                self.runner.discard(next_ahead.prepared)
             for entry in entries:
                 state = self._sequences[entry.request_id]
                 state.fail(f"{type(exc).__name__}: {exc}")
@@ -169,14 +206,72 @@ class Engine:
         for item in plan.prefill_items:
             self._sequences[item.request_id].commit_prefill(item.token_end)
         outputs: list[StepOutput] = []
+        ended = False
         for state, sample in zip(sampled, staged):
             state.append_sampled_token(sample.token_id)
             reason = state.should_finish()
             if reason is not None:
+                if next_ahead is not None:
+                    # a request of the step that was planned ahead ends (a stop token): that
+                    # step's reservation goes back before the request's pages can
+                    self.runner.discard(next_ahead.prepared)
+                    next_ahead = None
+                ended = True
                 state.finish(reason)
                 self._finalize(state)
             outputs.append(StepOutput(state.request_id, sample.token_id, reason is not None, reason))
+        if next_ahead is not None and not ended:
+            self._ahead = next_ahead
         return outputs
+
+    # ---- the next step, planned while the GPU runs this one -------------------------------
+    def _take_prepared_step(self) -> "_StepAhead | None":
+        """The step planned ahead, if nothing has happened since that it did not foresee."""
+
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None and ahead.version != self._version:
+            self.runner.discard(ahead.prepared)
+            return None
+        return ahead
+
+    def _prepare_step_ahead(self, plan: ExecutionPlan, sampled: Sequence[SequenceState]) -> "_StepAhead | None":
+        """When every request decodes and none can end by length, the next step is this one
+        again with each request one token further: it is scheduled from views that say so,
+        its cache transaction is opened and its numbers are written now, and only the token
+        ids are left for when they are known.  Anything else is left to the next call."""
+
+        prepare = getattr(self.runner, "prepare_decode", None)
+        if prepare is None or plan.prefill_items or plan.preempted or len(plan.decode_items) != len(self._sequences):
+            return None
+        views = []
+        for state in sampled:
+            if len(state.generated_token_ids) + 1 >= state.sampling_params.max_new_tokens:
+                return None
+            views.append(
+                SequenceView(
+                    request_id=state.request_id,
+                    status=RequestStatus.DECODING,
+                    prefill_target=state.prefill_target,
+                    prefill_cursor=state.prefill_cursor,
+                    computed_tokens=state.computed_tokens + 1,
+                    total_tokens=state.total_tokens + 1,
+                    num_generated=len(state.generated_token_ids) + 1,
+                    max_new_tokens=state.sampling_params.max_new_tokens,
+                    arrival_ns=state.arrival_ns,
+                    next_input_token_id=0,          # not known yet; the step reads it from the request
+                    num_preemptions=state.num_preemptions,
+                )
+            )
+        next_plan = self.scheduler.schedule(views, self.runner.cache.capacity())
+        if next_plan.prefill_items or next_plan.preempted or len(next_plan.decode_items) != len(views):
+            return None
+        try:
+            prepared = prepare([item.request_id for item in next_plan.decode_items])
+        except OutOfPagesError:
+            return None                # the plan's page count was an estimate; the next call decides
+        if prepared is None:
+            return None
+        return _StepAhead(self._version, next_plan, prepared)
 
     def _finalize(self, state: SequenceState) -> None:
         """A request that ended gives back its pages, its state slot and its random stream."""

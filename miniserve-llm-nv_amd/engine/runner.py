@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import gc
 import weakref
+from dataclasses import dataclass
 from pathlib import Path
 from typing import Sequence
 
@@ -56,8 +57,11 @@ class DecodeGraph:
         for name, size in sizes:
             self.offsets[name] = (total, size)
             total += size
-        self.host = torch.zeros(total, dtype=torch.int32).pin_memory()
-        self.host_np = self.host.numpy()
+        # two host buffers, used in turn: the next step's numbers may be written while the
+        # copy of this step's is still on its way
+        self.hosts = [torch.zeros(total, dtype=torch.int32).pin_memory() for _ in range(2)]
+        self.hosts_np = [host.numpy() for host in self.hosts]
+        self._turn = 0
         self.meta = torch.zeros(total, dtype=torch.int32, device=runner.device)
         self.width = width
         view = lambda name: self.meta[self.offsets[name][0] : self.offsets[name][0] + self.offsets[name][1]]
@@ -85,20 +89,26 @@ class DecodeGraph:
         self.rows = view("logit_rows")
         # the table object that each row of the host buffer was last filled from: a request's
         # table is the same object until it gets a page, so most steps rewrite no row
-        self._row_tables: list[list[object]] = [[None] * batch for _ in range(groups)]
+        self._row_tables: list[list[list[object]]] = [[[None] * batch for _ in range(groups)] for _ in range(2)]
         self.graph: torch.cuda.CUDAGraph | None = None
         self.logits: torch.Tensor | None = None
         self.replays = 0
 
-    def _fill(self, entries: Sequence[StepEntry], reservation) -> None:
-        host, offsets, batch, width = self.host_np, self.offsets, self.batch, self.width
+    def _next_buffer(self) -> int:
+        which = self._turn
+        self._turn ^= 1
+        return which
+
+    def _fill(self, reservation, which: int) -> None:
+        """Everything of the step but its token ids, into host buffer ``which``."""
+
+        host, offsets, batch, width = self.hosts_np[which], self.offsets, self.batch, self.width
 
         def put(name: str, values) -> None:
             start, size = offsets[name]
             host[start : start + size] = values
 
         metas = reservation.sequences
-        put("token_ids", [entry.token_ids[0] for entry in entries])
         put("positions", [meta.before for meta in metas])
         put("seq_of_token", range(batch))
         put("query_start", range(batch + 1))
@@ -111,6 +121,7 @@ class DecodeGraph:
             pool_pages = runner.cache.num_blocks[group]
             slots = []
             start, _ = offsets[f"table{group}"]
+            row_tables = self._row_tables[which][group]
             for row, meta in enumerate(metas):
                 table = meta.block_tables[group]
                 slot = meta.slot_mappings[group][0]
@@ -118,18 +129,34 @@ class DecodeGraph:
                 if not 0 <= page < pool_pages or slot != page * block_size + meta.before % block_size:
                     raise RuntimeError(f"request {meta.request_id!r}: slot {slot} disagrees with its block table.")
                 slots.append(slot)
-                if self._row_tables[group][row] is not table:
+                if row_tables[row] is not table:
                     # a page that was given back is never read; 0 keeps the entry inside the pool
                     host[start + row * width : start + row * width + len(table)] = [p if p >= 0 else 0 for p in table]
-                    self._row_tables[group][row] = table
+                    row_tables[row] = table
             put(f"slots{group}", slots)
 
-    def run(self, entries: Sequence[StepEntry], reservation) -> torch.Tensor:
-        """Logits ``[batch, vocab]`` of the step; the tensor is the graph's own output
-        buffer and holds these values until the next step of this batch size."""
+    def prepare(self, reservation) -> int | None:
+        """Fills a host buffer for a coming step whose token ids are not known yet and
+        returns its number; None when the step is not recorded yet."""
 
-        self._fill(entries, reservation)
-        self.meta.copy_(self.host, non_blocking=True)
+        if self.graph is None:
+            return None
+        which = self._next_buffer()
+        self._fill(reservation, which)
+        return which
+
+    def run(self, entries: Sequence[StepEntry], reservation, prepared: int | None = None) -> torch.Tensor:
+        """Logits ``[batch, vocab]`` of the step; the tensor is the graph's own output
+        buffer and holds these values until the next step of this batch size.
+        ``prepared``: the host buffer that :meth:`prepare` filled for this reservation."""
+
+        which = prepared
+        if which is None:
+            which = self._next_buffer()
+            self._fill(reservation, which)
+        start, size = self.offsets["token_ids"]
+        self.hosts_np[which][start : start + size] = [entry.token_ids[0] for entry in entries]
+        self.meta.copy_(self.hosts[which], non_blocking=True)
         runner = self._runner()
         model, views = runner.model, runner._call_views
         if self.graph is None:
@@ -155,6 +182,16 @@ class DecodeGraph:
         self.graph.replay()
         self.replays += 1
         return self.logits
+
+
+@dataclass(frozen=True)
+class PreparedDecode:
+    """A step of single tokens whose cache transaction is open and whose numbers are
+    written, but for the token ids."""
+
+    request_ids: tuple[str, ...]
+    reservation: object
+    buffer: int
 
 
 class ModelRunner:
@@ -203,6 +240,7 @@ class ModelRunner:
         self.steps_run = 0
         self.tokens_run = 0
         self.graph_steps = 0
+        self.prepared_steps = 0        # steps whose numbers were written while the step before ran
 
     # ---- construction -----------------------------------------------------------------
     @classmethod
@@ -247,7 +285,7 @@ class ModelRunner:
         blocks = max(1, min(by_memory, by_need))
         return blocks
 
-    def _decode_graph_step(self, entries: Sequence[StepEntry], reservation) -> torch.Tensor | None:
+    def _decode_graph_step(self, entries: Sequence[StepEntry], reservation, prepared: int | None = None) -> torch.Tensor | None:
         """A step of single tokens through the recorded graph of its batch size.  The
         graph computes the logits of every row; the wanted ones are picked."""
 
@@ -260,7 +298,7 @@ class ModelRunner:
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             graph = self._decode_graphs[batch] = DecodeGraph(self, batch)
-        logits = graph.run(entries, reservation)
+        logits = graph.run(entries, reservation, prepared)
         wanted = [index for index, entry in enumerate(entries) if entry.want]
         if len(wanted) == batch:
             return logits
@@ -276,24 +314,64 @@ class ModelRunner:
         self.cache.release(request_id)
 
     # ---- the step ---------------------------------------------------------------------
+    def prepare_decode(self, request_ids: Sequence[str]) -> "PreparedDecode | None":
+        """Opens the cache transaction of a coming step in which each of these requests
+        brings one token that is not known yet, and fills the recorded step's numbers
+        for it, so that :meth:`step` has only the token ids left to do.  None when such a
+        step is not served from a recording (then nothing is opened).  The result goes
+        to :meth:`step` with entries for the same requests in the same order, or to
+        :meth:`discard`."""
+
+        if not self.engine_config.decode_graphs or not request_ids:
+            return None
+        graph = self._decode_graphs.get(len(request_ids))
+        if graph is None or graph.graph is None:
+            return None
+        items = []
+        for request_id in request_ids:
+            start = self.cache.committed_tokens(request_id)
+            items.append(StepItem(request_id, start, start + 1))
+        reservation = self.cache.prepare_step(items)
+        try:
+            buffer = graph.prepare(reservation)
+        except BaseException:
+            self.cache.abort_step(reservation)
+            raise
+        return PreparedDecode(tuple(request_ids), reservation, buffer)
+
+    def discard(self, prepared: "PreparedDecode") -> None:
+        """Gives back what :meth:`prepare_decode` took."""
+
+        self.cache.abort_step(prepared.reservation)
+
     @torch.inference_mode()
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor | None:
+    def step(self, entries: Sequence[StepEntry], prepared: "PreparedDecode | None" = None) -> torch.Tensor | None:
         """Run one batch.  Every request of ``entries`` must be admitted; its tokens
         continue where its committed tokens end.  Returns float32 logits
         ``[wanted, vocab]`` in the order of the entries and of their ``want``, or
         None when nothing is wanted.  On an exception the step leaves no trace in
-        the cache manager."""
+        the cache manager.  ``prepared``: what :meth:`prepare_decode` returned for
+        exactly these requests."""
 
         if not entries:
             raise ValueError("a step needs at least one entry.")
-        items = []
-        for entry in entries:
-            start = self.cache.committed_tokens(entry.request_id)
-            items.append(StepItem(entry.request_id, start, start + len(entry.token_ids)))
-        reservation = self.cache.prepare_step(items)
+        if prepared is not None:
+            if tuple(entry.request_id for entry in entries) != prepared.request_ids or any(
+                len(entry.token_ids) != 1 for entry in entries
+            ):
+                self.cache.abort_step(prepared.reservation)
+                raise ValueError("the entries are not those the step was prepared for.")
+            reservation = prepared.reservation
+            self.prepared_steps += 1
+        else:
+            items = []
+            for entry in entries:
+                start = self.cache.committed_tokens(entry.request_id)
+                items.append(StepItem(entry.request_id, start, start + len(entry.token_ids)))
+            reservation = self.cache.prepare_step(items)
         if self.engine_config.decode_graphs and all(len(entry.token_ids) == 1 for entry in entries):
             try:
-                logits = self._decode_graph_step(entries, reservation)
+                logits = self._decode_graph_step(entries, reservation, None if prepared is None else prepared.buffer)
             except BaseException:
                 self.cache.abort_step(reservation)
                 raise

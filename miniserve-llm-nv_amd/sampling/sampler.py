@@ -57,6 +57,13 @@ class Sampler:
         """One token per row of float32 ``logits [R, V]`` (on the GPU) for the R
         requests, without advancing any generator."""
 
+        return self.finish(self.launch(logits, requests))
+
+    def launch(self, logits: torch.Tensor, requests: Sequence[tuple[str, SamplingParams]]):
+        """The first half of :meth:`stage`: the draws are made and the choice is launched
+        on the device; nothing waits for it.  The caller may do host work before
+        :meth:`finish` fetches the tokens."""
+
         from .. import ops
 
         if logits.ndim != 2 or logits.shape[0] != len(requests) or logits.shape[1] == 0:
@@ -90,6 +97,12 @@ class Sampler:
                 top_p=torch.tensor([p.top_p for _, p in requests], dtype=torch.float32, device=device),
                 uniform=torch.tensor(uniforms, dtype=torch.float32, device=device),
             )
+        return tokens, tuple(requests), states
+
+    def finish(self, launched) -> tuple[StagedSample, ...]:
+        """The second half of :meth:`stage`: waits for the tokens of :meth:`launch`."""
+
+        tokens, requests, states = launched
         token_ids = tokens.tolist()
         if any(token < 0 for token in token_ids):
             raise NonFiniteLogitsError("logits must contain only finite values.")

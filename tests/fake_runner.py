@@ -33,6 +33,8 @@ class FakeRunner:
         self.tokens: dict[str, list[int]] = {}
         self.steps: list[list[tuple[str, int, int]]] = []     # per step: (request, start, end)
         self.fail_on_step = fail_on_step
+        self.prepare_ahead = False          # tests switch it on
+        self.prepared_ahead = self.used_ahead = self.discarded_ahead = 0
 
     def admit(self, request_id):
         self.tokens[request_id] = []
@@ -42,13 +44,35 @@ class FakeRunner:
         self.tokens.pop(request_id, None)
         self.cache.release(request_id)
 
-    def step(self, entries):
+    def prepare_decode(self, request_ids):
+        """As the real runner's: the next step's cache transaction, opened ahead."""
+
+        if not self.prepare_ahead:
+            return None
+        items = []
+        for request_id in request_ids:
+            start = self.cache.committed_tokens(request_id)
+            items.append(StepItem(request_id, start, start + 1))
+        self.prepared_ahead += 1
+        return SimpleNamespace(request_ids=tuple(request_ids), reservation=self.cache.prepare_step(items))
+
+    def discard(self, prepared):
+        self.discarded_ahead += 1
+        self.cache.abort_step(prepared.reservation)
+
+    def step(self, entries, prepared=None):
         items = []
         for entry in entries:
             start = self.cache.committed_tokens(entry.request_id)
             assert start == len(self.tokens[entry.request_id]), "the engine skipped or repeated tokens"
             items.append(StepItem(entry.request_id, start, start + len(entry.token_ids)))
-        reservation = self.cache.prepare_step(items)
+        if prepared is not None:
+            assert tuple(entry.request_id for entry in entries) == prepared.request_ids
+            assert all(len(entry.token_ids) == 1 for entry in entries)
+            reservation = prepared.reservation
+            self.used_ahead += 1
+        else:
+            reservation = self.cache.prepare_step(items)
         if self.fail_on_step is not None and len(self.steps) == self.fail_on_step:
             self.fail_on_step = None
             self.cache.abort_step(reservation)
@@ -72,8 +96,15 @@ class ArgmaxSampler:
     """Greedy on the host; the engine's sampler interface."""
 
     def stage(self, logits, requests):
+        return self.finish(self.launch(logits, requests))
+
+    def launch(self, logits, requests):
+        return logits, tuple(requests)
+
+    def finish(self, launched):
         from miniserve_amd.sampling import StagedSample
 
+        logits, requests = launched
         return tuple(StagedSample(rid, int(torch.argmax(row)), None) for (rid, _), row in zip(requests, logits))
 
     def commit(self, samples):

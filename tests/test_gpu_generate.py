@@ -73,6 +73,7 @@ def test_greedy_generation_with_wide_heads_through_recorded_steps(model_folders)
     limits = [SamplingParams(max_new_tokens=n) for n in (40, 9, 33, 20)]
     got = llm.generate(prompts, limits)
     assert [len(tokens) for tokens in got] == [40, 9, 33, 20]
+    assert 0 < llm.runner.prepared_steps < llm.runner.graph_steps     # steps planned while the one before ran
     for tokens, prompt in zip(got, prompts):
         check_greedy(tokens, prompt, weights, config, "bfloat16")
     eager = LLM(str(folder), dtype="bfloat16", kv_block_size=block, num_kv_blocks=24, max_num_seqs=4, decode_graphs=False)

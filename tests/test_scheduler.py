@@ -317,6 +317,63 @@ def test_generate_is_the_same_whatever_the_scheduling():
     runner.cache.assert_invariants()
 
 
+def test_steps_planned_ahead_change_no_token():
+    """While a step of decoding requests runs, the next one is scheduled and its cache
+    transaction opened; what the requests generate is what they generate without that,
+    whatever ends it early: a stop token, a request that ends by length, a new request,
+    a cancelled one, too few pages."""
+
+    params = SamplingParams(max_new_tokens=12)
+    expected = [expected_generation(p, 12, 97) for p in PROMPTS]
+    engine, runner = make_engine()
+    runner.prepare_ahead = True
+    assert engine.generate(PROMPTS, params) == expected
+    assert runner.used_ahead >= 8 and runner.discarded_ahead == 0       # all four decode together for ten steps
+    assert runner.prepared_ahead == runner.used_ahead                  # the last steps end by length: not planned ahead
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
+    runner.cache.assert_invariants()
+
+    # a stop token ends a request inside a step that was planned ahead: the plan is dropped
+    stop = expected[0][4]
+    engine, runner = make_engine()
+    runner.prepare_ahead = True
+    got = engine.generate(PROMPTS, [SamplingParams(max_new_tokens=12, stop_token_ids=(stop,))] + [params] * 3)
+    assert got[0] == expected[0][: expected[0].index(stop) + 1] and got[1:] == expected[1:]
+    assert runner.discarded_ahead >= 1 and runner.used_ahead >= 4
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
+
+    # a request that arrives, and one that is cancelled, between two steps
+    engine, runner = make_engine()
+    runner.prepare_ahead = True
+    engine.add_request("a", PROMPTS[0], params, arrival_ns=0)
+    engine.add_request("b", PROMPTS[1], params, arrival_ns=1)
+    for _ in range(4):
+        engine.step()
+    assert runner.prepared_ahead > runner.used_ahead                   # one is waiting to be used
+    engine.add_request("c", PROMPTS[3], params, arrival_ns=2)
+    engine.step()                                                      # the plan ahead did not know "c"
+    assert runner.discarded_ahead == 1
+    for _ in range(3):
+        engine.step()
+    waiting = runner.prepared_ahead - runner.used_ahead - runner.discarded_ahead
+    assert waiting == 1
+    engine.cancel("b")                                                 # its pages go back: the open step first
+    assert runner.discarded_ahead == 2
+    runner.cache.assert_invariants()
+    while engine.has_unfinished():
+        engine.step()
+    assert list(engine.pop_result("a").token_ids) == expected[0] and list(engine.pop_result("c").token_ids) == expected[3]
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
+
+    # so few pages that decoding requests are preempted: plans ahead that would preempt are not made
+    tight, runner = make_engine(num_kv_blocks=14, enable_chunked_prefill=True, max_num_batched_tokens=64)
+    runner.prepare_ahead = True
+    assert tight.generate(PROMPTS, params) == expected
+    assert tight.counters["preemptions"] > 0
+    assert runner.cache.capacity().free_blocks == (14,)
+    runner.cache.assert_invariants()
+
+
 def test_stop_tokens_and_per_request_parameters():
     engine, _ = make_engine()
     first = expected_generation(PROMPTS[0], 12, 97)
