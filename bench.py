@@ -8,7 +8,9 @@ the paged cache, sampling) with ``--batch`` live requests, each after a prompt o
 of ``--size``) with random weights.  One JSON line is printed: decoded tokens a second, the prefill
 rate of one 2,048-token prompt with its fraction of the bf16 MFMA peak, the
 fraction of the HBM peak that the decode step reaches, decode rates at batch 1 and
-64, and what the card reaches on a plain device copy and a large library product.
+64, a mixed run (64 requests with prompts of 128 to 2,048 tokens, portions of 512
+beside decode tokens, through the scheduler), and what the card reaches on a plain
+device copy and a large library product.
 """
 
 from __future__ import annotations
@@ -52,7 +54,9 @@ def parse_args():
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--prefill-tokens", type=int, default=2048)
-    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the mixed run")
+    parser.add_argument("--mixed-requests", type=int, default=64, help="requests of the mixed continuous-batching run")
+    parser.add_argument("--mixed-new-tokens", type=int, default=128, help="tokens each of them generates")
     parser.add_argument("--eager", action="store_true", help="no HIP graphs for decode steps")
     return parser.parse_args()
 
@@ -141,6 +145,49 @@ def main() -> int:
         torch.cuda.empty_cache()
         return batch * steps / elapsed, 1000 * elapsed / steps, start_context + steps / 2
 
+    def mixed_rate(requests, new_tokens, chunk=512):
+        """Continuous batching as a server sees it: ``requests`` prompts of 128 to
+        ``prompt_len`` tokens (uniform, seeded) arrive at once, prompts go in portions of
+        ``chunk`` beside the decode tokens of the others, each request generates
+        ``new_tokens``.  All tokens, prompt and generated, over the wall time."""
+
+        longest = min(args.prompt_len, args.context - new_tokens)
+        rounds = []
+        for _ in range(2):      # the first is untimed: the library's choices for these shapes, the recorded steps
+            lengths = torch.randint(min(128, longest), longest + 1, (requests,), generator=generator).tolist()
+            rounds.append([random_prompts(1, length)[0] for length in lengths])
+        pages = max(sum(-(-(len(prompt) + new_tokens) // 16) for prompt in prompts) for prompts in rounds) + 16
+        engine_config = EngineConfig(
+            dtype=args.dtype, max_model_len=args.context, max_num_seqs=requests,
+            max_num_batched_tokens=min(args.context, 2 * chunk), kv_block_size=16, num_kv_blocks=pages,
+            enable_chunked_prefill=True, prefill_chunk_size=chunk, max_pending_requests=max(64, requests),
+            decode_graphs=not args.eager,
+        )
+        runner = ModelRunner.from_random(config, engine_config, seed=0, device=device)
+        params = SamplingParams(max_new_tokens=new_tokens)
+        for prompts in rounds:
+            engine = Engine(runner)
+            for index, prompt in enumerate(prompts):
+                engine.add_request(f"m{index}", prompt, params, arrival_ns=index)
+            torch.cuda.synchronize()
+            begin = time.perf_counter()
+            mixed_steps = 0
+            while engine.has_unfinished():
+                engine.step()
+                mixed_steps += bool(engine.last_plan.prefill_items and engine.last_plan.decode_items)
+            torch.cuda.synchronize()
+            elapsed = time.perf_counter() - begin
+            counters = dict(engine.counters)
+        del engine, runner
+        torch.cuda.empty_cache()
+        total = counters["prefill_tokens"] + counters["decode_tokens"]
+        return {
+            "value": round(total / elapsed, 1), "unit": "tokens/s, prompt and generated", "requests": requests,
+            "prompt_tokens": counters["prefill_tokens"], "generated_tokens": counters["decode_tokens"] + requests,
+            "steps": counters["steps"], "steps_with_both": mixed_steps, "chunk": chunk, "ms": round(1000 * elapsed, 1),
+            "preemptions": counters.get("preemptions", 0),
+        }
+
     value, ms_per_step, mean_context = decode_rate(args.batch, args.steps, args.warmup)
 
     # ---- roofline of the decode step --------------------------------------------------
@@ -193,6 +240,9 @@ def main() -> int:
         for batch in (1, 64):
             rate, _, _ = decode_rate(batch, max(16, args.steps // 4), min(args.warmup, 4))
             points[f"decode_b{batch}"] = round(rate, 1)
+    mixed = None
+    if not args.no_points:
+        mixed = mixed_rate(args.mixed_requests, args.mixed_new_tokens)
 
     line = {
         "metric": f"decode tok/s at batch {args.batch} (Qwen3-{args.size} sizes, {args.prompt_len:,}-token prompts, "
@@ -240,6 +290,7 @@ def main() -> int:
             "frac": round(achieved / HBM_GBPS, 5),
         },
         "points": points,
+        "mixed": mixed,
         "measured": {"copy_GBps": round(copy_gbps, 1), "library_gemm_8192_TFLOPs": round(gemm_tflops, 1)},
     }
     print(json.dumps(line))

@@ -115,12 +115,15 @@ class CacheManager:
 
     # ---- storage --------------------------------------------------------------------
     def allocate_storage(self, dtype, device) -> None:
-        """Per group a key pool ``[calls, pages, kv_heads, block_size, head_dim]`` and a
-        value pool ``[calls, pages, kv_heads, head_dim, block_size]`` (values lie
+        """Per group a key pool ``[calls, pages + 1, kv_heads, block_size, head_dim]`` and a
+        value pool ``[calls, pages + 1, kv_heads, head_dim, block_size]`` (values lie
         transposed inside a page: the matrix-core kernels read 4 consecutive keys
         of one column in one load), allocated once and never initialised (a page's content is read only below the
         committed length; reference: miniserve/kv/paged.py:39-41), and zeroed
-        state tensors ``[slots, *shape]``."""
+        state tensors ``[slots + 1, *shape]``.  The last page of a pool and the last
+        state slot are spare: no request ever holds them, and rows that only fill a
+        recorded step up to its size write there (:meth:`spare_page`,
+        :attr:`spare_state_slot`)."""
 
         import torch
 
@@ -128,13 +131,24 @@ class CacheManager:
         for group, count in zip(self.layout.groups, self.num_blocks):
             heads, dim = group.need.num_kv_heads, group.need.head_dim
             self.key_pools.append(
-                torch.empty((len(group.calls), count, heads, self.block_size, dim), dtype=dtype, device=device)
+                torch.empty((len(group.calls), count + 1, heads, self.block_size, dim), dtype=dtype, device=device)
             )
             self.value_pools.append(
-                torch.empty((len(group.calls), count, heads, dim, self.block_size), dtype=dtype, device=device)
+                torch.empty((len(group.calls), count + 1, heads, dim, self.block_size), dtype=dtype, device=device)
             )
         for need in self.layout.states:
-            self.state_tensors.append(torch.zeros((self.max_num_seqs, *need.shape), dtype=need.dtype, device=device))
+            self.state_tensors.append(torch.zeros((self.max_num_seqs + 1, *need.shape), dtype=need.dtype, device=device))
+
+    def spare_page(self, group: int) -> int:
+        """The page of ``group``'s pools that belongs to no request."""
+
+        return self.num_blocks[group]
+
+    @property
+    def spare_state_slot(self) -> int:
+        """The state slot that belongs to no request."""
+
+        return self.max_num_seqs
 
     def call_views(self) -> list:
         """The cache of every call of the run order: ``KVCacheView``, ``StateView`` or None."""

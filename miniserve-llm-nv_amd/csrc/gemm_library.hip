@@ -13,6 +13,7 @@
 #include <dlfcn.h>
 #include <hipblaslt/hipblaslt.h>
 
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -49,6 +50,20 @@ constexpr size_t kMaxPlans = 4096;
 
 constexpr int kCandidates = 8;
 constexpr int kTuneFromRows = 256;
+constexpr int kTuneBucketRows = 256;
+// The solution that timing chose for (device, n, k, out is float, m / kTuneBucketRows):
+// the first row count of a bucket is timed, the others take the same solution where
+// the library offers it for them, so that a stream of ever new row counts (portions
+// of prompts beside decode tokens) does not stop to time each of them.
+std::map<std::tuple<int, int, int, int, int>, int> g_tuned;
+
+// What the library itself calls the index of an algorithm: the first integer of its
+// opaque data.  Used only to recognise a candidate among those offered for a shape.
+int solution_index(const hipblasLtMatmulAlgo_t& algo) {
+  int index = 0;
+  std::memcpy(&index, algo.data, sizeof(index));
+  return index;
+}
 
 // Index of the candidate that runs this product fastest (two timed runs after a first
 // one).  The output goes to memory of its own, so that `out` is written once, by the call.
@@ -163,11 +178,24 @@ extern "C" int ms_gemm_library(const void* x, const void* w, void* out, int m, i
     MS_REQUIRE(status == HIPBLAS_STATUS_SUCCESS && returned > 0, "gemm_library: no algorithm for %d x %d x %d", m, n, k);
     int best = 0;
     // Many rows: the library's first choice is not always its fastest.  The candidates
-    // are timed once, on scratch output, unless the stream is recording (no waiting there).
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (m >= kTuneFromRows && returned > 1 && hipStreamIsCapturing(stream, &capture) == hipSuccess &&
-        capture == hipStreamCaptureStatusNone) {
-      best = fastest_candidate(handle, plan, result, returned, x, w, m, n, out_float, workspace, workspace_bytes, stream);
+    // are timed once for a bucket of row counts, on scratch output, unless the stream
+    // is recording (no waiting there).
+    if (m >= kTuneFromRows && returned > 1) {
+      const auto bucket = std::make_tuple(device, n, k, out_float, m / kTuneBucketRows);
+      const auto tuned = g_tuned.find(bucket);
+      hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+      if (tuned != g_tuned.end()) {
+        for (int i = 0; i < returned; ++i) {
+          if (result[i].state == HIPBLAS_STATUS_SUCCESS && result[i].workspaceSize <= workspace_bytes &&
+              solution_index(result[i].algo) == tuned->second) {
+            best = i;
+            break;
+          }
+        }
+      } else if (hipStreamIsCapturing(stream, &capture) == hipSuccess && capture == hipStreamCaptureStatusNone) {
+        best = fastest_candidate(handle, plan, result, returned, x, w, m, n, out_float, workspace, workspace_bytes, stream);
+        g_tuned[bucket] = solution_index(result[best].algo);
+      }
     }
     plan.algo = result[best].algo;
     plan.workspace = result[best].workspaceSize;

@@ -29,6 +29,21 @@ def _require_gpu(device: torch.device) -> None:
         raise RuntimeError("the engine runs on the GPU only (HIP kernels); no CPU path exists.")
 
 
+def recorded_batch_size(batch: int) -> int:
+    """The size of the recorded step that serves ``batch`` single tokens: itself up
+    to 8, then the next multiple of 4 up to 32, of 8 up to 128, of 16 beyond.  A
+    server's batch shrinks and grows by ones; recording a step for every size it
+    passes through would cost more than the few spare rows do."""
+
+    if batch <= 8:
+        return batch
+    step = 4 if batch <= 32 else 8 if batch <= 128 else 16
+    return -(-batch // step) * step
+
+
+_SPARE_ROW = object()       # marks a row of a host buffer that holds the values of a spare row
+
+
 class DecodeGraph:
     """One decode step of a fixed batch size, recorded as a HIP graph.
 
@@ -39,6 +54,11 @@ class DecodeGraph:
     memory) and replays.  Block tables have the static width of the longest
     request the engine admits.  The graph holds no memset node: nothing in the
     recorded step clears memory.
+
+    A step of fewer requests than ``batch`` fills the other rows with spare ones:
+    token 0 at position 0 of a sequence whose only page is the pools' spare page and
+    whose state slot is the spare slot.  They write and read nothing that a request
+    holds, and their logits are not returned.
     """
 
     def __init__(self, runner: "ModelRunner", batch: int) -> None:
@@ -109,14 +129,17 @@ class DecodeGraph:
             host[start : start + size] = values
 
         metas = reservation.sequences
-        put("positions", [meta.before for meta in metas])
-        put("seq_of_token", range(batch))
-        put("query_start", range(batch + 1))
-        put("context_lens", [meta.after for meta in metas])
-        put("state_slots", [meta.state_slot for meta in metas])
-        put("logit_rows", range(batch))
+        spare = batch - len(metas)
+        if spare < 0:
+            raise ValueError(f"{len(metas)} requests do not fit a recorded step of {batch}.")
         runner = self._runner()
         block_size = runner.block_size
+        put("positions", [meta.before for meta in metas] + [0] * spare)
+        put("seq_of_token", range(batch))
+        put("query_start", range(batch + 1))
+        put("context_lens", [meta.after for meta in metas] + [1] * spare)
+        put("state_slots", [meta.state_slot for meta in metas] + [runner.cache.spare_state_slot] * spare)
+        put("logit_rows", range(batch))
         for group in range(len(runner.cache.layout.groups)):
             pool_pages = runner.cache.num_blocks[group]
             slots = []
@@ -133,6 +156,12 @@ class DecodeGraph:
                     # a page that was given back is never read; 0 keeps the entry inside the pool
                     host[start + row * width : start + row * width + len(table)] = [p if p >= 0 else 0 for p in table]
                     row_tables[row] = table
+            spare_page = runner.cache.spare_page(group)
+            for row in range(len(metas), batch):
+                slots.append(spare_page * block_size)
+                if row_tables[row] is not _SPARE_ROW:
+                    host[start + row * width] = spare_page
+                    row_tables[row] = _SPARE_ROW
             put(f"slots{group}", slots)
 
     def prepare(self, reservation) -> int | None:
@@ -146,16 +175,17 @@ class DecodeGraph:
         return which
 
     def run(self, entries: Sequence[StepEntry], reservation, prepared: int | None = None) -> torch.Tensor:
-        """Logits ``[batch, vocab]`` of the step; the tensor is the graph's own output
-        buffer and holds these values until the next step of this batch size.
-        ``prepared``: the host buffer that :meth:`prepare` filled for this reservation."""
+        """Logits ``[len(entries), vocab]`` of the step; the tensor is a view of the
+        graph's own output buffer and holds these values until the next step of this
+        recorded size.  ``prepared``: the host buffer that :meth:`prepare` filled for
+        this reservation."""
 
         which = prepared
         if which is None:
             which = self._next_buffer()
             self._fill(reservation, which)
         start, size = self.offsets["token_ids"]
-        self.hosts_np[which][start : start + size] = [entry.token_ids[0] for entry in entries]
+        self.hosts_np[which][start : start + size] = [entry.token_ids[0] for entry in entries] + [0] * (size - len(entries))
         self.meta.copy_(self.hosts[which], non_blocking=True)
         runner = self._runner()
         model, views = runner.model, runner._call_views
@@ -181,7 +211,7 @@ class DecodeGraph:
             self.graph = graph
         self.graph.replay()
         self.replays += 1
-        return self.logits
+        return self.logits[: len(entries)]
 
 
 @dataclass(frozen=True)
@@ -293,11 +323,12 @@ class ModelRunner:
             if entry.token_ids[0] >= self.spec.vocab_size:
                 raise ValueError(f"entry {entry.request_id!r}: a token id is outside the vocabulary.")
         batch = len(entries)
-        graph = self._decode_graphs.get(batch)
+        recorded = recorded_batch_size(batch)
+        graph = self._decode_graphs.get(recorded)
         if graph is None:
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
-            graph = self._decode_graphs[batch] = DecodeGraph(self, batch)
+            graph = self._decode_graphs[recorded] = DecodeGraph(self, recorded)
         logits = graph.run(entries, reservation, prepared)
         wanted = [index for index, entry in enumerate(entries) if entry.want]
         if len(wanted) == batch:
@@ -324,7 +355,7 @@ class ModelRunner:
 
         if not self.engine_config.decode_graphs or not request_ids:
             return None
-        graph = self._decode_graphs.get(len(request_ids))
+        graph = self._decode_graphs.get(recorded_batch_size(len(request_ids)))
         if graph is None or graph.graph is None:
             return None
         items = []

@@ -305,3 +305,19 @@ def test_random_orders_lose_no_page(seed):
         m.release(name)
     m.assert_invariants()
     assert m.capacity().free_blocks == (12, 6) and m.capacity().free_slots == 3
+
+
+def test_a_spare_page_and_a_spare_state_slot_that_no_request_gets():
+    """Storage has one page and one state slot more than the manager hands out."""
+
+    import torch
+
+    made = manager([Need(0, KVCacheNeed(2, 4)), Need(1, StateNeed((3,)))], block_size=4, num_blocks=5, slots=2, max_len=20)
+    made.allocate_storage(torch.float32, "cpu")
+    assert made.key_pools[0].shape[1] == 6 and made.value_pools[0].shape[1] == 6
+    assert made.state_tensors[0].shape == (3, 3)
+    assert made.spare_page(0) == 5 and made.spare_state_slot == 2
+    assert {made.admit("a"), made.admit("b")} == {0, 1}
+    made.commit_step(made.prepare_step([StepItem("a", 0, 12), StepItem("b", 0, 8)]))
+    pages = set(made.block_table("a")) | set(made.block_table("b"))
+    assert pages == {0, 1, 2, 3, 4} and made.capacity().free_blocks == (0,)

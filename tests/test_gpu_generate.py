@@ -282,6 +282,66 @@ def test_decode_graphs_replay_like_eager_steps(dtype, model_folders):
     assert sorted(runners[0]._decode_graphs) == [1, 2, 3, 4]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_steps_filled_up_with_spare_rows(dtype, model_folders):
+    """Nine to eleven live requests are served by the recorded step of twelve: the rows
+    that fill it up write to the spare page and the spare state slot only, and every
+    request's logits are those of the eager step.  The pools are poisoned first, so
+    a spare row that read or wrote a request's page would show."""
+
+    from miniserve_amd.config import EngineConfig
+    from miniserve_amd.engine import ModelRunner, StepEntry
+    from miniserve_amd.engine.runner import recorded_batch_size
+
+    assert [recorded_batch_size(n) for n in (1, 7, 8, 9, 12, 13, 32, 33, 40, 128, 129)] == [
+        1, 7, 8, 12, 12, 16, 32, 40, 40, 128, 144]
+    folder, block = model_folders["b"]
+    config = read_config(folder)
+    runners = [
+        ModelRunner.from_folder(folder, EngineConfig(dtype=dtype, kv_block_size=block, num_kv_blocks=80, max_num_seqs=11,
+                                                    enable_chunked_prefill=True, decode_graphs=graphs))
+        for graphs in (True, False)
+    ]
+    for runner in runners:
+        for pool in (*runner.cache.key_pools, *runner.cache.value_pools):
+            pool.fill_(float("nan"))
+    names = [f"r{index}" for index in range(11)]
+    tokens = {name: random_tokens(60, config["vocab_size"], seed) for seed, name in enumerate(names)}
+    position = {name: 0 for name in names}
+
+    def both(entries_of):
+        outs = []
+        for runner in runners:
+            for name in entries_of:
+                if not runner.cache.is_live(name):
+                    runner.admit(name)
+            entries = [StepEntry(n, tuple(tokens[n][position[n] : position[n] + size]), (size - 1,)) for n, size in entries_of.items()]
+            outs.append(runner.step(entries).clone())
+            torch.cuda.synchronize()
+        for name, size in entries_of.items():
+            position[name] += size
+        assert outs[0].shape == (len(entries_of), config["vocab_size"]) and torch.isfinite(outs[0]).all()
+        if dtype == "float32":
+            assert torch.equal(outs[0], outs[1])
+        else:
+            torch.testing.assert_close(outs[0], outs[1], atol=2e-2, rtol=2e-2)
+
+    both({name: 3 + 2 * index for index, name in enumerate(names)})     # prompts of 3 to 23 tokens, eager
+    for _ in range(3):
+        both({name: 1 for name in names})                # eleven live: one spare row
+    for runner in runners:
+        runner.release("r4")                             # its pages go back; the rows below move up
+    for _ in range(10):
+        both({name: 1 for name in names if name != "r4"})
+    for runner in runners:
+        runner.release("r0")
+    for _ in range(10):
+        both({name: 1 for name in names if name not in ("r0", "r4")})    # nine live, across page edges of 8
+    assert sorted(runners[0]._decode_graphs) == [12] and runners[0].graph_steps == 23
+    cache = runners[0].cache
+    assert all(cache.spare_page(0) not in cache.block_table(name) for name in cache.live_requests())
+
+
 def test_a_dropped_runner_is_freed_at_once_and_recording_survives_a_collection(model_folders):
     """A runner's recorded steps hold no reference back to it: dropping the runner frees
     it, its graphs and its pinned memory without waiting for a collection of cycles -
