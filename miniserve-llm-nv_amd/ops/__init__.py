@@ -313,10 +313,12 @@ def attention(
 
 
 _EPILOGUE_BF16, _EPILOGUE_F32, _EPILOGUE_ADD_F32, _EPILOGUE_SILU_MUL = 0, 1, 2, 3
-# Rows up to which this library's product is used in bfloat16; the kernel takes up
-# to 64, but from 17 rows on the library product is faster (measured on MI355X at
-# the layer sizes of Qwen3-0.6B and 8B), so it serves those.
+# Rows up to which this library's product is always used in bfloat16.  The kernel
+# takes up to SKINNY_KERNEL_ROWS; from 17 rows on, which of the two products is the
+# faster one depends on the matrix (on MI355X: this one for the matrices of a small
+# model, hipBLASLt for large ones), so both are timed once for a shape.
 SKINNY_MAX_ROWS = 16
+SKINNY_KERNEL_ROWS = 64
 
 
 _GEMM_WORKSPACE_BYTES = 64 << 20
@@ -356,6 +358,53 @@ def _use_skinny(m: int, n: int, k: int, epilogue: int) -> bool:
     return m <= SKINNY_MAX_ROWS and bool(load().ms_gemm_skinny_supported(m, n, k, epilogue))
 
 
+# (device, blocks of 16 rows, n, k, gated) -> whether this library's product served a
+# timed call faster than hipBLASLt did (for ``gated``: than hipBLASLt and the activation kernel)
+_product_choice: dict[tuple[int, int, int, int, bool], bool] = {}
+
+
+def _elapsed_us(function, repeats: int = 8) -> float:
+    for _ in range(2):
+        function()
+    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record()
+    for _ in range(repeats):
+        function()
+    end.record()
+    end.synchronize()
+    return 1000.0 * begin.elapsed_time(end) / repeats
+
+
+def _skinny_for_some_rows(x: torch.Tensor, weight: torch.Tensor, gated: bool) -> bool:
+    """For 17 to ``SKINNY_KERNEL_ROWS`` rows: whether this library's product is the
+    faster one for this shape.  Both are timed at the first call for a shape, on
+    outputs of their own; while a stream records nothing is timed and nothing is
+    remembered, and the library product serves the call."""
+
+    m, k = x.shape
+    n = weight.shape[0]
+    epilogue = _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16
+    if not SKINNY_MAX_ROWS < m <= SKINNY_KERNEL_ROWS or not load().ms_gemm_skinny_supported(m, n, k, epilogue):
+        return False
+    index = x.device.index if x.device.index is not None else torch.cuda.current_device()
+    key = (index, -(-m // 16), n, k, gated)
+    choice = _product_choice.get(key)
+    if choice is None:
+        if torch.cuda.is_current_stream_capturing():
+            return False
+        ours = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=x.device)
+        theirs = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+
+        def library() -> None:
+            _library_product(x, weight, theirs, False)
+            if gated:
+                silu_mul(theirs)
+
+        choice = _elapsed_us(lambda: _skinny(x, weight, epilogue, ours)) < _elapsed_us(library)
+        _product_choice[key] = choice
+    return choice
+
+
 def _skinny(x: torch.Tensor, weight: torch.Tensor, epilogue: int, out: torch.Tensor) -> None:
     m, k = x.shape
     n = weight.shape[0]
@@ -376,7 +425,9 @@ def linear(
     float32: this library's FMA kernel (true 32-bit; row results do not depend on
     M).  bfloat16 with at most ``SKINNY_MAX_ROWS`` rows: this library's matrix-core
     kernel that streams the weights once; more rows: the library matrix product
-    (hipBLASLt, the copy that torch has loaded), both with 32-bit accumulation.  ``accumulate_into`` (float32
+    (hipBLASLt, the copy that torch has loaded); up to ``SKINNY_KERNEL_ROWS`` rows the
+    one of the two that was faster when the shape was first seen.  All with 32-bit
+    accumulation.  ``accumulate_into`` (float32
     ``[M, N]``) receives ``+=`` and is returned; ``out_float32`` returns the
     32-bit sums without a rounding to bfloat16 in between."""
 
@@ -393,7 +444,7 @@ def linear(
         call("ms_gemm_f32", _ptr(x), _ptr(weight), _ptr(out), m, n, k, int(accumulate_into is not None), _stream())
         return out
     _code(x.dtype)
-    if _use_skinny(m, n, k, _EPILOGUE_BF16):
+    if _use_skinny(m, n, k, _EPILOGUE_BF16) or _skinny_for_some_rows(x, weight, False):
         if accumulate_into is not None:
             _skinny(x, weight, _EPILOGUE_ADD_F32, accumulate_into)
             return accumulate_into
@@ -447,7 +498,7 @@ def linear_normed(
 
 def linear_silu_mul(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``silu(x Wg^T) * (x Wu^T)`` for ``weight [2 I, K]`` = gate rows, then up rows ->
-    ``[M, I]``.  bfloat16 with at most ``SKINNY_MAX_ROWS`` rows: one kernel, the
+    ``[M, I]``.  bfloat16 with few rows (as in :func:`linear`): one kernel, the
     activation in the product's epilogue; otherwise the product and :func:`silu_mul`."""
 
     _check(x, "x")
@@ -456,7 +507,7 @@ def linear_silu_mul(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         raise KernelError(f"linear_silu_mul: x {tuple(x.shape)} does not match weight {tuple(weight.shape)}.")
     m, k = x.shape
     n = weight.shape[0]
-    if x.dtype == torch.bfloat16 and _use_skinny(m, n, k, _EPILOGUE_SILU_MUL):
+    if x.dtype == torch.bfloat16 and (_use_skinny(m, n, k, _EPILOGUE_SILU_MUL) or _skinny_for_some_rows(x, weight, True)):
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
         _skinny(x, weight, _EPILOGUE_SILU_MUL, out)
         return out

@@ -564,12 +564,54 @@ def test_product_beyond_64_rows_uses_the_library(ops):
     torch.testing.assert_close(ops.linear_silu_mul(x, w[:32].contiguous()), ops.silu_mul(ops.linear(x, w[:32].contiguous())))
 
 
-@pytest.mark.parametrize("m,n,k", [(17, 509, 96), (65, 33, 60), (300, 1024, 200), (2048, 4096, 1024), (129, 300, 80)])
-def test_library_product_for_many_rows(ops, m, n, k):
-    """Beyond 16 rows the product goes to hipBLASLt, bound at run time to the copy the
-    process has: bfloat16 out, 32-bit out, and += into a 32-bit tensor; sizes off every
-    grid; the same shape again takes the kept plan."""
+@pytest.mark.parametrize("m,n,k", [(17, 512, 96), (40, 1024, 1024), (64, 300, 200)])
+def test_seventeen_to_sixty_four_rows_take_the_faster_of_the_two_products(ops, m, n, k, monkeypatch):
+    """The first call for a shape times both products and remembers which was faster;
+    either one gives the product, plain and with the gated activation; a call while a
+    stream records times nothing and remembers nothing."""
 
+    monkeypatch.setattr(ops, "_product_choice", {})
+    x, w = rand(m, k, seed=m, dtype=torch.bfloat16), rand(n, k, seed=n, dtype=torch.bfloat16, scale=0.1)
+    exact = x.cpu().double() @ w.cpu().double().T
+    scale = float(exact.abs().max())
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        recorded = ops.linear(x, w)
+    assert ops._product_choice == {}
+    graph.replay()
+    torch.cuda.synchronize()
+    torch.testing.assert_close(recorded.cpu().double(), exact, atol=scale * 2**-8, rtol=2**-7)
+
+    first = ops.linear(x, w)
+    gated_first = ops.linear_silu_mul(x, w)
+    keys = sorted(ops._product_choice)
+    assert [key[1:] for key in keys] == [(-(-m // 16), n, k, False), (-(-m // 16), n, k, True)]
+    results, gated = [], []
+    for choice in (True, False):
+        for key in keys:
+            ops._product_choice[key] = choice
+        results.append(ops.linear(x, w))
+        gated.append(ops.linear_silu_mul(x, w))
+        torch.testing.assert_close(results[-1].cpu().double(), exact, atol=scale * 2**-8, rtol=2**-7)
+        wide = ops.linear(x, w, out_float32=True)
+        torch.testing.assert_close(wide.cpu().double(), exact, atol=scale * 1e-5, rtol=1e-5)
+        total = torch.ones(m, n, device=DEVICE)
+        ops.linear(x, w, accumulate_into=total)
+        torch.testing.assert_close(total.cpu().double(), 1 + exact, atol=scale * 1e-5, rtol=1e-5)
+    assert any(torch.equal(first, result) for result in results)
+    assert any(torch.equal(gated_first, result) for result in gated)
+    # the activation of the rounded product, whichever kernel made it
+    assert torch.equal(gated[0], ops.silu_mul(results[0])) and torch.equal(gated[1], ops.silu_mul(results[1]))
+
+
+@pytest.mark.parametrize("m,n,k", [(17, 509, 96), (65, 33, 60), (300, 1024, 200), (2048, 4096, 1024), (129, 300, 80)])
+def test_library_product_for_many_rows(ops, m, n, k, monkeypatch):
+    """The product through hipBLASLt, bound at run time to the copy the process has:
+    bfloat16 out, 32-bit out, and += into a 32-bit tensor; sizes off every grid; the
+    same shape again takes the kept plan."""
+
+    monkeypatch.setattr(ops, "SKINNY_KERNEL_ROWS", 16)       # no choice between the two products here
     x, w = rand(m, k, seed=m, dtype=torch.bfloat16), rand(n, k, seed=n, dtype=torch.bfloat16, scale=0.1)
     exact = x.cpu().double() @ w.cpu().double().T
     scale = float(exact.abs().max())
@@ -589,10 +631,11 @@ def test_library_product_for_many_rows(ops, m, n, k):
         ops.linear(x, w, accumulate_into=torch.zeros(m, n + 1, device=DEVICE))
 
 
-def test_library_product_inside_a_recorded_graph(ops):
+def test_library_product_inside_a_recorded_graph(ops, monkeypatch):
     """Replayed several times with eager work between the replays; every replay gives
     what the eager call gives for the inputs of that moment."""
 
+    monkeypatch.setattr(ops, "SKINNY_KERNEL_ROWS", 16)
     x = rand(64, 256, seed=1, dtype=torch.bfloat16)
     w = rand(512, 256, seed=2, dtype=torch.bfloat16, scale=0.1)
     ops.linear(x, w)                                        # plan and workspace exist before the recording
