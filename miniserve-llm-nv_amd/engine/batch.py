@@ -12,6 +12,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Sequence
 
+import numpy as np
 import torch
 
 from ..cache.manager import StepReservation
@@ -56,91 +57,113 @@ def build_step_context(
     # the entries as given.
     layout = sorted(range(len(entries)), key=lambda i: len(entries[i].token_ids) != 1)
     decode_prefix = sum(1 for entry in entries if len(entry.token_ids) == 1)
-    base_of_entry = [0] * len(entries)
-    token_ids: list[int] = []
-    positions: list[int] = []
-    seq_of_token: list[int] = []
-    query_start = [0]
-    context_lens: list[int] = []
-    state_slots: list[int] = []
-    logit_rows: list[int] = []
-    query_lens: list[int] = []
-    first_positions: list[int] = []
+    metas_in_layout = [reservation.sequences[i] for i in layout]
     num_groups = len(pool_pages)
-    slot_mappings: list[list[int]] = [[] for _ in range(num_groups)]
-    widest = [1] * num_groups
+    s = len(entries)
+    query_lens = [len(entries[original].token_ids) for original in layout]
+    n = sum(query_lens)
+    num_tiles = sum(-(-length // QUERY_TILE) for length in query_lens[decode_prefix:])
+    num_rows = sum(len(entry.want) for entry in entries)
+    widest = [max(1, max(len(meta.block_tables[group]) for meta in metas_in_layout)) for group in range(num_groups)]
 
+    offsets: dict[str, tuple[int, int]] = {}
+    total = 0
+    sizes = [("token_ids", n), ("positions", n), ("seq_of_token", n), ("query_start", s + 1), ("context_lens", s),
+             ("state_slots", s), ("logit_rows", num_rows), ("tile_seq", num_tiles), ("tile_token", num_tiles),
+             ("tile_length", num_tiles)]
+    for group in range(num_groups):
+        sizes += [(f"slots{group}", n), (f"table{group}", s * widest[group])]
+    for name, size in sizes:
+        offsets[name] = (total, size)
+        total += size
+    on_gpu = torch.device(device).type == "cuda"
+    host = torch.empty(total, dtype=torch.int32, pin_memory=on_gpu)
+    numbers = host.numpy()
+
+    def region(name: str) -> np.ndarray:
+        start, size = offsets[name]
+        return numbers[start : start + size]
+
+    token_ids, positions, seq_of_token = region("token_ids"), region("positions"), region("seq_of_token")
+    slot_regions = [region(f"slots{group}") for group in range(num_groups)]
+    table_regions = [region(f"table{group}") for group in range(num_groups)]
+    for table_region in table_regions:
+        table_region[:] = 0
+    context_lens = [meta.after for meta in metas_in_layout]
+    state_slots = [meta.state_slot for meta in metas_in_layout]
+    first_positions = [meta.before for meta in metas_in_layout]
+    query_start = [0] * (s + 1)
+    base_of_entry = [0] * s
     tile_seq: list[int] = []
     tile_token: list[int] = []
     tile_length: list[int] = []
-    metas_in_layout = [reservation.sequences[i] for i in layout]
-    for index, original in enumerate(layout):
-        entry, meta = entries[original], reservation.sequences[original]
-        if entry.request_id != meta.request_id or len(entry.token_ids) != meta.after - meta.before:
-            raise ValueError(f"entry {entry.request_id!r} does not match its reservation.")
-        if any(token >= vocab_size for token in entry.token_ids):
-            raise ValueError(f"entry {entry.request_id!r}: a token id is outside the vocabulary of {vocab_size}.")
-        base = len(token_ids)
-        base_of_entry[original] = base
-        if index >= decode_prefix:
-            for start in range(0, len(entry.token_ids), QUERY_TILE):
-                tile_seq.append(index)
-                tile_token.append(base + start)
-                tile_length.append(min(QUERY_TILE, len(entry.token_ids) - start))
-        token_ids.extend(entry.token_ids)
-        positions.extend(range(meta.before, meta.after))
-        seq_of_token.extend([index] * len(entry.token_ids))
-        query_start.append(len(token_ids))
-        context_lens.append(meta.after)
-        state_slots.append(meta.state_slot)
-        query_lens.append(len(entry.token_ids))
-        first_positions.append(meta.before)
-        for group in range(num_groups):
-            table = meta.block_tables[group]
-            slots = meta.slot_mappings[group]
-            # slot == table[pos // bs] * bs + pos % bs, and the page lies in the pool
-            for position, slot in zip(range(meta.before, meta.after), slots):
-                page = table[position // block_size]
-                if not 0 <= page < pool_pages[group] or slot != page * block_size + position % block_size:
-                    raise RuntimeError(f"request {entry.request_id!r}: slot {slot} disagrees with its block table.")
-            slot_mappings[group].extend(slots)
-            widest[group] = max(widest[group], len(table))
 
+    for index, original in enumerate(layout):
+        entry, meta = entries[original], metas_in_layout[index]
+        length = query_lens[index]
+        if entry.request_id != meta.request_id or length != meta.after - meta.before:
+            raise ValueError(f"entry {entry.request_id!r} does not match its reservation.")
+        base = query_start[index]
+        query_start[index + 1] = base + length
+        base_of_entry[original] = base
+        if length == 1:
+            # one token: plain integers (an array per row would cost more than it saves)
+            token = entry.token_ids[0]
+            if token >= vocab_size:
+                raise ValueError(f"entry {entry.request_id!r}: a token id is outside the vocabulary of {vocab_size}.")
+            token_ids[base] = token
+            positions[base] = meta.before
+            seq_of_token[base] = index
+            logical, offset = divmod(meta.before, block_size)
+            for group in range(num_groups):
+                table = meta.block_tables[group]
+                slot = meta.slot_mappings[group][0]
+                page = table[logical]
+                # slot == table[pos // bs] * bs + pos % bs, and the page lies in the pool
+                if not 0 <= page < pool_pages[group] or slot != page * block_size + offset:
+                    raise RuntimeError(f"request {entry.request_id!r}: slot {slot} disagrees with its block table.")
+                slot_regions[group][base] = slot
+                start = index * widest[group]
+                table_regions[group][start : start + len(table)] = table
+            continue
+        tokens = np.asarray(entry.token_ids, dtype=np.int64)
+        if int(tokens.max()) >= vocab_size:
+            raise ValueError(f"entry {entry.request_id!r}: a token id is outside the vocabulary of {vocab_size}.")
+        token_ids[base : base + length] = tokens
+        run = np.arange(meta.before, meta.after, dtype=np.int64)
+        positions[base : base + length] = run
+        seq_of_token[base : base + length] = index
+        for start in range(0, length, QUERY_TILE):
+            tile_seq.append(index)
+            tile_token.append(base + start)
+            tile_length.append(min(QUERY_TILE, length - start))
+        logical, offset = np.divmod(run, block_size)
+        for group in range(num_groups):
+            table = np.asarray(meta.block_tables[group], dtype=np.int64)
+            slots = np.asarray(meta.slot_mappings[group], dtype=np.int64)
+            pages = table[logical]
+            agree = (pages >= 0) & (pages < pool_pages[group]) & (slots == pages * block_size + offset)
+            if not bool(agree.all()):
+                slot = int(slots[int(np.argmin(agree))])
+                raise RuntimeError(f"request {entry.request_id!r}: slot {slot} disagrees with its block table.")
+            slot_regions[group][base : base + length] = slots
+            start = index * widest[group]
+            table_regions[group][start : start + len(table)] = table
+    for table_region in table_regions:
+        # a page that was given back is never read; 0 keeps the entry inside the pool
+        np.maximum(table_region, 0, out=table_region)
+
+    logit_rows: list[int] = []
     for original, entry in enumerate(entries):
         logit_rows.extend(base_of_entry[original] + place for place in entry.want)
-
-    n, s = len(token_ids), len(entries)
-    packed: list[int] = []
-    offsets: dict[str, tuple[int, int]] = {}
-
-    def put(name: str, values: Sequence[int]) -> None:
-        offsets[name] = (len(packed), len(values))
-        packed.extend(values)
-
-    put("token_ids", token_ids)
-    put("positions", positions)
-    put("seq_of_token", seq_of_token)
-    put("query_start", query_start)
-    put("context_lens", context_lens)
-    put("state_slots", state_slots)
-    put("logit_rows", logit_rows)
-    put("tile_seq", tile_seq)
-    put("tile_token", tile_token)
-    put("tile_length", tile_length)
-    for group in range(num_groups):
-        put(f"slots{group}", slot_mappings[group])
-        flat: list[int] = []
-        for meta in metas_in_layout:
-            table = meta.block_tables[group]
-            # a page that was given back is never read; 0 keeps the entry inside the pool
-            flat.extend(page if page >= 0 else 0 for page in table)
-            flat.extend([0] * (widest[group] - len(table)))
-        put(f"table{group}", flat)
-
-    host = torch.tensor(packed, dtype=torch.int32)
-    if torch.device(device).type == "cuda":
-        host = host.pin_memory()
-    buffer = host.to(device, non_blocking=True)
+    region("query_start")[:] = query_start
+    region("context_lens")[:] = context_lens
+    region("state_slots")[:] = state_slots
+    region("logit_rows")[:] = logit_rows
+    region("tile_seq")[:] = tile_seq
+    region("tile_token")[:] = tile_token
+    region("tile_length")[:] = tile_length
+    buffer = host.to(device, non_blocking=True) if on_gpu else host
 
     def view(name: str) -> torch.Tensor:
         start, length = offsets[name]

@@ -206,22 +206,20 @@ class Engine:
         for item in plan.prefill_items:
             self._sequences[item.request_id].commit_prefill(item.token_end)
         outputs: list[StepOutput] = []
-        ended = False
+        planned = set() if next_ahead is None else {item.request_id for item in next_ahead.plan.decode_items}
         for state, sample in zip(sampled, staged):
             state.append_sampled_token(sample.token_id)
             reason = state.should_finish()
             if reason is not None:
-                if next_ahead is not None:
+                if next_ahead is not None and state.request_id in planned:
                     # a request of the step that was planned ahead ends (a stop token): that
                     # step's reservation goes back before the request's pages can
                     self.runner.discard(next_ahead.prepared)
                     next_ahead = None
-                ended = True
                 state.finish(reason)
                 self._finalize(state)
             outputs.append(StepOutput(state.request_id, sample.token_id, reason is not None, reason))
-        if next_ahead is not None and not ended:
-            self._ahead = next_ahead
+        self._ahead = next_ahead
         return outputs
 
     # ---- the next step, planned while the GPU runs this one -------------------------------
@@ -235,10 +233,11 @@ class Engine:
         return ahead
 
     def _prepare_step_ahead(self, plan: ExecutionPlan, sampled: Sequence[SequenceState]) -> "_StepAhead | None":
-        """When every request decodes and none can end by length, the next step is this one
-        again with each request one token further: it is scheduled from views that say so,
-        its cache transaction is opened and its numbers are written now, and only the token
-        ids are left for when they are known.  Anything else is left to the next call."""
+        """When every request decodes, the next step is this one again with each request one
+        token further and without those that end by length now: it is scheduled from views
+        that say so, its cache transaction is opened and its numbers are written now, and
+        only the token ids are left for when they are known.  Anything else is left to the
+        next call."""
 
         prepare = getattr(self.runner, "prepare_decode", None)
         if prepare is None or plan.prefill_items or plan.preempted or len(plan.decode_items) != len(self._sequences):
@@ -246,7 +245,7 @@ class Engine:
         views = []
         for state in sampled:
             if len(state.generated_token_ids) + 1 >= state.sampling_params.max_new_tokens:
-                return None
+                continue                # ends with the token sampled now
             views.append(
                 SequenceView(
                     request_id=state.request_id,
@@ -262,6 +261,8 @@ class Engine:
                     num_preemptions=state.num_preemptions,
                 )
             )
+        if not views:
+            return None
         next_plan = self.scheduler.schedule(views, self.runner.cache.capacity())
         if next_plan.prefill_items or next_plan.preempted or len(next_plan.decode_items) != len(views):
             return None

@@ -329,7 +329,18 @@ def test_steps_planned_ahead_change_no_token():
     runner.prepare_ahead = True
     assert engine.generate(PROMPTS, params) == expected
     assert runner.used_ahead >= 8 and runner.discarded_ahead == 0       # all four decode together for ten steps
-    assert runner.prepared_ahead == runner.used_ahead                  # the last steps end by length: not planned ahead
+    assert runner.prepared_ahead == runner.used_ahead                  # the last step ends all by length: nothing to plan
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
+    runner.cache.assert_invariants()
+
+    # requests that end by length at different steps: the step after goes on without them, planned ahead
+    lengths = (5, 12, 8, 10)
+    engine, runner = make_engine()
+    runner.prepare_ahead = True
+    got = engine.generate(PROMPTS, [SamplingParams(max_new_tokens=n) for n in lengths])
+    assert got == [tokens[:n] for tokens, n in zip(expected, lengths)]
+    assert runner.discarded_ahead == 0 and runner.prepared_ahead == runner.used_ahead
+    assert runner.used_ahead >= 9                                       # eleven decode steps, the first not foreseen
     assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
     runner.cache.assert_invariants()
 
