@@ -6,6 +6,8 @@ torch is the allocator and gives the stream.
 
 from __future__ import annotations
 
+import gc
+
 import torch
 
 from .library import KernelError, call, library_path, load
@@ -361,25 +363,43 @@ def _use_skinny(m: int, n: int, k: int, epilogue: int) -> bool:
 # (device, blocks of 16 rows, n, k, gated) -> whether this library's product served a
 # timed call faster than hipBLASLt did (for ``gated``: than hipBLASLt and the activation kernel)
 _product_choice: dict[tuple[int, int, int, int, bool], bool] = {}
+_COLD_BYTES = 768 << 20
 
 
-def _elapsed_us(function, repeats: int = 8) -> float:
-    for _ in range(2):
-        function()
+def _recorded_us(function, calls: int, replays: int = 4) -> float:
+    """Microseconds of one of ``function(0) .. function(calls - 1)`` inside a recorded
+    graph: what the call costs the GPU where few rows are at home, in recorded decode
+    steps, without the host's share of a launch.  No collection of cycles while the
+    stream records (a free inside a recording aborts the process)."""
+
+    function(0)                     # plans and workspaces exist before the recording
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    collecting = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            for index in range(calls):
+                function(index)
+    finally:
+        if collecting:
+            gc.enable()
+    graph.replay()
     begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     begin.record()
-    for _ in range(repeats):
-        function()
+    for _ in range(replays):
+        graph.replay()
     end.record()
     end.synchronize()
-    return 1000.0 * begin.elapsed_time(end) / repeats
+    return 1000.0 * begin.elapsed_time(end) / (replays * calls)
 
 
 def _skinny_for_some_rows(x: torch.Tensor, weight: torch.Tensor, gated: bool) -> bool:
     """For 17 to ``SKINNY_KERNEL_ROWS`` rows: whether this library's product is the
-    faster one for this shape.  Both are timed at the first call for a shape, on
-    outputs of their own; while a stream records nothing is timed and nothing is
-    remembered, and the library product serves the call."""
+    faster one for this shape.  Both are timed at the first call for a shape, as
+    recorded graphs over copies of the matrix, on outputs of their own; while a stream
+    records nothing is timed and nothing is remembered, and the library product
+    serves the call."""
 
     m, k = x.shape
     n = weight.shape[0]
@@ -392,15 +412,22 @@ def _skinny_for_some_rows(x: torch.Tensor, weight: torch.Tensor, gated: bool) ->
     if choice is None:
         if torch.cuda.is_current_stream_capturing():
             return False
-        ours = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=x.device)
-        theirs = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+        # As in a decode step, every call streams a matrix that no cache holds: copies
+        # of the matrix, more of them than the card's last-level cache takes.
+        calls = min(128, max(4, -(-_COLD_BYTES // (weight.numel() * weight.element_size()))))
+        try:
+            matrices = [weight] + [weight.clone() for _ in range(calls - 1)]
+            ours = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=x.device)
+            theirs = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+        except torch.OutOfMemoryError:
+            return False
 
-        def library() -> None:
-            _library_product(x, weight, theirs, False)
+        def library(index: int) -> None:
+            _library_product(x, matrices[index], theirs, False)
             if gated:
                 silu_mul(theirs)
 
-        choice = _elapsed_us(lambda: _skinny(x, weight, epilogue, ours)) < _elapsed_us(library)
+        choice = _recorded_us(lambda index: _skinny(x, matrices[index], epilogue, ours), calls) < _recorded_us(library, calls)
         _product_choice[key] = choice
     return choice
 
