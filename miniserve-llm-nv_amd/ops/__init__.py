@@ -315,12 +315,14 @@ def attention(
 
 
 _EPILOGUE_BF16, _EPILOGUE_F32, _EPILOGUE_ADD_F32, _EPILOGUE_SILU_MUL = 0, 1, 2, 3
-# Rows up to which this library's product is always used in bfloat16.  The kernel
-# takes up to SKINNY_KERNEL_ROWS; from 17 rows on, which of the two products is the
-# faster one depends on the matrix (on MI355X: this one for the matrices of a small
-# model, hipBLASLt for large ones), so both are timed once for a shape.
+# This library's product takes up to SKINNY_KERNEL_ROWS rows.  Up to SKINNY_MAX_ROWS
+# rows and for a matrix below SKINNY_ALWAYS_BYTES it is always the faster one; beyond
+# either, which of the two products is faster depends on the matrix (on MI355X: this
+# one for the matrices of a small model, hipBLASLt for most large ones), so both are
+# timed once for a shape.
 SKINNY_MAX_ROWS = 16
 SKINNY_KERNEL_ROWS = 64
+SKINNY_ALWAYS_BYTES = 32 << 20
 
 
 _GEMM_WORKSPACE_BYTES = 64 << 20
@@ -394,33 +396,36 @@ def _recorded_us(function, calls: int, replays: int = 4) -> float:
     return 1000.0 * begin.elapsed_time(end) / (replays * calls)
 
 
-def _skinny_for_some_rows(x: torch.Tensor, weight: torch.Tensor, gated: bool) -> bool:
-    """For 17 to ``SKINNY_KERNEL_ROWS`` rows: whether this library's product is the
+def _skinny_is_faster(x: torch.Tensor, weight: torch.Tensor, gated: bool) -> bool:
+    """For up to ``SKINNY_KERNEL_ROWS`` rows: whether this library's product is the
     faster one for this shape.  Both are timed at the first call for a shape, as
     recorded graphs over copies of the matrix, on outputs of their own; while a stream
-    records nothing is timed and nothing is remembered, and the library product
-    serves the call."""
+    records nothing is timed and nothing is remembered, and the call is served as it
+    was before there was a choice (this library's product up to ``SKINNY_MAX_ROWS``
+    rows)."""
 
     m, k = x.shape
     n = weight.shape[0]
     epilogue = _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16
-    if not SKINNY_MAX_ROWS < m <= SKINNY_KERNEL_ROWS or not load().ms_gemm_skinny_supported(m, n, k, epilogue):
+    if m > SKINNY_KERNEL_ROWS or not load().ms_gemm_skinny_supported(m, n, k, epilogue):
         return False
+    if m <= SKINNY_MAX_ROWS and (gated or weight.numel() * weight.element_size() < SKINNY_ALWAYS_BYTES):
+        return True
     index = x.device.index if x.device.index is not None else torch.cuda.current_device()
     key = (index, -(-m // 16), n, k, gated)
     choice = _product_choice.get(key)
     if choice is None:
         if torch.cuda.is_current_stream_capturing():
-            return False
+            return m <= SKINNY_MAX_ROWS
         # As in a decode step, every call streams a matrix that no cache holds: copies
         # of the matrix, more of them than the card's last-level cache takes.
-        calls = min(128, max(4, -(-_COLD_BYTES // (weight.numel() * weight.element_size()))))
+        calls = min(128, max(2, -(-_COLD_BYTES // (weight.numel() * weight.element_size()))))
         try:
             matrices = [weight] + [weight.clone() for _ in range(calls - 1)]
             ours = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=x.device)
             theirs = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
         except torch.OutOfMemoryError:
-            return False
+            return m <= SKINNY_MAX_ROWS
 
         def library(index: int) -> None:
             _library_product(x, matrices[index], theirs, False)
@@ -471,7 +476,7 @@ def linear(
         call("ms_gemm_f32", _ptr(x), _ptr(weight), _ptr(out), m, n, k, int(accumulate_into is not None), _stream())
         return out
     _code(x.dtype)
-    if _use_skinny(m, n, k, _EPILOGUE_BF16) or _skinny_for_some_rows(x, weight, False):
+    if _skinny_is_faster(x, weight, False):
         if accumulate_into is not None:
             _skinny(x, weight, _EPILOGUE_ADD_F32, accumulate_into)
             return accumulate_into
@@ -534,7 +539,7 @@ def linear_silu_mul(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         raise KernelError(f"linear_silu_mul: x {tuple(x.shape)} does not match weight {tuple(weight.shape)}.")
     m, k = x.shape
     n = weight.shape[0]
-    if x.dtype == torch.bfloat16 and (_use_skinny(m, n, k, _EPILOGUE_SILU_MUL) or _skinny_for_some_rows(x, weight, True)):
+    if x.dtype == torch.bfloat16 and _skinny_is_faster(x, weight, True):
         out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
         _skinny(x, weight, _EPILOGUE_SILU_MUL, out)
         return out
