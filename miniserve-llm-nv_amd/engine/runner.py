@@ -30,13 +30,13 @@ def _require_gpu(device: torch.device) -> None:
 
 
 def recorded_batch_size(batch: int) -> int:
-    """The size of the recorded step that serves ``batch`` single tokens: itself up
-    to 8, then the next multiple of 4 up to 32, of 8 up to 128, of 16 beyond.  A
-    server's batch shrinks and grows by ones; recording a step for every size it
-    passes through would cost more than the few spare rows do."""
+    """The size of the recorded step that serves ``batch`` single tokens: 1, 2, 4, 8,
+    then the next multiple of 4 up to 32, of 8 up to 128, of 16 beyond.  A server's
+    batch shrinks and grows by ones; recording a step for every size it passes
+    through would cost more than the few spare rows do."""
 
     if batch <= 8:
-        return batch
+        return 1 << (batch - 1).bit_length()
     step = 4 if batch <= 32 else 8 if batch <= 128 else 16
     return -(-batch // step) * step
 
@@ -200,7 +200,6 @@ class DecodeGraph:
             # owners left behind (pinned memory, other graphs), and a free is not allowed
             # inside a recording - the process would abort.
             collecting = gc.isenabled()
-            gc.collect()
             gc.disable()
             try:
                 with torch.cuda.graph(graph, pool=runner._graph_pool):
