@@ -39,6 +39,39 @@ class StepEntry:
             raise ValueError(f"entry {self.request_id!r}: wanted places must index its tokens.")
 
 
+@dataclass
+class BuiltStep:
+    """A step's tensors, made but not yet sent: the context's tensors are views of
+    ``buffer``, which holds nothing before :meth:`send`.  Token ids of entries that
+    bring one token may still be set until then."""
+
+    ctx: StepContext
+    rows: torch.Tensor | None
+    request_ids: tuple[str, ...]
+    query_lens_of_entries: tuple[int, ...]
+    vocab_size: int
+    _host: torch.Tensor
+    _buffer: torch.Tensor
+    _token_places: tuple[int, ...]        # of each entry's first token, in the host buffer
+    _sent: bool = False
+
+    def set_single_token(self, entry_index: int, token: int) -> None:
+        if self._sent or self.query_lens_of_entries[entry_index] != 1:
+            raise RuntimeError("only a single token of a step that is not sent yet can be set.")
+        if not 0 <= token < self.vocab_size:
+            raise ValueError(
+                f"entry {self.request_ids[entry_index]!r}: a token id is outside the vocabulary of {self.vocab_size}."
+            )
+        self._host[self._token_places[entry_index]] = token
+
+    def send(self) -> None:
+        if self._sent:
+            raise RuntimeError("the step was sent already.")
+        if self._buffer is not self._host:
+            self._buffer.copy_(self._host, non_blocking=True)
+        self._sent = True
+
+
 def build_step_context(
     entries: Sequence[StepEntry],
     reservation: StepReservation,
@@ -48,8 +81,27 @@ def build_step_context(
     vocab_size: int,
     device: torch.device | str,
 ) -> tuple[StepContext, torch.Tensor | None]:
-    """All integer metadata of the step is packed into one host buffer and sent to
-    the device in one copy; the context's tensors are views of it."""
+    """The step's tensors, sent: see :func:`build_step`."""
+
+    built = build_step(
+        entries, reservation, block_size=block_size, pool_pages=pool_pages, vocab_size=vocab_size, device=device
+    )
+    built.send()
+    return built.ctx, built.rows
+
+
+def build_step(
+    entries: Sequence[StepEntry],
+    reservation: StepReservation,
+    *,
+    block_size: int,
+    pool_pages: Sequence[int],
+    vocab_size: int,
+    device: torch.device | str,
+) -> BuiltStep:
+    """All integer metadata of the step is packed into one host buffer that goes to
+    the device in one copy (:meth:`BuiltStep.send`); the context's tensors are views
+    of the device buffer."""
 
     if len(entries) != len(reservation.sequences):
         raise ValueError("entries and reservation disagree.")
@@ -163,7 +215,7 @@ def build_step_context(
     region("tile_seq")[:] = tile_seq
     region("tile_token")[:] = tile_token
     region("tile_length")[:] = tile_length
-    buffer = host.to(device, non_blocking=True) if on_gpu else host
+    buffer = torch.empty(total, dtype=torch.int32, device=device) if on_gpu else host
 
     def view(name: str) -> torch.Tensor:
         start, length = offsets[name]
@@ -192,4 +244,14 @@ def build_step_context(
         tiles=QueryTiles(len(tile_seq), view("tile_seq"), view("tile_token"), view("tile_length")) if tile_seq else None,
     )
     rows = view("logit_rows") if logit_rows else None
-    return ctx, rows
+    token_start = offsets["token_ids"][0]
+    return BuiltStep(
+        ctx=ctx,
+        rows=rows,
+        request_ids=tuple(entry.request_id for entry in entries),
+        query_lens_of_entries=tuple(len(entry.token_ids) for entry in entries),
+        vocab_size=vocab_size,
+        _host=host,
+        _buffer=buffer,
+        _token_places=tuple(token_start + base for base in base_of_entry),
+    )

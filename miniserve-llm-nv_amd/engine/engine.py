@@ -163,7 +163,8 @@ class Engine:
         for item in plan.prefill_items:
             state = self._sequences[item.request_id]
             if state.status is RequestStatus.WAITING:
-                self.runner.admit(item.request_id)
+                if not self.runner.cache.is_live(item.request_id):       # (a step planned ahead admitted it)
+                    self.runner.admit(item.request_id)
                 state.begin_prefill()
             tokens = state.tokens_between(item.token_start, item.token_end)
             final = item.token_end == state.prefill_target
@@ -207,6 +208,7 @@ class Engine:
             self._sequences[item.request_id].commit_prefill(item.token_end)
         outputs: list[StepOutput] = []
         planned = set() if next_ahead is None else {item.request_id for item in next_ahead.plan.decode_items}
+        # (the requests of its prompt portions are not sampled now and cannot end now)
         for state, sample in zip(sampled, staged):
             state.append_sampled_token(sample.token_id)
             reason = state.should_finish()
@@ -233,41 +235,64 @@ class Engine:
         return ahead
 
     def _prepare_step_ahead(self, plan: ExecutionPlan, sampled: Sequence[SequenceState]) -> "_StepAhead | None":
-        """When every request decodes, the next step is this one again with each request one
-        token further and without those that end by length now: it is scheduled from views
-        that say so, its cache transaction is opened and its numbers are written now, and
-        only the token ids are left for when they are known.  Anything else is left to the
-        next call."""
+        """The step after the running one, as far as it can be foreseen: every request as
+        the running step will leave it, each sampled one a token further (the token itself
+        not known yet) and without those that end by length now.  It is scheduled from
+        views that say so, its cache transaction is opened and its numbers are written
+        now; only the sampled token ids are left for when they are known.  A step of
+        single tokens goes to the recorded step's second host buffer, any other has its
+        tensors built.  A plan that would preempt is left to the next call, and so is one
+        that could make use of what a request that ends now gives back."""
 
-        prepare = getattr(self.runner, "prepare_decode", None)
-        if prepare is None or plan.prefill_items or plan.preempted or len(plan.decode_items) != len(self._sequences):
+        prepare_decode = getattr(self.runner, "prepare_decode", None)
+        prepare_step = getattr(self.runner, "prepare_step", None)
+        if prepare_decode is None or plan.preempted:
             return None
+        sampled_ids = {state.request_id for state in sampled}
+        prefill_end = {item.request_id: item.token_end for item in plan.prefill_items}
+        decoded = {item.request_id for item in plan.decode_items}
         views = []
-        for state in sampled:
-            if len(state.generated_token_ids) + 1 >= state.sampling_params.max_new_tokens:
-                continue                # ends with the token sampled now
+        ending = False
+        for state in self._sequences.values():
+            is_sampled = state.request_id in sampled_ids
+            if is_sampled and len(state.generated_token_ids) + 1 >= state.sampling_params.max_new_tokens:
+                ending = True           # ends with the token sampled now
+                continue
             views.append(
-                SequenceView(
-                    request_id=state.request_id,
-                    status=RequestStatus.DECODING,
-                    prefill_target=state.prefill_target,
-                    prefill_cursor=state.prefill_cursor,
-                    computed_tokens=state.computed_tokens + 1,
-                    total_tokens=state.total_tokens + 1,
-                    num_generated=len(state.generated_token_ids) + 1,
-                    max_new_tokens=state.sampling_params.max_new_tokens,
-                    arrival_ns=state.arrival_ns,
-                    next_input_token_id=0,          # not known yet; the step reads it from the request
-                    num_preemptions=state.num_preemptions,
+                state.view_after(
+                    prefill_end=prefill_end.get(state.request_id),
+                    decoded=state.request_id in decoded,
+                    sampled=is_sampled,
                 )
             )
         if not views:
             return None
         next_plan = self.scheduler.schedule(views, self.runner.cache.capacity())
-        if next_plan.prefill_items or next_plan.preempted or len(next_plan.decode_items) != len(views):
+        if next_plan.preempted or next_plan.empty:
+            return None
+        if ending and (next_plan.prefill_items or len(next_plan.decode_items) != len(views)):
+            # the pages and the slot of a request that ends now are not free yet; a plan
+            # made without them may hold less than the one made when they are
             return None
         try:
-            prepared = prepare([item.request_id for item in next_plan.decode_items])
+            if not next_plan.prefill_items:
+                prepared = prepare_decode([item.request_id for item in next_plan.decode_items])
+            elif prepare_step is not None:
+                entries, admit = [], []
+                for item in next_plan.decode_items:
+                    state = self._sequences[item.request_id]
+                    token = 0 if item.request_id in sampled_ids else state.token_at(state.computed_tokens)
+                    entries.append(StepEntry(item.request_id, (token,), (0,)))
+                for item in next_plan.prefill_items:
+                    state = self._sequences[item.request_id]
+                    if not self.runner.cache.is_live(item.request_id):
+                        admit.append(item.request_id)
+                    tokens = state.tokens_between(item.token_start, item.token_end)
+                    final = item.token_end == state.prefill_target
+                    entries.append(StepEntry(item.request_id, tuple(tokens), (len(tokens) - 1,) if final else ()))
+                prepared = prepare_step(entries, admit)
+            else:
+                prepared = None
         except OutOfPagesError:
             return None                # the plan's page count was an estimate; the next call decides
         if prepared is None:

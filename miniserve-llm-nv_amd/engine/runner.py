@@ -21,7 +21,7 @@ from ..config import EngineConfig, load_config
 from ..parts.model import TORCH_DTYPES, DecoderModel
 from ..weights import WeightLoadReport, load_weights, random_device_tensors
 from ..parts.base import GroupStepView, StepContext
-from .batch import StepEntry, build_step_context
+from .batch import BuiltStep, StepEntry, build_step
 
 
 def _require_gpu(device: torch.device) -> None:
@@ -223,6 +223,18 @@ class PreparedDecode:
     buffer: int
 
 
+@dataclass(frozen=True)
+class PreparedStep:
+    """Any other step whose cache transaction is open and whose tensors are made, but
+    for the single tokens that were not known yet; ``admitted``: the requests that
+    were admitted for it."""
+
+    request_ids: tuple[str, ...]
+    reservation: object
+    built: BuiltStep
+    admitted: tuple[str, ...]
+
+
 class ModelRunner:
     """Owns the model, its weights and the cache; offers ``step``."""
 
@@ -270,6 +282,7 @@ class ModelRunner:
         self.tokens_run = 0
         self.graph_steps = 0
         self.prepared_steps = 0        # steps whose numbers were written while the step before ran
+        self.prepared_mixed_steps = 0  # those of them that are not recorded steps
 
     # ---- construction -----------------------------------------------------------------
     @classmethod
@@ -369,10 +382,45 @@ class ModelRunner:
             raise
         return PreparedDecode(tuple(request_ids), reservation, buffer)
 
-    def discard(self, prepared: "PreparedDecode") -> None:
-        """Gives back what :meth:`prepare_decode` took."""
+    def prepare_step(self, entries: Sequence[StepEntry], admit: Sequence[str] = ()) -> "PreparedStep":
+        """Opens the cache transaction of a coming step and makes its tensors, without
+        sending them: entries that bring one token may bring any token id here, the
+        true one is taken from the entries that :meth:`step` gets.  ``admit``: requests
+        of the step that are not admitted yet.  On an exception nothing is kept."""
+
+        admitted: list[str] = []
+        try:
+            for request_id in admit:
+                self.admit(request_id)
+                admitted.append(request_id)
+            reservation = self._open_step(entries)
+            try:
+                built = build_step(
+                    entries, reservation, block_size=self.block_size, pool_pages=self.cache.num_blocks,
+                    vocab_size=self.spec.vocab_size, device=self.device,
+                )
+            except BaseException:
+                self.cache.abort_step(reservation)
+                raise
+        except BaseException:
+            for request_id in admitted:
+                self.release(request_id)
+            raise
+        return PreparedStep(tuple(entry.request_id for entry in entries), reservation, built, tuple(admitted))
+
+    def discard(self, prepared: "PreparedDecode | PreparedStep") -> None:
+        """Gives back what :meth:`prepare_decode` or :meth:`prepare_step` took."""
 
         self.cache.abort_step(prepared.reservation)
+        for request_id in getattr(prepared, "admitted", ()):
+            self.release(request_id)
+
+    def _open_step(self, entries: Sequence[StepEntry]):
+        items = []
+        for entry in entries:
+            start = self.cache.committed_tokens(entry.request_id)
+            items.append(StepItem(entry.request_id, start, start + len(entry.token_ids)))
+        return self.cache.prepare_step(items)
 
     @torch.inference_mode()
     def step(self, entries: Sequence[StepEntry], prepared: "PreparedDecode | None" = None) -> torch.Tensor | None:
@@ -385,6 +433,8 @@ class ModelRunner:
 
         if not entries:
             raise ValueError("a step needs at least one entry.")
+        if isinstance(prepared, PreparedStep):
+            return self._run_prepared_step(entries, prepared)
         if prepared is not None:
             if tuple(entry.request_id for entry in entries) != prepared.request_ids or any(
                 len(entry.token_ids) != 1 for entry in entries
@@ -394,11 +444,7 @@ class ModelRunner:
             reservation = prepared.reservation
             self.prepared_steps += 1
         else:
-            items = []
-            for entry in entries:
-                start = self.cache.committed_tokens(entry.request_id)
-                items.append(StepItem(entry.request_id, start, start + len(entry.token_ids)))
-            reservation = self.cache.prepare_step(items)
+            reservation = self._open_step(entries)
         if self.engine_config.decode_graphs and all(len(entry.token_ids) == 1 for entry in entries):
             try:
                 logits = self._decode_graph_step(entries, reservation, None if prepared is None else prepared.buffer)
@@ -411,7 +457,7 @@ class ModelRunner:
             self.graph_steps += 1
             return logits
         try:
-            ctx, rows = build_step_context(
+            built = build_step(
                 entries,
                 reservation,
                 block_size=self.block_size,
@@ -419,11 +465,36 @@ class ModelRunner:
                 vocab_size=self.spec.vocab_size,
                 device=self.device,
             )
-            logits = self.model.forward(ctx, self._call_views, rows)
+            built.send()
+            logits = self.model.forward(built.ctx, self._call_views, built.rows)
         except BaseException:
             self.cache.abort_step(reservation)
             raise
         self.cache.commit_step(reservation)
         self.steps_run += 1
-        self.tokens_run += ctx.num_tokens
+        self.tokens_run += built.ctx.num_tokens
+        return logits
+
+    def _run_prepared_step(self, entries: Sequence[StepEntry], prepared: PreparedStep) -> torch.Tensor | None:
+        """The step that :meth:`prepare_step` made, with the single tokens of ``entries``."""
+
+        built = prepared.built
+        try:
+            if tuple(entry.request_id for entry in entries) != prepared.request_ids or tuple(
+                len(entry.token_ids) for entry in entries
+            ) != built.query_lens_of_entries:
+                raise ValueError("the entries are not those the step was prepared for.")
+            for index, entry in enumerate(entries):
+                if len(entry.token_ids) == 1:
+                    built.set_single_token(index, entry.token_ids[0])
+            built.send()
+            logits = self.model.forward(built.ctx, self._call_views, built.rows)
+        except BaseException:
+            self.cache.abort_step(prepared.reservation)
+            raise
+        self.cache.commit_step(prepared.reservation)
+        self.steps_run += 1
+        self.tokens_run += built.ctx.num_tokens
+        self.prepared_steps += 1
+        self.prepared_mixed_steps += 1
         return logits

@@ -117,6 +117,35 @@ class SequenceState:
             num_preemptions=self.num_preemptions,
         )
 
+    def view_after(self, *, prefill_end: int | None = None, decoded: bool = False, sampled: bool = False) -> SequenceView:
+        """What :meth:`snapshot` will give once a running step is done: a step that ran
+        this request's prompt up to ``prefill_end``, or its pending token
+        (``decoded``), and that samples a token for it (``sampled``) which is not
+        known yet, so ``next_input_token_id`` is 0 in its place."""
+
+        computed = self.computed_tokens + 1 if decoded else self.computed_tokens if prefill_end is None else prefill_end
+        if sampled:
+            status = RequestStatus.DECODING
+        elif prefill_end is not None:
+            status = RequestStatus.PREFILLING
+        else:
+            status = self.status
+        return SequenceView(
+            request_id=self.request_id,
+            status=status,
+            prefill_target=self.prefill_target,
+            prefill_cursor=self.prefill_cursor if prefill_end is None else prefill_end,
+            computed_tokens=computed,
+            total_tokens=self.total_tokens + int(sampled),
+            num_generated=len(self.generated_token_ids) + int(sampled),
+            max_new_tokens=self.sampling_params.max_new_tokens,
+            arrival_ns=self.arrival_ns,
+            next_input_token_id=(
+                0 if sampled else self.token_at(self.computed_tokens) if status is RequestStatus.DECODING else None
+            ),
+            num_preemptions=self.num_preemptions,
+        )
+
     # ---- transitions ------------------------------------------------------------------
     def begin_prefill(self) -> None:
         if self.status is not RequestStatus.WAITING:

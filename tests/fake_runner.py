@@ -34,7 +34,7 @@ class FakeRunner:
         self.steps: list[list[tuple[str, int, int]]] = []     # per step: (request, start, end)
         self.fail_on_step = fail_on_step
         self.prepare_ahead = False          # tests switch it on
-        self.prepared_ahead = self.used_ahead = self.discarded_ahead = 0
+        self.prepared_ahead = self.used_ahead = self.discarded_ahead = self.prepared_mixed = 0
 
     def admit(self, request_id):
         self.tokens[request_id] = []
@@ -56,9 +56,39 @@ class FakeRunner:
         self.prepared_ahead += 1
         return SimpleNamespace(request_ids=tuple(request_ids), reservation=self.cache.prepare_step(items))
 
+    def prepare_step(self, entries, admit=()):
+        """As the real runner's: any other step's cache transaction, opened ahead; the
+        single tokens it is given are placeholders."""
+
+        if not self.prepare_ahead:
+            return None
+        admitted = []
+        try:
+            for request_id in admit:
+                self.admit(request_id)
+                admitted.append(request_id)
+            items = []
+            for entry in entries:
+                start = self.cache.committed_tokens(entry.request_id)
+                items.append(StepItem(entry.request_id, start, start + len(entry.token_ids)))
+            reservation = self.cache.prepare_step(items)
+        except BaseException:
+            for request_id in admitted:
+                self.release(request_id)
+            raise
+        self.prepared_ahead += 1
+        self.prepared_mixed += 1
+        return SimpleNamespace(
+            request_ids=tuple(entry.request_id for entry in entries), reservation=reservation, admitted=tuple(admitted),
+            lengths=tuple(len(entry.token_ids) for entry in entries),
+            known={e.request_id: e.token_ids for e in entries if len(e.token_ids) > 1},
+        )
+
     def discard(self, prepared):
         self.discarded_ahead += 1
         self.cache.abort_step(prepared.reservation)
+        for request_id in getattr(prepared, "admitted", ()):
+            self.release(request_id)
 
     def step(self, entries, prepared=None):
         items = []
@@ -68,7 +98,11 @@ class FakeRunner:
             items.append(StepItem(entry.request_id, start, start + len(entry.token_ids)))
         if prepared is not None:
             assert tuple(entry.request_id for entry in entries) == prepared.request_ids
-            assert all(len(entry.token_ids) == 1 for entry in entries)
+            if hasattr(prepared, "lengths"):
+                assert tuple(len(entry.token_ids) for entry in entries) == prepared.lengths
+                assert all(entry.token_ids == prepared.known[entry.request_id] for entry in entries if len(entry.token_ids) > 1)
+            else:
+                assert all(len(entry.token_ids) == 1 for entry in entries)
             reservation = prepared.reservation
             self.used_ahead += 1
         else:

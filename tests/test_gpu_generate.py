@@ -100,6 +100,8 @@ def test_chunked_prefill_mixed_with_decode_tiny_b(dtype, model_folders):
     for tokens, prompt in zip(got, prompts):
         check_greedy(tokens, prompt, weights, config, dtype)
     assert llm.engine.counters["prefill_tokens"] == sum(len(p) for p in prompts)
+    # steps of portions beside decode tokens were built while the step before ran
+    assert llm.runner.prepared_mixed_steps > 0
     whole = LLM(str(folder), dtype=dtype, kv_block_size=block, num_kv_blocks=40, max_num_seqs=4)
     again = whole.generate(prompts, SamplingParams(max_new_tokens=10))
     if dtype == "float32":

@@ -385,6 +385,73 @@ def test_steps_planned_ahead_change_no_token():
     runner.cache.assert_invariants()
 
 
+def test_steps_with_prompt_portions_are_planned_ahead_too():
+    """Portions of prompts beside decode tokens: the step after is foreseen as well (a
+    request that is admitted in it is admitted ahead), and the steps that run are the
+    very steps that run without planning ahead."""
+
+    params = SamplingParams(max_new_tokens=12)
+    expected = [expected_generation(p, 12, 97) for p in PROMPTS]
+    options = dict(enable_chunked_prefill=True, prefill_chunk_size=7, max_num_batched_tokens=16, max_num_seqs=3)
+    plain, plain_runner = make_engine(**options)
+    assert plain.generate(PROMPTS, params) == expected
+    engine, runner = make_engine(**options)
+    runner.prepare_ahead = True
+    assert engine.generate(PROMPTS, params) == expected
+    assert runner.steps == plain_runner.steps
+    assert runner.prepared_mixed >= 5 and runner.discarded_ahead == 0 and runner.prepared_ahead == runner.used_ahead
+    assert runner.used_ahead >= len(runner.steps) - 3                   # all but the first step and the last ones
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
+    assert runner.cache.capacity().free_slots == 3
+    runner.cache.assert_invariants()
+
+    # a stop token in a request that has just finished its prompt; a request cancelled while it waits, admitted ahead
+    # (a budget of 8 tokens a step: the last request waits until the plan for the eighth step admits it)
+    stop = expected[1][0]
+    engine, runner = make_engine(**{**options, "max_num_batched_tokens": 8})
+    runner.prepare_ahead = True
+    for index, prompt in enumerate(PROMPTS):
+        stops = (stop,) if index == 1 else ()
+        engine.add_request(f"r{index}", prompt, SamplingParams(max_new_tokens=12, stop_token_ids=stops), arrival_ns=index)
+    cancelled = False
+    while engine.has_unfinished():
+        engine.step()
+        if not cancelled and runner.cache.is_live("r3") and engine._sequences["r3"].status.name == "WAITING":
+            engine.cancel("r3")                                            # admitted by the plan ahead, not yet begun
+            cancelled = True
+            assert not runner.cache.is_live("r3")
+        runner.cache.assert_invariants()
+    assert cancelled and runner.discarded_ahead >= 2
+    assert list(engine.pop_result("r0").token_ids) == expected[0]
+    assert list(engine.pop_result("r1").token_ids) == expected[1][:1]
+    assert list(engine.pop_result("r2").token_ids) == expected[2]
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
+    assert runner.cache.capacity().free_slots == 3
+
+    # requests that arrive while others run, in random order, with few pages: the same tokens
+    rng = random.Random(5)
+    for trial in range(20):
+        engine, runner = make_engine(num_kv_blocks=rng.choice([14, 20, 64]), max_num_seqs=rng.choice([2, 3, 4]), **{
+            k: v for k, v in options.items() if k != "max_num_seqs"})
+        runner.prepare_ahead = True
+        order = list(range(len(PROMPTS)))
+        rng.shuffle(order)
+        pending = [(rng.randrange(0, 12), index) for index in order]
+        step = 0
+        while pending or engine.has_unfinished():
+            for due, index in list(pending):
+                if due <= step:
+                    engine.add_request(f"r{index}", PROMPTS[index], params, arrival_ns=step * 10 + index)
+                    pending.remove((due, index))
+            engine.step()
+            runner.cache.assert_invariants()
+            step += 1
+            assert step < 500
+        for index in range(len(PROMPTS)):
+            assert list(engine.pop_result(f"r{index}").token_ids) == expected[index], (trial, index)
+        assert runner.cache.live_requests() == () and runner.used_ahead > 0
+
+
 def test_stop_tokens_and_per_request_parameters():
     engine, _ = make_engine()
     first = expected_generation(PROMPTS[0], 12, 97)
