@@ -10,7 +10,7 @@ import time
 from dataclasses import dataclass
 from typing import Callable, Sequence
 
-from ..cache import OutOfPagesError
+from ..cache import CacheError, OutOfPagesError
 from ..sampling import Sampler
 from .batch import StepEntry
 from .plan import ExecutionPlan
@@ -293,8 +293,8 @@ class Engine:
                 prepared = prepare_step(entries, admit)
             else:
                 prepared = None
-        except OutOfPagesError:
-            return None                # the plan's page count was an estimate; the next call decides
+        except (OutOfPagesError, CacheError):
+            return None                # the plan's page and slot counts were estimates; the next call decides
         if prepared is None:
             return None
         return _StepAhead(self._version, next_plan, prepared)
