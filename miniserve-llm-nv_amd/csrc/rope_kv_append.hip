@@ -138,6 +138,7 @@ int launch(const void* packed, const void* q_weight, const void* k_weight, const
 
 constexpr int kTiledThreads = 256;
 constexpr int kTiledMaxElements = kTiledThreads * 16;   // elements of one head of a tile
+constexpr int kTiledHeads = 4;                          // query and key heads that one workgroup rotates
 
 __device__ __forceinline__ void load8(const ms::bf16* src, float out[8]) {
   const uint4 raw = *reinterpret_cast<const uint4*>(src);
@@ -173,14 +174,17 @@ __global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kerne
     T* __restrict__ value_pool, int num_tokens, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
     float eps) {
   constexpr int kGroup = 16 / static_cast<int>(sizeof(T));   // values of one 16-byte store
-  __shared__ float square_s[kTiledThreads];
+  __shared__ float square_s[kTiledHeads][kTiledThreads];
   __shared__ int32_t slot_s[kTiledThreads];
   __shared__ __align__(16) T tile_s[kTiledMaxElements];
 
+  // blockIdx.y: first the groups of kTiledHeads query and key heads (one workgroup reads
+  // the tile's cos and sin once for all of them), then one block per value head
   const int half = head_dim / 2;
   const int lanes_per_row = half / 8;
   const int tile_tokens = kTiledThreads / lanes_per_row;
-  const int head = blockIdx.y;
+  const int rotated_heads = num_q_heads + num_kv_heads;
+  const int rotated_groups = (rotated_heads + kTiledHeads - 1) / kTiledHeads;
   const int64_t first_token = static_cast<int64_t>(blockIdx.x) * tile_tokens;
   const int live_tokens = static_cast<int>(min(static_cast<int64_t>(tile_tokens), num_tokens - first_token));
   const int item = threadIdx.x / lanes_per_row;
@@ -188,21 +192,15 @@ __global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kerne
   const bool live = item < live_tokens;
   const int64_t token = first_token + (live ? item : 0);
   const int packed_heads = num_q_heads + 2 * num_kv_heads;
-  const T* row = packed + (token * packed_heads + head) * head_dim;
 
-  const bool is_q = head < num_q_heads;
-  const bool is_k = !is_q && head < num_q_heads + num_kv_heads;
-
-  float lo[8], hi[8];
-  if (live) {
-    load8(row + 8 * part, lo);
-    load8(row + half + 8 * part, hi);
-  }
-
-  if (!is_q && !is_k) {
+  if (static_cast<int>(blockIdx.y) >= rotated_groups) {
     // values: through LDS, written along the page's offset axis
-    const int kv_head = head - num_q_heads - num_kv_heads;
+    const int kv_head = static_cast<int>(blockIdx.y) - rotated_groups;
+    const T* row = packed + (token * packed_heads + rotated_heads + kv_head) * head_dim;
     if (live) {
+      float lo[8], hi[8];
+      load8(row + 8 * part, lo);
+      load8(row + half + 8 * part, hi);
       store8(tile_s + item * head_dim + 8 * part, lo);
       store8(tile_s + item * head_dim + half + 8 * part, hi);
     }
@@ -239,58 +237,83 @@ __global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kerne
     return;
   }
 
-  const T* weight = is_q ? q_weight : k_weight;
-  if (weight) {
-    float partial = 0.f;
-    if (live) {
+  // query and key heads first_head .. first_head + heads_here - 1: all their loads go
+  // out together, with the tile's cos and sin
+  const int first_head = static_cast<int>(blockIdx.y) * kTiledHeads;
+  const int heads_here = min(kTiledHeads, rotated_heads - first_head);
+  float lo[kTiledHeads][8], hi[kTiledHeads][8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        partial = fmaf(lo[i], lo[i], partial);
-        partial = fmaf(hi[i], hi[i], partial);
-      }
+  for (int i = 0; i < kTiledHeads; ++i) {
+    if (live && i < heads_here) {
+      const T* row = packed + (token * packed_heads + first_head + i) * head_dim;
+      load8(row + 8 * part, lo[i]);
+      load8(row + half + 8 * part, hi[i]);
     }
-    square_s[threadIdx.x] = partial;
+  }
+  float cs[8], sn[8];
+  if (live && cos_table != nullptr) {
+    load8(cos_table + token * half + 8 * part, cs);
+    load8(sin_table + token * half + 8 * part, sn);
+  }
+  int64_t slot = 0;
+  if (live && first_head + heads_here > num_q_heads) slot = slot_mapping[token];
+
+  if (q_weight != nullptr || k_weight != nullptr) {
+#pragma unroll
+    for (int i = 0; i < kTiledHeads; ++i) {
+      float partial = 0.f;
+      if (live && i < heads_here) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          partial = fmaf(lo[i][e], lo[i][e], partial);
+          partial = fmaf(hi[i][e], hi[i][e], partial);
+        }
+      }
+      square_s[i][threadIdx.x] = partial;
+    }
     __syncthreads();
-    if (live) {
+  }
+  if (!live) return;
+
+#pragma unroll
+  for (int i = 0; i < kTiledHeads; ++i) {
+    if (i >= heads_here) break;
+    const int head = first_head + i;
+    const bool is_q = head < num_q_heads;
+    const T* weight = is_q ? q_weight : k_weight;
+    if (weight) {
       float total = 0.f;
-      for (int p = 0; p < lanes_per_row; ++p) total += square_s[item * lanes_per_row + p];
+      for (int p = 0; p < lanes_per_row; ++p) total += square_s[i][item * lanes_per_row + p];
       const float inv = 1.0f / sqrtf(total / static_cast<float>(head_dim) + eps);
       float w_lo[8], w_hi[8];
       load8(weight + 8 * part, w_lo);
       load8(weight + half + 8 * part, w_hi);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        lo[i] = ms::round_to<T>(w_lo[i] * ms::round_to<T>(lo[i] * inv));
-        hi[i] = ms::round_to<T>(w_hi[i] * ms::round_to<T>(hi[i] * inv));
+      for (int e = 0; e < 8; ++e) {
+        lo[i][e] = ms::round_to<T>(w_lo[e] * ms::round_to<T>(lo[i][e] * inv));
+        hi[i][e] = ms::round_to<T>(w_hi[e] * ms::round_to<T>(hi[i][e] * inv));
       }
     }
-  }
-  if (!live) return;
-
-  if (cos_table != nullptr) {
-    float cs[8], sn[8];
-    load8(cos_table + token * half + 8 * part, cs);
-    load8(sin_table + token * half + 8 * part, sn);
+    if (cos_table != nullptr) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float a = lo[i], b = hi[i];
-      lo[i] = a * cs[i] - b * sn[i];
-      hi[i] = b * cs[i] + a * sn[i];
+      for (int e = 0; e < 8; ++e) {
+        const float a = lo[i][e], b = hi[i][e];
+        lo[i][e] = a * cs[e] - b * sn[e];
+        hi[i][e] = b * cs[e] + a * sn[e];
+      }
     }
+    T* dst;
+    if (is_q) {
+      dst = q_out + (token * num_q_heads + head) * head_dim;
+    } else {
+      const int kv_head = head - num_q_heads;
+      const int64_t page = slot / block_size;
+      const int64_t offset = slot - page * block_size;
+      dst = key_pool + ((page * num_kv_heads + kv_head) * block_size + offset) * head_dim;
+    }
+    store8(dst + 8 * part, lo[i]);
+    store8(dst + half + 8 * part, hi[i]);
   }
-
-  T* dst;
-  if (is_q) {
-    dst = q_out + (token * num_q_heads + head) * head_dim;
-  } else {
-    const int kv_head = head - num_q_heads;
-    const int64_t slot = slot_mapping[token];
-    const int64_t page = slot / block_size;
-    const int64_t offset = slot - page * block_size;
-    dst = key_pool + ((page * num_kv_heads + kv_head) * block_size + offset) * head_dim;
-  }
-  store8(dst + 8 * part, lo);
-  store8(dst + half + 8 * part, hi);
 }
 
 template <typename T>
@@ -299,7 +322,8 @@ void launch_tiled(const void* packed, const void* q_weight, const void* k_weight
                   int num_tokens, int num_q_heads, int num_kv_heads, int head_dim, int block_size, float eps,
                   hipStream_t stream) {
   const int tile_tokens = kTiledThreads / (head_dim / 16);
-  const dim3 grid((num_tokens + tile_tokens - 1) / tile_tokens, num_q_heads + 2 * num_kv_heads);
+  const int rotated_groups = (num_q_heads + num_kv_heads + kTiledHeads - 1) / kTiledHeads;
+  const dim3 grid((num_tokens + tile_tokens - 1) / tile_tokens, rotated_groups + num_kv_heads);
   hipLaunchKernelGGL((qk_norm_rope_append_tiled_kernel<T>), grid, dim3(kTiledThreads), 0, stream,
       static_cast<const T*>(packed), static_cast<const T*>(q_weight), static_cast<const T*>(k_weight),
       static_cast<const float*>(cos_table), static_cast<const float*>(sin_table),

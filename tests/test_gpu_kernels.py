@@ -172,7 +172,7 @@ def test_qk_norm_rope_append(ops, dtype, heads, kv_heads, dim, block):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,dim,block,start", [(4, 2, 128, 16, 5), (2, 1, 80, 8, 0), (3, 3, 16, 12, 7), (2, 2, 64, 4, 3), (1, 1, 512, 16, 9)])
+@pytest.mark.parametrize("heads,kv_heads,dim,block,start", [(4, 2, 128, 16, 5), (2, 1, 80, 8, 0), (3, 3, 16, 12, 7), (2, 2, 64, 4, 3), (1, 1, 512, 16, 9), (16, 8, 128, 16, 2), (5, 2, 32, 16, 0)])
 def test_append_of_a_run_of_tokens_beside_single_ones(ops, dtype, heads, kv_heads, dim, block, start):
     """A portion of a prompt that starts in the middle of a page and runs over several
     pages (handed out in reverse), behind three single tokens in pages of their own:
