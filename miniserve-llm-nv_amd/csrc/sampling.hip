@@ -17,12 +17,20 @@
 //   draw                  : first index whose running sum of exp(x - max) over
 //                           the kept tokens exceeds uniform * total
 // A row with a NaN or infinite logit yields -1.
+//
+// The thresholds of top-k and top-p are found digit by digit, four bits a pass over
+// the candidates.  With top-k or top-p only tokens near the row's maximum can stay:
+// one pass over the row finds a distance below the maximum within which all of them
+// lie, they are gathered into LDS in token order (at most 4096), and every later
+// pass runs over that short list; a row whose candidates do not fit, and a row with
+// neither top-k nor top-p, is handled over its whole length.
 #include "common.hpp"
 
 namespace {
 
 constexpr int kThreads = 1024;
 constexpr int kWaves = kThreads / ms::kWave;
+constexpr int kDigits = 15;     // candidates of one pass of a threshold search: four bits
 
 // Monotone map from float to unsigned: a < b  <=>  ordered(a) < ordered(b).
 __device__ __forceinline__ uint32_t ordered(float value) {
@@ -51,6 +59,217 @@ struct Keep {
   }
 };
 
+// What the choice is made from: the whole row, or the few tokens of it that can
+// still matter, gathered in LDS in token order.  value(i) is logit / temperature.
+struct RowView {
+  const float* x;
+  float temp;
+  int size;
+  __device__ __forceinline__ float value(int i) const { return x[i] / temp; }
+  __device__ __forceinline__ int index(int i) const { return i; }
+};
+
+struct ListView {
+  const float* values;
+  const int* indices;
+  int size;
+  __device__ __forceinline__ float value(int i) const { return values[i]; }
+  __device__ __forceinline__ int index(int i) const { return indices[i]; }
+};
+
+constexpr int kListCap = 4096;      // tokens that the short list holds at most
+// Distances below the row's maximum (in units of logit / temperature) at which the
+// row is cut to make the short list: the first of them that keeps enough is taken.
+constexpr int kLadder = 8;
+constexpr float kLadderDepth[kLadder] = {1.f, 2.f, 4.f, 6.f, 9.f, 13.f, 18.f, 26.f};
+
+struct Scratch {
+  float* f_scratch;       // [kWaves]
+  int* i_scratch;         // [kWaves]
+  float* seg_sum;         // [kThreads]
+  int* seg_count;         // [kThreads]
+  int* shared_index;
+  float* shared_total;
+  int (*digit_count)[kDigits];     // [kWaves][kDigits]
+  float (*digit_mass)[kDigits];    // [kWaves][kDigits]
+};
+
+// temperature -> top-k -> top-p -> draw over `view`; `limit_index`: an index beyond
+// every token's; `whole_mass`: the mass of all tokens where the view holds only some
+// of them and top-k is off (top_p is a share of that), else negative.  All threads of
+// the workgroup call it and get the same result.
+template <typename View>
+__device__ int choose(const View& view, int limit_index, float scaled_max, int k, float p, float uniform,
+                      float whole_mass, const Scratch& sc) {
+  const int tid = threadIdx.x;
+  const int n = view.size;
+  // Contiguous segment of this thread, for everything that needs token order.
+  const int seg = (n + kThreads - 1) / kThreads;
+  const int seg_begin = min(tid * seg, n);
+  const int seg_end = min(seg_begin + seg, n);
+
+  Keep keep;
+  keep.k_threshold = 0u;
+  keep.tie_limit = limit_index;
+  keep.p_threshold = 0u;
+
+  // ---- top-k ----------------------------------------------------------------
+  if (k > 0 && k < n) {
+    // The k-th largest ordered value, four bits a pass: a thread counts, for each of the
+    // 15 candidates threshold | c << shift, the values at or above it; the counts fall as c
+    // rises, and the largest c that still has k values is the next digit.
+    uint32_t threshold = 0u;
+    for (int shift = 28; shift >= 0; shift -= 4) {
+      int count[kDigits];
+#pragma unroll
+      for (int c = 0; c < kDigits; ++c) count[c] = 0;
+      for (int i = tid; i < n; i += kThreads) {
+        const uint32_t o = ordered(view.value(i));
+#pragma unroll
+        for (int c = 0; c < kDigits; ++c) count[c] += o >= (threshold | (static_cast<uint32_t>(c + 1) << shift));
+      }
+      __syncthreads();                    // the tables' last readers are done
+#pragma unroll
+      for (int c = 0; c < kDigits; ++c) {
+        const int v = ms::wave_sum_int(count[c]);
+        if ((tid & (ms::kWave - 1)) == 0) sc.digit_count[tid / ms::kWave][c] = v;
+      }
+      __syncthreads();
+      if (tid < kDigits) {
+        int total = 0;
+        for (int w = 0; w < kWaves; ++w) total += sc.digit_count[w][tid];
+        sc.digit_count[0][tid] = total;      // (only this thread reads column tid)
+      }
+      __syncthreads();
+      int digit = 0;
+      for (int c = 0; c < kDigits; ++c)
+        if (sc.digit_count[0][c] >= k) digit = c + 1;
+      threshold |= static_cast<uint32_t>(digit) << shift;
+    }
+    int greater = 0, equal = 0;
+    for (int i = seg_begin; i < seg_end; ++i) {
+      const uint32_t o = ordered(view.value(i));
+      greater += o > threshold;
+      equal += o == threshold;
+    }
+    const int total_greater = block_sum_int(greater, sc.i_scratch);
+    const int wanted = k - total_greater;  // >= 1 equal values to keep, lowest indices first
+    sc.seg_count[tid] = equal;
+    __syncthreads();
+    if (tid == 0) {
+      int running = 0;
+      for (int t = 0; t < kThreads; ++t) {
+        const int c = sc.seg_count[t];
+        sc.seg_count[t] = running;  // exclusive prefix
+        running += c;
+      }
+      *sc.shared_index = limit_index;
+    }
+    __syncthreads();
+    int seen = sc.seg_count[tid];
+    for (int i = seg_begin; i < seg_end; ++i) {
+      if (ordered(view.value(i)) == threshold) {
+        ++seen;
+        if (seen == wanted) *sc.shared_index = view.index(i);  // exactly one thread reaches `wanted`
+      }
+    }
+    __syncthreads();
+    keep.k_threshold = threshold;
+    keep.tie_limit = *sc.shared_index;
+    __syncthreads();
+  }
+
+  // ---- top-p ----------------------------------------------------------------
+  if (p < 1.f) {
+    float mass = 0.f;
+    for (int i = tid; i < n; i += kThreads) {
+      const float v = view.value(i);
+      if (keep(ordered(v), view.index(i))) mass += expf(v - scaled_max);
+    }
+    const float kept_mass = ms::block_sum(mass, sc.f_scratch);
+    const float limit = p * (whole_mass >= 0.f ? whole_mass : kept_mass);
+    // Largest t with mass{ordered >= t} > limit; tokens at or above it stay.  Four bits a
+    // pass, as for top-k, with the mass at or above each candidate in place of the count.
+    uint32_t threshold = 0u;
+    for (int shift = 28; shift >= 0; shift -= 4) {
+      float part[kDigits];
+#pragma unroll
+      for (int c = 0; c < kDigits; ++c) part[c] = 0.f;
+      for (int i = tid; i < n; i += kThreads) {
+        const float v = view.value(i);
+        const uint32_t o = ordered(v);
+        if (o >= threshold && keep(o, view.index(i))) {
+          const float weight = expf(v - scaled_max);
+#pragma unroll
+          for (int c = 0; c < kDigits; ++c)
+            part[c] += o >= (threshold | (static_cast<uint32_t>(c + 1) << shift)) ? weight : 0.f;
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int c = 0; c < kDigits; ++c) {
+        const float v = ms::wave_sum(part[c]);
+        if ((tid & (ms::kWave - 1)) == 0) sc.digit_mass[tid / ms::kWave][c] = v;
+      }
+      __syncthreads();
+      if (tid < kDigits) {
+        float total = 0.f;
+        for (int w = 0; w < kWaves; ++w) total += sc.digit_mass[w][tid];
+        sc.digit_mass[0][tid] = total;
+      }
+      __syncthreads();
+      int digit = 0;
+      for (int c = 0; c < kDigits; ++c)
+        if (sc.digit_mass[0][c] > limit) digit = c + 1;
+      threshold |= static_cast<uint32_t>(digit) << shift;
+    }
+    keep.p_threshold = threshold;
+  }
+
+  // ---- draw -----------------------------------------------------------------
+  float mine = 0.f;
+  int last_kept = -1;
+  for (int i = seg_begin; i < seg_end; ++i) {
+    const float v = view.value(i);
+    if (keep(ordered(v), view.index(i))) {
+      mine += expf(v - scaled_max);
+      last_kept = view.index(i);
+    }
+  }
+  __syncthreads();
+  sc.seg_sum[tid] = mine;
+  sc.seg_count[tid] = last_kept;
+  __syncthreads();
+  if (tid == 0) {
+    float running = 0.f;
+    int last = -1;
+    for (int t = 0; t < kThreads; ++t) {
+      const float s = sc.seg_sum[t];
+      sc.seg_sum[t] = running;  // exclusive prefix, in token order
+      running += s;
+      if (sc.seg_count[t] > last) last = sc.seg_count[t];
+    }
+    *sc.shared_total = running;
+    *sc.shared_index = last;  // fallback: the last kept token
+  }
+  __syncthreads();
+  const float target = uniform * *sc.shared_total;
+  __syncthreads();
+  float running = sc.seg_sum[tid];
+  for (int i = seg_begin; i < seg_end; ++i) {
+    const float v = view.value(i);
+    if (keep(ordered(v), view.index(i))) {
+      running += expf(v - scaled_max);
+      if (running > target) {
+        atomicMin(sc.shared_index, view.index(i));
+        break;
+      }
+    }
+  }
+  __syncthreads();
+  return *sc.shared_index;
+}
+
 __global__ __launch_bounds__(kThreads) void sample_rows_kernel(const float* __restrict__ logits,
                                                                const float* __restrict__ temperature,
                                                                const int32_t* __restrict__ top_k,
@@ -63,16 +282,23 @@ __global__ __launch_bounds__(kThreads) void sample_rows_kernel(const float* __re
   __shared__ int seg_count[kThreads];
   __shared__ int shared_index;
   __shared__ float shared_total;
+  __shared__ int digit_count[kWaves][kDigits];
+  __shared__ float digit_mass[kWaves][kDigits];
+  __shared__ int ladder_count[kWaves][kLadder];
+  __shared__ float ladder_mass[kWaves][kLadder + 1];
+  __shared__ int list_base[kWaves + 1];
+  __shared__ int list_rung;
+  __shared__ float list_whole_mass;
+  __shared__ float list_values[kListCap];
+  __shared__ int list_indices[kListCap];
 
   const int row = blockIdx.x;
   const int tid = threadIdx.x;
+  const int lane = tid & (ms::kWave - 1);
+  const int wave = tid / ms::kWave;
   const float* x = logits + static_cast<int64_t>(row) * vocab;
   const float temp = temperature ? temperature[row] : 0.f;
-
-  // Contiguous segment of this thread, for everything that needs token order.
-  const int seg = (vocab + kThreads - 1) / kThreads;
-  const int seg_begin = min(tid * seg, vocab);
-  const int seg_end = min(seg_begin + seg, vocab);
+  Scratch sc{f_scratch, i_scratch, seg_sum, seg_count, &shared_index, &shared_total, digit_count, digit_mass};
 
   // ---- finiteness, maximum and its lowest index ---------------------------
   float best = -INFINITY;
@@ -101,120 +327,111 @@ __global__ __launch_bounds__(kThreads) void sample_rows_kernel(const float* __re
     return;
   }
 
-  Keep keep;
-  keep.k_threshold = 0u;
-  keep.tie_limit = vocab;
-  keep.p_threshold = 0u;
   const float scaled_max = row_max / temp;
-
-  // ---- top-k ----------------------------------------------------------------
   const int k = top_k ? top_k[row] : 0;
-  if (k > 0 && k < vocab) {
-    uint32_t threshold = 0u;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t candidate = threshold | (1u << bit);
-      int count = 0;
-      for (int i = tid; i < vocab; i += kThreads) count += ordered(x[i] / temp) >= candidate;
-      if (block_sum_int(count, i_scratch) >= k) threshold = candidate;
+  const float p = top_p ? top_p[row] : 1.f;
+  const bool cut_k = k > 0 && k < vocab;
+  const bool cut_p = p < 1.f;
+
+  // ---- the short list ---------------------------------------------------------
+  // With top-k or top-p only tokens near the maximum can stay.  One pass counts, for
+  // each rung of a ladder of distances below the maximum, the tokens at or above it
+  // (and their mass): the first rung that holds k tokens (top-k), or more than top_p
+  // of the whole mass (top-p alone), holds every token that can stay.  If they fit,
+  // they are gathered in token order and the choice is made among them; else, and
+  // without top-k and top-p, it is made over the whole row.  A wave reads a contiguous
+  // part of the row, so that its share of the list is contiguous too.
+  if (cut_k || cut_p) {
+    const int chunk = ((vocab + kWaves - 1) / kWaves + ms::kWave - 1) / ms::kWave * ms::kWave;
+    const int chunk_begin = min(wave * chunk, vocab);
+    const int chunk_end = min(chunk_begin + chunk, vocab);
+    int count[kLadder];
+    float mass[kLadder + 1];
+#pragma unroll
+    for (int c = 0; c < kLadder; ++c) count[c] = 0, mass[c] = 0.f;
+    mass[kLadder] = 0.f;
+    for (int i = chunk_begin + lane; i < chunk_end; i += ms::kWave) {
+      const float v = x[i] / temp;
+      const float depth = scaled_max - v;
+      const float weight = cut_k ? 0.f : expf(v - scaled_max);
+      mass[kLadder] += weight;
+#pragma unroll
+      for (int c = 0; c < kLadder; ++c) {
+        const bool in = depth <= kLadderDepth[c];
+        count[c] += in;
+        mass[c] += in ? weight : 0.f;
+      }
     }
-    int greater = 0, equal = 0;
-    for (int i = seg_begin; i < seg_end; ++i) {
-      const uint32_t o = ordered(x[i] / temp);
-      greater += o > threshold;
-      equal += o == threshold;
+#pragma unroll
+    for (int c = 0; c < kLadder; ++c) {
+      const int total = ms::wave_sum_int(count[c]);
+      const float sum = ms::wave_sum(mass[c]);
+      if (lane == 0) ladder_count[wave][c] = total, ladder_mass[wave][c] = sum;
     }
-    const int total_greater = block_sum_int(greater, i_scratch);
-    const int wanted = k - total_greater;  // >= 1 equal values to keep, lowest indices first
-    seg_count[tid] = equal;
+    {
+      const float sum = ms::wave_sum(mass[kLadder]);
+      if (lane == 0) ladder_mass[wave][kLadder] = sum;
+    }
     __syncthreads();
     if (tid == 0) {
-      int running = 0;
-      for (int t = 0; t < kThreads; ++t) {
-        const int c = seg_count[t];
-        seg_count[t] = running;  // exclusive prefix
-        running += c;
+      float whole = 0.f;
+      for (int w = 0; w < kWaves; ++w) whole += ladder_mass[w][kLadder];
+      int rung = -1;
+      for (int c = 0; c < kLadder && rung < 0; ++c) {
+        int total = 0;
+        float sum = 0.f;
+        for (int w = 0; w < kWaves; ++w) total += ladder_count[w][c], sum += ladder_mass[w][c];
+        // (a little more than top_p of the mass: the sums here and those of the choice differ in rounding)
+        const bool enough = cut_k ? total >= k : sum > (p + 1e-4f) * whole;
+        if (enough && total <= kListCap) rung = c;
+        if (total > kListCap) break;
       }
-      shared_index = vocab;
+      list_rung = rung;
+      list_whole_mass = whole;
+      if (rung >= 0) {
+        int running = 0;
+        for (int w = 0; w < kWaves; ++w) {
+          list_base[w] = running;
+          running += ladder_count[w][rung];
+        }
+        list_base[kWaves] = running;
+      }
     }
     __syncthreads();
-    int seen = seg_count[tid];
-    for (int i = seg_begin; i < seg_end; ++i) {
-      if (ordered(x[i] / temp) == threshold) {
-        ++seen;
-        if (seen == wanted) shared_index = i;  // exactly one thread reaches `wanted`
+    const int rung = list_rung;
+    if (rung >= 0) {
+      float deepest = 0.f;
+#pragma unroll
+      for (int c = 0; c < kLadder; ++c)
+        if (c == rung) deepest = kLadderDepth[c];
+      int written = list_base[wave];
+      for (int base = chunk_begin; base < chunk_end; base += ms::kWave) {
+        const int i = base + lane;
+        float v = 0.f;
+        bool in = false;
+        if (i < chunk_end) {
+          v = x[i] / temp;
+          in = scaled_max - v <= deepest;
+        }
+        const unsigned long long mask = __ballot(in);
+        if (in) {
+          const int place = written + __popcll(mask & ((1ull << lane) - 1ull));
+          list_values[place] = v;
+          list_indices[place] = i;
+        }
+        written += __popcll(mask);
       }
-    }
-    __syncthreads();
-    keep.k_threshold = threshold;
-    keep.tie_limit = shared_index;
-    __syncthreads();
-  }
-
-  // ---- top-p ----------------------------------------------------------------
-  const float p = top_p ? top_p[row] : 1.f;
-  if (p < 1.f) {
-    float mass = 0.f;
-    for (int i = seg_begin; i < seg_end; ++i) {
-      const float v = x[i] / temp;
-      if (keep(ordered(v), i)) mass += expf(v - scaled_max);
-    }
-    const float limit = p * ms::block_sum(mass, f_scratch);
-    // Largest t with mass{ordered >= t} > limit; tokens at or above it stay.
-    uint32_t threshold = 0u;
-    for (int bit = 31; bit >= 0; --bit) {
-      const uint32_t candidate = threshold | (1u << bit);
-      float part = 0.f;
-      for (int i = seg_begin; i < seg_end; ++i) {
-        const float v = x[i] / temp;
-        const uint32_t o = ordered(v);
-        if (o >= candidate && keep(o, i)) part += expf(v - scaled_max);
-      }
-      if (ms::block_sum(part, f_scratch) > limit) threshold = candidate;
-    }
-    keep.p_threshold = threshold;
-  }
-
-  // ---- draw -----------------------------------------------------------------
-  float mine = 0.f;
-  int last_kept = -1;
-  for (int i = seg_begin; i < seg_end; ++i) {
-    const float v = x[i] / temp;
-    if (keep(ordered(v), i)) {
-      mine += expf(v - scaled_max);
-      last_kept = i;
+      __syncthreads();
+      const ListView list{list_values, list_indices, list_base[kWaves]};
+      const int chosen = choose(list, vocab, scaled_max, cut_k ? k : 0, p, uniform[row],
+                                cut_k ? -1.f : list_whole_mass, sc);
+      if (tid == 0) out[row] = chosen;
+      return;
     }
   }
-  seg_sum[tid] = mine;
-  seg_count[tid] = last_kept;
-  __syncthreads();
-  if (tid == 0) {
-    float running = 0.f;
-    int last = -1;
-    for (int t = 0; t < kThreads; ++t) {
-      const float s = seg_sum[t];
-      seg_sum[t] = running;  // exclusive prefix, in token order
-      running += s;
-      if (seg_count[t] > last) last = seg_count[t];
-    }
-    shared_total = running;
-    shared_index = last;  // fallback: the last kept token
-  }
-  __syncthreads();
-  const float target = uniform[row] * shared_total;
-  __syncthreads();
-  float running = seg_sum[tid];
-  for (int i = seg_begin; i < seg_end; ++i) {
-    const float v = x[i] / temp;
-    if (keep(ordered(v), i)) {
-      running += expf(v - scaled_max);
-      if (running > target) {
-        atomicMin(&shared_index, i);
-        break;
-      }
-    }
-  }
-  __syncthreads();
-  if (tid == 0) out[row] = shared_index;
+  const RowView whole{x, temp, vocab};
+  const int chosen = choose(whole, vocab, scaled_max, cut_k ? k : 0, p, uniform[row], -1.f, sc);
+  if (tid == 0) out[row] = chosen;
 }
 
 // Greedy choice for large vocabularies in two stages, so that a row is read by many

@@ -728,6 +728,52 @@ def test_sampling_matches_the_plain_implementation(ops, vocab):
         assert out[row] == expected, f"row {row}: T={temperature[row]} k={top_k[row]} p={top_p[row]} u={uniform[row]}"
 
 
+def test_sampling_from_the_short_list_and_from_the_whole_row(ops):
+    """With top-k or top-p the kernel gathers the tokens near the maximum into a short
+    list when they fit (4096) and chooses among them, else over the whole row; both give
+    the plain implementation's token.  Rows with a few outstanding tokens (as a model's
+    logits have) and flat rows; top-k beyond the list's size; top-p close to 1."""
+
+    vocab, rows = 50021, 36
+    generator = torch.Generator().manual_seed(7)
+    logits = torch.randn(rows, vocab, generator=generator) * 2
+    for row in range(0, rows, 2):                       # every other row: 40 tokens stand out
+        chosen = torch.randperm(vocab, generator=generator)[:40]
+        logits[row, chosen] += 8 + 6 * torch.rand(40, generator=generator)
+    temperature = torch.tensor([0.6, 0.6, 1.0, 1.0, 1.3, 1.3] * 6)
+    top_k = torch.tensor([0, 0, 20, 20, 5000, 5000, 0, 0, 1, 1, 4096, 4097] * 3, dtype=torch.int32)
+    top_p = torch.tensor([0.5, 0.5, 0.95, 0.95, 0.9, 0.9, 0.9999, 0.9999, 0.3, 0.3, 1.0, 0.8] * 3)
+    uniform = torch.rand(rows, generator=generator)
+    out = ops.sample_rows(logits.to(DEVICE), temperature=temperature.to(DEVICE), top_k=top_k.to(DEVICE),
+                          top_p=top_p.to(DEVICE), uniform=uniform.to(DEVICE)).cpu().tolist()
+    for row in range(rows):
+        expected = plain_sampling.sample_row(
+            logits[row], float(temperature[row]), int(top_k[row]), float(top_p[row]), float(uniform[row])
+        )
+        assert out[row] == expected, f"row {row}: T={temperature[row]} k={top_k[row]} p={top_p[row]} u={uniform[row]}"
+
+
+def test_equal_values_at_the_edge_of_top_k_keep_the_lowest_indices(ops):
+    """A hundred tokens share the k-th largest value, spread over a long row: exactly k
+    tokens stay, the equal ones with the lowest indices, and every one of them can be drawn."""
+
+    vocab, k, rows = 30011, 30, 200
+    generator = torch.Generator().manual_seed(11)
+    row = torch.randn(vocab, generator=generator) - 6
+    above = torch.randperm(vocab, generator=generator)[:110]
+    row[above[:10]] = 7.0 + torch.arange(10) * 0.25            # ten tokens above the tie
+    tied = torch.sort(above[10:]).values
+    row[tied] = 6.5                                             # a hundred equal ones; twenty of them stay
+    logits = row.repeat(rows, 1).to(DEVICE)
+    out = ops.sample_rows(
+        logits, temperature=torch.ones(rows, device=DEVICE), top_k=torch.full((rows,), k, dtype=torch.int32, device=DEVICE),
+        top_p=torch.ones(rows, device=DEVICE), uniform=((torch.arange(rows) + 0.5) / rows).to(DEVICE),
+    ).cpu().tolist()
+    allowed = set(above[:10].tolist()) | set(tied[:20].tolist())
+    assert set(out) <= allowed
+    assert set(tied[:20].tolist()) <= set(out)                  # 200 evenly spaced draws reach each of the 30
+
+
 def test_sampling_vectors_of_the_reference(ops):
     # [5,4,3,2], T=1, k=2, p=0.6 -> always 0 (tests/unit/test_sampling.py:44-49)
     logits = torch.tensor([[5.0, 4.0, 3.0, 2.0]] * 20, device=DEVICE)
