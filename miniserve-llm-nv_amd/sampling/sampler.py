@@ -13,6 +13,7 @@ import os
 from dataclasses import dataclass
 from typing import Sequence
 
+import numpy as np
 import torch
 
 from ..engine.request import SamplingParams
@@ -89,13 +90,17 @@ class Sampler:
         if all(state is None for state in states):
             tokens = ops.sample_rows(logits)
         else:
-            device = logits.device
+            # the four numbers of every row in one pinned buffer and one copy that nothing waits for
+            # (a copy from pageable memory would wait for the step that is still running)
+            host = torch.empty((4, len(requests)), dtype=torch.float32, pin_memory=logits.is_cuda)
+            numbers = host.numpy()
+            numbers[0] = [p.temperature for _, p in requests]
+            numbers[1] = [p.top_p for _, p in requests]
+            numbers[2] = uniforms
+            numbers[3].view(np.int32)[:] = [p.top_k for _, p in requests]
+            sent = host.to(logits.device, non_blocking=True)
             tokens = ops.sample_rows(
-                logits,
-                temperature=torch.tensor([p.temperature for _, p in requests], dtype=torch.float32, device=device),
-                top_k=torch.tensor([p.top_k for _, p in requests], dtype=torch.int32, device=device),
-                top_p=torch.tensor([p.top_p for _, p in requests], dtype=torch.float32, device=device),
-                uniform=torch.tensor(uniforms, dtype=torch.float32, device=device),
+                logits, temperature=sent[0], top_p=sent[1], uniform=sent[2], top_k=sent[3].view(torch.int32)
             )
         return tokens, tuple(requests), states
 
