@@ -96,11 +96,13 @@ struct Scratch {
 
 // temperature -> top-k -> top-p -> draw over `view`; `limit_index`: an index beyond
 // every token's; `whole_mass`: the mass of all tokens where the view holds only some
-// of them and top-k is off (top_p is a share of that), else negative.  All threads of
-// the workgroup call it and get the same result.
+// of them and top-k is off (top_p is a share of that), else negative; `mass_before`:
+// with top-k and top-p off and a view that is one part of the row, the mass of the
+// tokens before it (the draw is then at uniform * whole_mass).  All threads of the
+// workgroup call it and get the same result.
 template <typename View>
 __device__ int choose(const View& view, int limit_index, float scaled_max, int k, float p, float uniform,
-                      float whole_mass, const Scratch& sc) {
+                      float whole_mass, float mass_before, const Scratch& sc) {
   const int tid = threadIdx.x;
   const int n = view.size;
   // Contiguous segment of this thread, for everything that needs token order.
@@ -253,7 +255,8 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
     *sc.shared_index = last;  // fallback: the last kept token
   }
   __syncthreads();
-  const float target = uniform * *sc.shared_total;
+  const float target = (k == 0 && !(p < 1.f) && whole_mass >= 0.f) ? uniform * whole_mass - mass_before
+                                                                     : uniform * *sc.shared_total;
   __syncthreads();
   float running = sc.seg_sum[tid];
   for (int i = seg_begin; i < seg_end; ++i) {
@@ -424,13 +427,13 @@ __global__ __launch_bounds__(kThreads) void sample_rows_kernel(const float* __re
       __syncthreads();
       const ListView list{list_values, list_indices, list_base[kWaves]};
       const int chosen = choose(list, vocab, scaled_max, cut_k ? k : 0, p, uniform[row],
-                                cut_k ? -1.f : list_whole_mass, sc);
+                                cut_k ? -1.f : list_whole_mass, 0.f, sc);
       if (tid == 0) out[row] = chosen;
       return;
     }
   }
   const RowView whole{x, temp, vocab};
-  const int chosen = choose(whole, vocab, scaled_max, cut_k ? k : 0, p, uniform[row], -1.f, sc);
+  const int chosen = choose(whole, vocab, scaled_max, cut_k ? k : 0, p, uniform[row], -1.f, 0.f, sc);
   if (tid == 0) out[row] = chosen;
 }
 
@@ -508,6 +511,369 @@ extern "C" int ms_argmax_rows(const void* logits, void* chunk_max, void* chunk_i
   return 0;
 }
 
+// ---- the same choice for a large vocabulary: a row is read by many workgroups ----------
+//
+// One workgroup a row reads 600 KB of logits several times at the speed of one
+// compute unit.  Here the passes over the row are cut into kRowChunks chunks, a
+// workgroup each: (1) finiteness, maximum and its lowest index per chunk; (2) the
+// ladder's counts and masses per chunk; (3) the short list, every chunk writing its
+// share at its place in token order; (4) one workgroup a row makes the choice: among
+// the list, or, without top-k and top-p, inside the chunk that the running mass
+// singles out, or - the candidates do not fit a list - over the whole row as above.
+// Tables between the stages (per row): chunk_max, chunk_arg [chunks]; ladder_count
+// [chunks][kLadder]; ladder_mass [chunks][kLadder + 1]; list_values, list_indices [kListCap].
+constexpr int kRowChunks = 32;
+constexpr int kChunkThreads = 256;
+constexpr int kChunkWaves = kChunkThreads / ms::kWave;
+
+struct RowTables {
+  float* chunk_max;
+  int* chunk_arg;
+  int* ladder_count;
+  float* ladder_mass;
+  float* list_values;
+  int* list_indices;
+};
+
+__host__ __device__ inline size_t row_table_floats() {
+  return static_cast<size_t>(kRowChunks) * (2 + kLadder + kLadder + 1) + 2 * static_cast<size_t>(kListCap);
+}
+
+__device__ __forceinline__ RowTables row_tables(float* workspace, int row) {
+  float* base = workspace + static_cast<size_t>(row) * row_table_floats();
+  RowTables t;
+  t.chunk_max = base;
+  t.chunk_arg = reinterpret_cast<int*>(base + kRowChunks);
+  t.ladder_count = reinterpret_cast<int*>(base + 2 * kRowChunks);
+  t.ladder_mass = base + 2 * kRowChunks + kRowChunks * kLadder;
+  t.list_values = base + 2 * kRowChunks + kRowChunks * (2 * kLadder + 1);
+  t.list_indices = reinterpret_cast<int*>(t.list_values + kListCap);
+  return t;
+}
+
+__device__ __forceinline__ int chunk_length(int vocab) {
+  return ((vocab + kRowChunks - 1) / kRowChunks + ms::kWave - 1) / ms::kWave * ms::kWave;
+}
+
+// Which rung of the ladder makes the short list (-1: none), from the tables of stage 2;
+// every caller gets the same answer.  `whole`: the mass of the whole row.
+__device__ int choose_rung(const RowTables& t, bool cut_k, int k, float p, float* whole_out, int* total_out) {
+  float whole = 0.f;
+  for (int c = 0; c < kRowChunks; ++c) whole += t.ladder_mass[c * (kLadder + 1) + kLadder];
+  *whole_out = whole;
+  for (int r = 0; r < kLadder; ++r) {
+    int total = 0;
+    float sum = 0.f;
+    for (int c = 0; c < kRowChunks; ++c) {
+      total += t.ladder_count[c * kLadder + r];
+      sum += t.ladder_mass[c * (kLadder + 1) + r];
+    }
+    if (total > kListCap) return -1;
+    // (a little more than top_p of the mass: the sums here and those of the choice differ in rounding)
+    const bool enough = cut_k ? total >= k : sum > (p + 1e-4f) * whole;
+    if (enough) {
+      *total_out = total;
+      return r;
+    }
+  }
+  return -1;
+}
+
+__global__ __launch_bounds__(kChunkThreads) void sample_scan_kernel(const float* __restrict__ logits,
+                                                                    float* __restrict__ workspace, int vocab) {
+  __shared__ float f_scratch[kChunkWaves];
+  __shared__ int i_scratch[kChunkWaves];
+  __shared__ int shared_index;
+  const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+  const RowTables t = row_tables(workspace, row);
+  const int length = chunk_length(vocab);
+  const int begin = min(chunk * length, vocab), end = min(begin + length, vocab);
+  const float* x = logits + static_cast<int64_t>(row) * vocab;
+  float best = -INFINITY;
+  int best_index = vocab, bad = 0;
+  for (int i = begin + tid; i < end; i += kChunkThreads) {
+    const float v = x[i];
+    if (!(fabsf(v) <= 3.402823466e38f)) bad = 1;
+    if (v > best) {
+      best = v;
+      best_index = i;
+    }
+  }
+  bad = ms::wave_sum_int(bad);
+  if ((tid & (ms::kWave - 1)) == 0) i_scratch[tid / ms::kWave] = bad;
+  if (tid == 0) shared_index = vocab;
+  const float chunk_best = ms::block_max(best, f_scratch);    // has barriers: i_scratch and shared_index are visible
+  if (best == chunk_best) atomicMin(&shared_index, best_index);
+  __syncthreads();
+  if (tid == 0) {
+    int any_bad = 0;
+    for (int w = 0; w < kChunkWaves; ++w) any_bad += i_scratch[w];
+    t.chunk_max[chunk] = chunk_best;                 // -inf for a chunk past the row's end
+    t.chunk_arg[chunk] = any_bad ? -1 : shared_index;
+  }
+}
+
+// The row's maximum and whether any chunk met a non-finite value, from stage 1's table.
+__device__ __forceinline__ float row_maximum(const RowTables& t, bool* bad) {
+  float row_max = -INFINITY;
+  bool any_bad = false;
+  for (int c = 0; c < kRowChunks; ++c) {
+    row_max = fmaxf(row_max, t.chunk_max[c]);
+    any_bad = any_bad || t.chunk_arg[c] < 0;
+  }
+  *bad = any_bad;
+  return row_max;
+}
+
+__global__ __launch_bounds__(kChunkThreads) void sample_ladder_kernel(const float* __restrict__ logits,
+                                                                      const float* __restrict__ temperature,
+                                                                      const int32_t* __restrict__ top_k,
+                                                                      float* __restrict__ workspace, int vocab) {
+  __shared__ int count_s[kChunkWaves][kLadder];
+  __shared__ float mass_s[kChunkWaves][kLadder + 1];
+  const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid & (ms::kWave - 1), wave = tid / ms::kWave;
+  const RowTables t = row_tables(workspace, row);
+  const float temp = temperature[row];
+  bool bad;
+  const float row_max = row_maximum(t, &bad);
+  if (bad || temp == 0.f) return;
+  const int k = top_k ? top_k[row] : 0;
+  const bool cut_k = k > 0 && k < vocab;
+  const float scaled_max = row_max / temp;
+  const int length = chunk_length(vocab);
+  const int begin = min(chunk * length, vocab), end = min(begin + length, vocab);
+  const float* x = logits + static_cast<int64_t>(row) * vocab;
+  int count[kLadder];
+  float mass[kLadder + 1];
+#pragma unroll
+  for (int c = 0; c < kLadder; ++c) count[c] = 0, mass[c] = 0.f;
+  mass[kLadder] = 0.f;
+  for (int i = begin + tid; i < end; i += kChunkThreads) {
+    const float v = x[i] / temp;
+    const float depth = scaled_max - v;
+    const float weight = cut_k ? 0.f : expf(v - scaled_max);
+    mass[kLadder] += weight;
+#pragma unroll
+    for (int c = 0; c < kLadder; ++c) {
+      const bool in = depth <= kLadderDepth[c];
+      count[c] += in;
+      mass[c] += in ? weight : 0.f;
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < kLadder; ++c) {
+    const int total = ms::wave_sum_int(count[c]);
+    const float sum = ms::wave_sum(mass[c]);
+    if (lane == 0) count_s[wave][c] = total, mass_s[wave][c] = sum;
+  }
+  {
+    const float sum = ms::wave_sum(mass[kLadder]);
+    if (lane == 0) mass_s[wave][kLadder] = sum;
+  }
+  __syncthreads();
+  if (tid <= kLadder) {
+    float sum = 0.f;
+    for (int w = 0; w < kChunkWaves; ++w) sum += mass_s[w][tid];
+    t.ladder_mass[chunk * (kLadder + 1) + tid] = sum;
+    if (tid < kLadder) {
+      int total = 0;
+      for (int w = 0; w < kChunkWaves; ++w) total += count_s[w][tid];
+      t.ladder_count[chunk * kLadder + tid] = total;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kChunkThreads) void sample_gather_kernel(const float* __restrict__ logits,
+                                                                      const float* __restrict__ temperature,
+                                                                      const int32_t* __restrict__ top_k,
+                                                                      const float* __restrict__ top_p,
+                                                                      float* __restrict__ workspace, int vocab) {
+  __shared__ int rung_s, base_s;
+  __shared__ int wave_count[kChunkWaves];
+  const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid & (ms::kWave - 1), wave = tid / ms::kWave;
+  const RowTables t = row_tables(workspace, row);
+  const float temp = temperature[row];
+  bool bad;
+  const float row_max = row_maximum(t, &bad);
+  if (bad || temp == 0.f) return;
+  const int k = top_k ? top_k[row] : 0;
+  const float p = top_p ? top_p[row] : 1.f;
+  const bool cut_k = k > 0 && k < vocab;
+  if (!cut_k && !(p < 1.f)) return;
+  if (tid == 0) {
+    float whole;
+    int total = 0;
+    const int rung = choose_rung(t, cut_k, k, p, &whole, &total);
+    int base = 0;
+    if (rung >= 0)
+      for (int c = 0; c < chunk; ++c) base += t.ladder_count[c * kLadder + rung];
+    rung_s = rung;
+    base_s = base;
+  }
+  __syncthreads();
+  const int rung = rung_s;
+  if (rung < 0) return;
+  float deepest = 0.f;
+#pragma unroll
+  for (int c = 0; c < kLadder; ++c)
+    if (c == rung) deepest = kLadderDepth[c];
+  const float scaled_max = row_max / temp;
+  const int length = chunk_length(vocab);
+  const int begin = min(chunk * length, vocab), end = min(begin + length, vocab);
+  const float* x = logits + static_cast<int64_t>(row) * vocab;
+  int written = base_s;
+  // 256 consecutive tokens a round; a token's place: what was written before, the
+  // tokens of the waves before its own in this round, those of the lanes before it
+  for (int first = begin; first < end; first += kChunkThreads) {
+    const int i = first + tid;
+    float v = 0.f;
+    bool in = false;
+    if (i < end) {
+      v = x[i] / temp;
+      in = scaled_max - v <= deepest;
+    }
+    const unsigned long long mask = __ballot(in);
+    __syncthreads();                         // the last round's counts are read
+    if (lane == 0) wave_count[wave] = __popcll(mask);
+    __syncthreads();
+    int before = 0, round_total = 0;
+    for (int w = 0; w < kChunkWaves; ++w) {
+      before += w < wave ? wave_count[w] : 0;
+      round_total += wave_count[w];
+    }
+    if (in) {
+      const int place = written + before + __popcll(mask & ((1ull << lane) - 1ull));
+      if (place < kListCap) {               // (the rung was chosen so that all fit)
+        t.list_values[place] = v;
+        t.list_indices[place] = i;
+      }
+    }
+    written += round_total;
+  }
+}
+
+// The view of one chunk of a row, for the draw without top-k and top-p.
+struct ChunkView {
+  const float* x;
+  float temp;
+  int begin;
+  int size;
+  __device__ __forceinline__ float value(int i) const { return x[begin + i] / temp; }
+  __device__ __forceinline__ int index(int i) const { return begin + i; }
+};
+
+__global__ __launch_bounds__(kThreads) void sample_choose_kernel(const float* __restrict__ logits,
+                                                                 const float* __restrict__ temperature,
+                                                                 const int32_t* __restrict__ top_k,
+                                                                 const float* __restrict__ top_p,
+                                                                 const float* __restrict__ uniform,
+                                                                 float* __restrict__ workspace,
+                                                                 int32_t* __restrict__ out, int vocab) {
+  __shared__ float f_scratch[kWaves];
+  __shared__ int i_scratch[kWaves];
+  __shared__ float seg_sum[kThreads];
+  __shared__ int seg_count[kThreads];
+  __shared__ int shared_index;
+  __shared__ float shared_total;
+  __shared__ int digit_count[kWaves][kDigits];
+  __shared__ float digit_mass[kWaves][kDigits];
+  __shared__ int rung_s, total_s, chunk_s;
+  __shared__ float whole_s, before_s;
+  __shared__ float list_values[kListCap];
+  __shared__ int list_indices[kListCap];
+
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const RowTables t = row_tables(workspace, row);
+  const float* x = logits + static_cast<int64_t>(row) * vocab;
+  const float temp = temperature[row];
+  Scratch sc{f_scratch, i_scratch, seg_sum, seg_count, &shared_index, &shared_total, digit_count, digit_mass};
+  bool bad;
+  const float row_max = row_maximum(t, &bad);
+  if (bad) {
+    if (tid == 0) out[row] = -1;
+    return;
+  }
+  if (temp == 0.f) {
+    // the first chunk that holds the maximum has its lowest index
+    if (tid == 0) {
+      int index = vocab;
+      for (int c = kRowChunks - 1; c >= 0; --c)
+        if (t.chunk_max[c] == row_max) index = t.chunk_arg[c];
+      out[row] = index;
+    }
+    return;
+  }
+  const float scaled_max = row_max / temp;
+  const int k = top_k ? top_k[row] : 0;
+  const float p = top_p ? top_p[row] : 1.f;
+  const bool cut_k = k > 0 && k < vocab;
+  const bool cut_p = p < 1.f;
+  const float u = uniform[row];
+
+  if (cut_k || cut_p) {
+    if (tid == 0) {
+      float whole;
+      int total = 0;
+      rung_s = choose_rung(t, cut_k, k, p, &whole, &total);
+      whole_s = whole;
+      total_s = total;
+    }
+    __syncthreads();
+    if (rung_s >= 0) {
+      const int n = total_s;
+      for (int i = tid; i < n; i += kThreads) {
+        list_values[i] = t.list_values[i];
+        list_indices[i] = t.list_indices[i];
+      }
+      __syncthreads();
+      const ListView list{list_values, list_indices, n};
+      const int chosen = choose(list, vocab, scaled_max, cut_k ? k : 0, p, u, cut_k ? -1.f : whole_s, 0.f, sc);
+      if (tid == 0) out[row] = chosen;
+      return;
+    }
+    const RowView whole{x, temp, vocab};
+    const int chosen = choose(whole, vocab, scaled_max, cut_k ? k : 0, p, u, -1.f, 0.f, sc);
+    if (tid == 0) out[row] = chosen;
+    return;
+  }
+
+  // Neither top-k nor top-p: the chunk in which the running mass passes uniform * whole
+  // is found from the chunks' masses, and the draw is made inside it.
+  if (tid == 0) {
+    float whole = 0.f;
+    for (int c = 0; c < kRowChunks; ++c) whole += t.ladder_mass[c * (kLadder + 1) + kLadder];
+    const float target = u * whole;
+    float running = 0.f;
+    int chunk = -1;
+    float before = 0.f;
+    int last_live = 0;
+    for (int c = 0; c < kRowChunks; ++c) {
+      const float mass = t.ladder_mass[c * (kLadder + 1) + kLadder];
+      if (mass > 0.f) last_live = c;
+      if (chunk < 0 && running + mass > target) {
+        chunk = c;
+        before = running;
+      }
+      running += mass;
+    }
+    if (chunk < 0) {                          // rounding: the target lies at the very end
+      chunk = last_live;
+      before = -INFINITY;                     // nothing in the chunk passes the target: its last token is taken
+    }
+    chunk_s = chunk;
+    before_s = before;
+    whole_s = whole;
+  }
+  __syncthreads();
+  const int length = chunk_length(vocab);
+  const int begin = min(chunk_s * length, vocab), end = min(begin + length, vocab);
+  const ChunkView part{x, temp, begin, end - begin};
+  const int chosen = choose(part, vocab, scaled_max, 0, 1.f, u, whole_s, before_s, sc);
+  if (tid == 0) out[row] = chosen;
+}
+
 // logits: float [rows, vocab]; temperature, top_p, uniform: float [rows] (null
 // temperature = all rows greedy); top_k: int32 [rows]; out: int32 [rows].
 extern "C" int ms_sample_rows(const void* logits, const void* temperature, const void* top_k, const void* top_p,
@@ -519,5 +885,42 @@ extern "C" int ms_sample_rows(const void* logits, const void* temperature, const
       static_cast<const int32_t*>(top_k), static_cast<const float*>(top_p), static_cast<const float*>(uniform),
       static_cast<int32_t*>(out), vocab);
   MS_CHECK_LAUNCH("sample_rows");
+  return 0;
+}
+
+// Bytes of the workspace that ms_sample_rows_chunked needs for `rows` rows.
+extern "C" size_t ms_sample_rows_workspace_bytes(int rows) {
+  return static_cast<size_t>(rows > 0 ? rows : 0) * row_table_floats() * sizeof(float);
+}
+
+// The same choice as ms_sample_rows for a large vocabulary, the passes over a row
+// shared by 32 workgroups; temperature is not null.  workspace: device memory of
+// ms_sample_rows_workspace_bytes(rows), aligned to 4 bytes, the caller's until the
+// call's work on the stream is done.
+extern "C" int ms_sample_rows_chunked(const void* logits, const void* temperature, const void* top_k,
+                                      const void* top_p, const void* uniform, void* out, void* workspace,
+                                      size_t workspace_bytes, int rows, int vocab, hipStream_t stream) {
+  MS_REQUIRE(rows > 0 && rows <= 65535 && vocab > 0, "sample_rows_chunked: bad shape %d x %d", rows, vocab);
+  MS_REQUIRE(temperature && uniform, "sample_rows_chunked: temperature and uniform numbers are needed");
+  MS_REQUIRE(workspace && workspace_bytes >= ms_sample_rows_workspace_bytes(rows),
+             "sample_rows_chunked: the workspace has %zu bytes, %zu are needed", workspace_bytes,
+             ms_sample_rows_workspace_bytes(rows));
+  float* tables = static_cast<float*>(workspace);
+  const dim3 grid(kRowChunks, rows);
+  hipLaunchKernelGGL(sample_scan_kernel, grid, dim3(kChunkThreads), 0, stream, static_cast<const float*>(logits),
+                     tables, vocab);
+  MS_CHECK_LAUNCH("sample_scan");
+  hipLaunchKernelGGL(sample_ladder_kernel, grid, dim3(kChunkThreads), 0, stream, static_cast<const float*>(logits),
+                     static_cast<const float*>(temperature), static_cast<const int32_t*>(top_k), tables, vocab);
+  MS_CHECK_LAUNCH("sample_ladder");
+  hipLaunchKernelGGL(sample_gather_kernel, grid, dim3(kChunkThreads), 0, stream, static_cast<const float*>(logits),
+                     static_cast<const float*>(temperature), static_cast<const int32_t*>(top_k),
+                     static_cast<const float*>(top_p), tables, vocab);
+  MS_CHECK_LAUNCH("sample_gather");
+  hipLaunchKernelGGL(sample_choose_kernel, dim3(rows), dim3(kThreads), 0, stream, static_cast<const float*>(logits),
+                     static_cast<const float*>(temperature), static_cast<const int32_t*>(top_k),
+                     static_cast<const float*>(top_p), static_cast<const float*>(uniform), tables,
+                     static_cast<int32_t*>(out), vocab);
+  MS_CHECK_LAUNCH("sample_choose");
   return 0;
 }

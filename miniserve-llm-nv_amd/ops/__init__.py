@@ -560,6 +560,12 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     return out
 
 
+# Vocabulary from which a sampled row is handled by many workgroups, and the bytes of
+# the tables that this takes a row (csrc/sampling.hip: row_table_floats).
+SAMPLE_CHUNKED_FROM = 8192
+_SAMPLE_ROW_TABLE_BYTES = 4 * (32 * (2 + 8 + 8 + 1) + 2 * 4096)
+
+
 def sample_rows(
     logits: torch.Tensor,
     *,
@@ -595,6 +601,12 @@ def sample_rows(
         chunk_index = torch.empty((rows, chunks), dtype=torch.int32, device=logits.device)
         call("ms_argmax_rows", _ptr(logits), _ptr(chunk_max), _ptr(chunk_index), _ptr(out), rows, vocab, chunks,
              _stream())
+        return out
+    if temperature is not None and vocab >= SAMPLE_CHUNKED_FROM and rows <= 65535:
+        # a long row: its passes are shared by many workgroups; tables of a few KB a row between the stages
+        workspace = torch.empty(rows * _SAMPLE_ROW_TABLE_BYTES, dtype=torch.uint8, device=logits.device)
+        call("ms_sample_rows_chunked", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
+             _ptr(out), _ptr(workspace), workspace.numel(), rows, vocab, _stream())
         return out
     call("ms_sample_rows", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(out),
          rows, vocab, _stream())
