@@ -10,7 +10,8 @@ rate of one 2,048-token prompt with its fraction of the bf16 MFMA peak, the
 fraction of the HBM peak that the decode step reaches, decode rates at batch 1 and
 64, a mixed run (64 requests with prompts of 128 to 2,048 tokens, portions of 512
 beside decode tokens, through the scheduler), and what the card reaches on a plain
-device copy and a large library product.
+device copy and a large library product (the two fractions are given against these
+measured rates as well as against the published peaks).
 """
 
 from __future__ import annotations
@@ -281,6 +282,7 @@ def main() -> int:
             "tokens": args.prefill_tokens,
             "ms": round(1000 * prefill_s, 3),
             "frac": round(flops / prefill_s / (PEAK_TFLOPS[args.dtype] * 1e12), 5),
+            "frac_of_measured_gemm": round(flops / prefill_s / (gemm_tflops * 1e12), 5),
         },
         "roofline": {
             "bound": "hbm",
@@ -288,6 +290,7 @@ def main() -> int:
             "peak": HBM_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_GBPS, 5),
+            "frac_of_measured_copy": round(achieved / copy_gbps, 5),
         },
         "points": points,
         "mixed": mixed,
