@@ -519,9 +519,11 @@ extern "C" int ms_argmax_rows(const void* logits, void* chunk_max, void* chunk_i
 // ladder's counts and masses per chunk; (3) the short list, every chunk writing its
 // share at its place in token order; (4) one workgroup a row makes the choice: among
 // the list, or, without top-k and top-p, inside the chunk that the running mass
-// singles out, or - the candidates do not fit a list - over the whole row as above.
-// Tables between the stages (per row): chunk_max, chunk_arg [chunks]; ladder_count
-// [chunks][kLadder]; ladder_mass [chunks][kLadder + 1]; list_values, list_indices [kListCap].
+// singles out, or - no rung of the ladder holds the candidates - over the whole row as above.
+// The list lies in device memory and may be as long as the row; the last stage copies
+// it into LDS when it is short.  Tables between the stages (per row): chunk_max,
+// chunk_arg [chunks]; ladder_count [chunks][kLadder]; ladder_mass [chunks][kLadder + 1];
+// list_values, list_indices [vocab].
 constexpr int kRowChunks = 32;
 constexpr int kChunkThreads = 256;
 constexpr int kChunkWaves = kChunkThreads / ms::kWave;
@@ -535,19 +537,19 @@ struct RowTables {
   int* list_indices;
 };
 
-__host__ __device__ inline size_t row_table_floats() {
-  return static_cast<size_t>(kRowChunks) * (2 + kLadder + kLadder + 1) + 2 * static_cast<size_t>(kListCap);
+__host__ __device__ inline size_t row_table_floats(int vocab) {
+  return static_cast<size_t>(kRowChunks) * (2 + kLadder + kLadder + 1) + 2 * static_cast<size_t>(vocab);
 }
 
-__device__ __forceinline__ RowTables row_tables(float* workspace, int row) {
-  float* base = workspace + static_cast<size_t>(row) * row_table_floats();
+__device__ __forceinline__ RowTables row_tables(float* workspace, int row, int vocab) {
+  float* base = workspace + static_cast<size_t>(row) * row_table_floats(vocab);
   RowTables t;
   t.chunk_max = base;
   t.chunk_arg = reinterpret_cast<int*>(base + kRowChunks);
   t.ladder_count = reinterpret_cast<int*>(base + 2 * kRowChunks);
   t.ladder_mass = base + 2 * kRowChunks + kRowChunks * kLadder;
   t.list_values = base + 2 * kRowChunks + kRowChunks * (2 * kLadder + 1);
-  t.list_indices = reinterpret_cast<int*>(t.list_values + kListCap);
+  t.list_indices = reinterpret_cast<int*>(t.list_values + vocab);
   return t;
 }
 
@@ -568,7 +570,6 @@ __device__ int choose_rung(const RowTables& t, bool cut_k, int k, float p, float
       total += t.ladder_count[c * kLadder + r];
       sum += t.ladder_mass[c * (kLadder + 1) + r];
     }
-    if (total > kListCap) return -1;
     // (a little more than top_p of the mass: the sums here and those of the choice differ in rounding)
     const bool enough = cut_k ? total >= k : sum > (p + 1e-4f) * whole;
     if (enough) {
@@ -585,7 +586,7 @@ __global__ __launch_bounds__(kChunkThreads) void sample_scan_kernel(const float*
   __shared__ int i_scratch[kChunkWaves];
   __shared__ int shared_index;
   const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
-  const RowTables t = row_tables(workspace, row);
+  const RowTables t = row_tables(workspace, row, vocab);
   const int length = chunk_length(vocab);
   const int begin = min(chunk * length, vocab), end = min(begin + length, vocab);
   const float* x = logits + static_cast<int64_t>(row) * vocab;
@@ -633,7 +634,7 @@ __global__ __launch_bounds__(kChunkThreads) void sample_ladder_kernel(const floa
   __shared__ float mass_s[kChunkWaves][kLadder + 1];
   const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
   const int lane = tid & (ms::kWave - 1), wave = tid / ms::kWave;
-  const RowTables t = row_tables(workspace, row);
+  const RowTables t = row_tables(workspace, row, vocab);
   const float temp = temperature[row];
   bool bad;
   const float row_max = row_maximum(t, &bad);
@@ -693,7 +694,7 @@ __global__ __launch_bounds__(kChunkThreads) void sample_gather_kernel(const floa
   __shared__ int wave_count[kChunkWaves];
   const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
   const int lane = tid & (ms::kWave - 1), wave = tid / ms::kWave;
-  const RowTables t = row_tables(workspace, row);
+  const RowTables t = row_tables(workspace, row, vocab);
   const float temp = temperature[row];
   bool bad;
   const float row_max = row_maximum(t, &bad);
@@ -745,7 +746,7 @@ __global__ __launch_bounds__(kChunkThreads) void sample_gather_kernel(const floa
     }
     if (in) {
       const int place = written + before + __popcll(mask & ((1ull << lane) - 1ull));
-      if (place < kListCap) {               // (the rung was chosen so that all fit)
+      if (place < vocab) {                  // (it is: the places are the ranks of tokens of the row)
         t.list_values[place] = v;
         t.list_indices[place] = i;
       }
@@ -785,7 +786,7 @@ __global__ __launch_bounds__(kThreads) void sample_choose_kernel(const float* __
   __shared__ int list_indices[kListCap];
 
   const int row = blockIdx.x, tid = threadIdx.x;
-  const RowTables t = row_tables(workspace, row);
+  const RowTables t = row_tables(workspace, row, vocab);
   const float* x = logits + static_cast<int64_t>(row) * vocab;
   const float temp = temperature[row];
   Scratch sc{f_scratch, i_scratch, seg_sum, seg_count, &shared_index, &shared_total, digit_count, digit_mass};
@@ -823,13 +824,19 @@ __global__ __launch_bounds__(kThreads) void sample_choose_kernel(const float* __
     __syncthreads();
     if (rung_s >= 0) {
       const int n = total_s;
-      for (int i = tid; i < n; i += kThreads) {
-        list_values[i] = t.list_values[i];
-        list_indices[i] = t.list_indices[i];
+      int chosen;
+      if (n <= kListCap) {
+        for (int i = tid; i < n; i += kThreads) {
+          list_values[i] = t.list_values[i];
+          list_indices[i] = t.list_indices[i];
+        }
+        __syncthreads();
+        const ListView list{list_values, list_indices, n};
+        chosen = choose(list, vocab, scaled_max, cut_k ? k : 0, p, u, cut_k ? -1.f : whole_s, 0.f, sc);
+      } else {
+        const ListView list{t.list_values, t.list_indices, n};      // a long list stays where it is
+        chosen = choose(list, vocab, scaled_max, cut_k ? k : 0, p, u, cut_k ? -1.f : whole_s, 0.f, sc);
       }
-      __syncthreads();
-      const ListView list{list_values, list_indices, n};
-      const int chosen = choose(list, vocab, scaled_max, cut_k ? k : 0, p, u, cut_k ? -1.f : whole_s, 0.f, sc);
       if (tid == 0) out[row] = chosen;
       return;
     }
@@ -888,23 +895,23 @@ extern "C" int ms_sample_rows(const void* logits, const void* temperature, const
   return 0;
 }
 
-// Bytes of the workspace that ms_sample_rows_chunked needs for `rows` rows.
-extern "C" size_t ms_sample_rows_workspace_bytes(int rows) {
-  return static_cast<size_t>(rows > 0 ? rows : 0) * row_table_floats() * sizeof(float);
+// Bytes of the workspace that ms_sample_rows_chunked needs for `rows` rows of `vocab` tokens.
+extern "C" size_t ms_sample_rows_workspace_bytes(int rows, int vocab) {
+  return static_cast<size_t>(rows > 0 ? rows : 0) * row_table_floats(vocab > 0 ? vocab : 0) * sizeof(float);
 }
 
 // The same choice as ms_sample_rows for a large vocabulary, the passes over a row
 // shared by 32 workgroups; temperature is not null.  workspace: device memory of
-// ms_sample_rows_workspace_bytes(rows), aligned to 4 bytes, the caller's until the
+// ms_sample_rows_workspace_bytes(rows, vocab), aligned to 4 bytes, the caller's until the
 // call's work on the stream is done.
 extern "C" int ms_sample_rows_chunked(const void* logits, const void* temperature, const void* top_k,
                                       const void* top_p, const void* uniform, void* out, void* workspace,
                                       size_t workspace_bytes, int rows, int vocab, hipStream_t stream) {
   MS_REQUIRE(rows > 0 && rows <= 65535 && vocab > 0, "sample_rows_chunked: bad shape %d x %d", rows, vocab);
   MS_REQUIRE(temperature && uniform, "sample_rows_chunked: temperature and uniform numbers are needed");
-  MS_REQUIRE(workspace && workspace_bytes >= ms_sample_rows_workspace_bytes(rows),
+  MS_REQUIRE(workspace && workspace_bytes >= ms_sample_rows_workspace_bytes(rows, vocab),
              "sample_rows_chunked: the workspace has %zu bytes, %zu are needed", workspace_bytes,
-             ms_sample_rows_workspace_bytes(rows));
+             ms_sample_rows_workspace_bytes(rows, vocab));
   float* tables = static_cast<float*>(workspace);
   const dim3 grid(kRowChunks, rows);
   hipLaunchKernelGGL(sample_scan_kernel, grid, dim3(kChunkThreads), 0, stream, static_cast<const float*>(logits),

@@ -560,10 +560,14 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     return out
 
 
-# Vocabulary from which a sampled row is handled by many workgroups, and the bytes of
-# the tables that this takes a row (csrc/sampling.hip: row_table_floats).
+# Vocabulary from which a sampled row is handled by many workgroups.
 SAMPLE_CHUNKED_FROM = 8192
-_SAMPLE_ROW_TABLE_BYTES = 4 * (32 * (2 + 8 + 8 + 1) + 2 * 4096)
+
+
+def _sample_row_table_bytes(vocab: int) -> int:
+    """Bytes a row that the stages of the chunked choice share (csrc/sampling.hip: row_table_floats)."""
+
+    return 4 * (32 * (2 + 8 + 8 + 1) + 2 * vocab)
 
 
 def sample_rows(
@@ -603,8 +607,9 @@ def sample_rows(
              _stream())
         return out
     if temperature is not None and vocab >= SAMPLE_CHUNKED_FROM and rows <= 65535:
-        # a long row: its passes are shared by many workgroups; tables of a few KB a row between the stages
-        workspace = torch.empty(rows * _SAMPLE_ROW_TABLE_BYTES, dtype=torch.uint8, device=logits.device)
+        # a long row: its passes are shared by many workgroups; between the stages small tables and room for
+        # the list of the tokens that can stay
+        workspace = torch.empty(rows * _sample_row_table_bytes(vocab), dtype=torch.uint8, device=logits.device)
         call("ms_sample_rows_chunked", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
              _ptr(out), _ptr(workspace), workspace.numel(), rows, vocab, _stream())
         return out
