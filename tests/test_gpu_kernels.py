@@ -729,10 +729,11 @@ def test_sampling_matches_the_plain_implementation(ops, vocab):
 
 
 def test_sampling_from_the_short_list_and_from_the_whole_row(ops):
-    """With top-k or top-p the kernel gathers the tokens near the maximum into a short
-    list when they fit (4096) and chooses among them, else over the whole row; both give
-    the plain implementation's token.  Rows with a few outstanding tokens (as a model's
-    logits have) and flat rows; top-k beyond the list's size; top-p close to 1."""
+    """With top-k or top-p the kernels gather the tokens near the maximum into a list and
+    choose among them: in LDS when they are few (4096), in device memory when they are
+    many (top-k 4097 and 5000 here), and over the whole row when no distance from the
+    maximum holds them (top-p 0.9999); all give the plain implementation's token.  Rows
+    with a few outstanding tokens (as a model's logits have) and flat rows."""
 
     vocab, rows = 50021, 36
     generator = torch.Generator().manual_seed(7)
