@@ -94,6 +94,70 @@ struct Scratch {
   float (*digit_mass)[kDigits];    // [kWaves][kDigits]
 };
 
+// The same choice among at most kSmallView tokens, one to a thread: no thresholds are
+// searched; a token's rank (by value, lower index first among equals), the mass ahead of
+// it and the running mass up to it are sums over the few tokens, which every thread takes
+// in the same order.  seg_sum holds the values, then the weights; seg_count the indices.
+constexpr int kSmallView = 256;
+
+template <typename View>
+__device__ int choose_among_few(const View& view, int limit_index, float scaled_max, int k, float p, float uniform,
+                                float whole_mass, float mass_before, const Scratch& sc) {
+  const int tid = threadIdx.x;
+  const int n = view.size;
+  const bool live = tid < n;
+  const float value = live ? view.value(tid) : 0.f;
+  const int index = live ? view.index(tid) : limit_index;
+  const float weight = live ? expf(value - scaled_max) : 0.f;
+  float* values = sc.seg_sum;
+  float* weights = sc.seg_sum + kSmallView;
+  int* indices = sc.seg_count;
+  __syncthreads();                     // whoever read these arrays last is done
+  if (live) values[tid] = value, indices[tid] = index;
+  __syncthreads();
+  bool kept = live;
+  if (live && k > 0 && k < n) {
+    int rank = 0;
+    for (int j = 0; j < n; ++j) rank += values[j] > value || (values[j] == value && indices[j] < index);
+    kept = rank < k;
+  }
+  if (live) weights[tid] = kept ? weight : 0.f;
+  __syncthreads();
+  if (p < 1.f) {
+    float kept_mass = 0.f, ahead = 0.f;
+    for (int j = 0; j < n; ++j) {
+      kept_mass += weights[j];
+      ahead += values[j] > value ? weights[j] : 0.f;
+    }
+    const float limit = p * (whole_mass >= 0.f ? whole_mass : kept_mass);
+    kept = kept && !(ahead > limit);
+    __syncthreads();                   // every thread has read the weights
+    if (live) weights[tid] = kept ? weight : 0.f;
+    __syncthreads();
+  }
+  float total = 0.f, running = 0.f;
+  for (int j = 0; j < n; ++j) {
+    total += weights[j];
+    if (j == tid) running = total;     // the running mass up to and with this token
+  }
+  const float target = (k == 0 && !(p < 1.f) && whole_mass >= 0.f) ? uniform * whole_mass - mass_before
+                                                                     : uniform * total;
+  if (tid == 0) *sc.shared_index = limit_index;
+  __syncthreads();
+  if (live && kept && running > target) atomicMin(sc.shared_index, index);
+  __syncthreads();
+  const int chosen = *sc.shared_index;
+  __syncthreads();
+  // no token's running mass passes the target (rounding at the very end): the last kept one
+  if (chosen == limit_index) {
+    int last_kept = -1;
+    for (int j = 0; j < n; ++j)
+      if (weights[j] > 0.f) last_kept = max(last_kept, indices[j]);
+    return last_kept >= 0 ? last_kept : indices[0];
+  }
+  return chosen;
+}
+
 // temperature -> top-k -> top-p -> draw over `view`; `limit_index`: an index beyond
 // every token's; `whole_mass`: the mass of all tokens where the view holds only some
 // of them and top-k is off (top_p is a share of that), else negative; `mass_before`:
@@ -109,6 +173,8 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
   const int seg = (n + kThreads - 1) / kThreads;
   const int seg_begin = min(tid * seg, n);
   const int seg_end = min(seg_begin + seg, n);
+
+  if (n <= kSmallView) return choose_among_few(view, limit_index, scaled_max, k, p, uniform, whole_mass, mass_before, sc);
 
   Keep keep;
   keep.k_threshold = 0u;
