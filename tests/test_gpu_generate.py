@@ -284,6 +284,59 @@ def test_decode_graphs_replay_like_eager_steps(dtype, model_folders):
     assert sorted(runners[0]._decode_graphs) == [1, 2, 4]           # three requests ran in the step of four
 
 
+def test_steps_planned_ahead_on_the_device_change_no_token(model_folders):
+    """The engine over the real runner, requests arriving while others run, one cancelled
+    while it waits: with the next step planned while the GPU runs this one (recorded
+    steps and steps with prompt portions) every request gets the tokens it gets when
+    nothing is planned ahead, to the bit in 32-bit arithmetic, and nothing is left held."""
+
+    from miniserve_amd.config import EngineConfig
+    from miniserve_amd.engine import Engine, ModelRunner, SamplingParams
+
+    folder, block = model_folders["b"]
+    config = read_config(folder)
+    prompts = [random_tokens(n, config["vocab_size"], 900 + n) for n in (3, 41, 18, 29, 7, 55)]
+    arrivals = [0, 0, 2, 5, 9, 9]
+    limits = [14, 6, 11, 9, 20, 5]
+
+    class NothingAhead:
+        """The runner without the two calls that plan ahead."""
+
+        def __init__(self, runner):
+            self._runner = runner
+
+        def __getattr__(self, name):
+            if name in ("prepare_decode", "prepare_step"):
+                raise AttributeError(name)
+            return getattr(self._runner, name)
+
+    def run(plan_ahead):
+        runner = ModelRunner.from_folder(folder, EngineConfig(
+            dtype="float32", kv_block_size=block, num_kv_blocks=40, max_num_seqs=3, enable_chunked_prefill=True,
+            prefill_chunk_size=7, max_num_batched_tokens=12))
+        engine = Engine(runner if plan_ahead else NothingAhead(runner))
+        step, added, cancelled = 0, 0, False
+        while added < len(prompts) or engine.has_unfinished():
+            while added < len(prompts) and arrivals[added] <= step:
+                engine.add_request(f"r{added}", prompts[added], SamplingParams(max_new_tokens=limits[added]), arrival_ns=added)
+                added += 1
+            engine.step()
+            if not cancelled and added == len(prompts) and "r5" in engine._sequences and step >= 11:
+                engine.cancel("r5")
+                cancelled = True
+            runner.cache.assert_invariants()
+            step += 1
+            assert step < 400
+        assert cancelled and runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (40,)
+        return [list(engine.pop_result(f"r{i}").token_ids) for i in range(5)], runner
+
+    expected, _ = run(False)
+    got, runner = run(True)
+    assert got == expected
+    assert [len(tokens) for tokens in got] == limits[:5]
+    assert runner.prepared_mixed_steps > 0 and runner.prepared_steps > runner.prepared_mixed_steps
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_recorded_steps_filled_up_with_spare_rows(dtype, model_folders):
     """Nine to eleven live requests are served by the recorded step of twelve: the rows
