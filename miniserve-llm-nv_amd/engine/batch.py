@@ -31,6 +31,9 @@ class StepEntry:
     want: tuple[int, ...] = ()
 
     def __post_init__(self) -> None:
+        tokens, want = self.token_ids, self.want
+        if len(tokens) == 1 and type(tokens[0]) is int and tokens[0] >= 0 and (want == (0,) or want == ()):
+            return          # a decoded token: the common case, checked without loops
         if not self.token_ids:
             raise ValueError(f"entry {self.request_id!r} brings no tokens.")
         if any(not isinstance(t, int) or isinstance(t, bool) or t < 0 for t in self.token_ids):
