@@ -634,25 +634,34 @@ def test_library_product_for_many_rows(ops, m, n, k, monkeypatch):
         ops.linear(x, w, accumulate_into=torch.zeros(m, n + 1, device=DEVICE))
 
 
-def test_library_product_inside_a_recorded_graph(ops, monkeypatch):
+@pytest.mark.parametrize("m,n,k", [(64, 512, 256), (64, 1024, 2048), (33, 1024, 3072), (48, 4096, 1024), (64, 6144, 1024)])
+def test_library_product_inside_a_recorded_graph(ops, monkeypatch, m, n, k):
     """Replayed several times with eager work between the replays; every replay gives
-    what the eager call gives for the inputs of that moment."""
+    what the eager call gives for the inputs of that moment: plain, and added into a
+    32-bit tensor (the shapes of a decode step of 33 to 64 rows among them)."""
 
     monkeypatch.setattr(ops, "SKINNY_KERNEL_ROWS", 16)
-    x = rand(64, 256, seed=1, dtype=torch.bfloat16)
-    w = rand(512, 256, seed=2, dtype=torch.bfloat16, scale=0.1)
+    x = rand(m, k, seed=1, dtype=torch.bfloat16)
+    w = rand(n, k, seed=2, dtype=torch.bfloat16, scale=0.1)
+    base = rand(m, n, seed=3)
     ops.linear(x, w)                                        # plan and workspace exist before the recording
+    ops.linear(x, w, accumulate_into=base.clone())
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
+    total = base.clone()
     with torch.cuda.graph(graph):
         out = ops.linear(x, w, out_float32=True)
+        ops.linear(x, w, accumulate_into=total)
     for round_index in range(4):
-        x.copy_(rand(64, 256, seed=10 + round_index, dtype=torch.bfloat16))
+        x.copy_(rand(m, k, seed=10 + round_index, dtype=torch.bfloat16))
+        total.copy_(base)
         graph.replay()
         torch.cuda.synchronize()
         expected = ops.linear(x, w, out_float32=True)       # eager work between the replays
+        expected_total = ops.linear(x, w, accumulate_into=base.clone())
         torch.cuda.synchronize()
         assert torch.equal(out, expected)
+        assert torch.equal(total, expected_total)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
