@@ -9,7 +9,7 @@ of ``--size``) with random weights.  One JSON line is printed: decoded tokens a 
 rate of one 2,048-token prompt with its fraction of the bf16 MFMA peak, the
 fraction of the HBM peak that the decode step reaches, decode rates at batch 1 and
 64, a mixed run (64 requests with prompts of 128 to 2,048 tokens, portions of 512
-beside decode tokens, through the scheduler), and what the card reaches on a plain
+beside decode tokens under a budget of 2,048 tokens a step, through the scheduler), and what the card reaches on a plain
 device copy and a large library product (the two fractions are given against these
 measured rates as well as against the published peaks).
 """
@@ -160,7 +160,7 @@ def main() -> int:
         pages = max(sum(-(-(len(prompt) + new_tokens) // 16) for prompt in prompts) for prompts in rounds) + 16
         engine_config = EngineConfig(
             dtype=args.dtype, max_model_len=args.context, max_num_seqs=requests,
-            max_num_batched_tokens=min(args.context, 2 * chunk), kv_block_size=16, num_kv_blocks=pages,
+            max_num_batched_tokens=min(args.context, 4 * chunk), kv_block_size=16, num_kv_blocks=pages,
             enable_chunked_prefill=True, prefill_chunk_size=chunk, max_pending_requests=max(64, requests),
             decode_graphs=not args.eager,
         )
@@ -185,7 +185,8 @@ def main() -> int:
         return {
             "value": round(total / elapsed, 1), "unit": "tokens/s, prompt and generated", "requests": requests,
             "prompt_tokens": counters["prefill_tokens"], "generated_tokens": counters["decode_tokens"] + requests,
-            "steps": counters["steps"], "steps_with_both": mixed_steps, "chunk": chunk, "ms": round(1000 * elapsed, 1),
+            "steps": counters["steps"], "steps_with_both": mixed_steps, "chunk": chunk,
+            "token_budget": engine_config.max_num_batched_tokens, "ms": round(1000 * elapsed, 1),
             "preemptions": counters.get("preemptions", 0),
         }
 
