@@ -25,6 +25,9 @@
 // pass runs over that short list; a row whose candidates do not fit, and a row with
 // neither top-k nor top-p, is handled over its whole length.
 #include "common.hpp"
+#include "miniserve_hip.h"
+
+#include <mutex>
 
 namespace {
 
@@ -574,6 +577,68 @@ extern "C" int ms_argmax_rows(const void* logits, void* chunk_max, void* chunk_i
                      static_cast<const float*>(chunk_max), static_cast<const int32_t*>(chunk_index),
                      static_cast<int32_t*>(out), chunks);
   MS_CHECK_LAUNCH("argmax_rows");
+  return 0;
+}
+
+// ---- the greedy choice for callers that cannot allocate ---------------------------------
+//
+// The partial results of stage 1 lie in a file-scope device array instead of buffers
+// that the caller brings: kStaticArgmaxMaxRows rows x kStaticArgmaxChunks chunks x
+// (one float + one int32) = 512 KiB, which every GPU that the library runs on holds
+// until the process ends.  In host code the array's name is only a stand-in; its
+// device address is asked for once per device and kept.
+constexpr int kStaticArgmaxMaxRows = 1024;
+constexpr int kStaticArgmaxChunks = 64;
+constexpr size_t kStaticArgmaxBytes = static_cast<size_t>(kStaticArgmaxMaxRows) * kStaticArgmaxChunks * 8;
+static __device__ __align__(256) unsigned char scratch[kStaticArgmaxBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void* g_scratch_of_device[kMaxDevices] = {};
+
+// The address of `scratch` on the current device (asked for at the first call on that device).
+int scratch_of_current_device(void** address) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return ms_fail("argmax_rows_static: hipGetDevice: %s", hipGetErrorString(err));
+  MS_REQUIRE(device >= 0 && device < kMaxDevices, "argmax_rows_static: device %d is outside 0..%d", device,
+             kMaxDevices - 1);
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (g_scratch_of_device[device] == nullptr) {
+    void* found = nullptr;
+    err = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || found == nullptr)
+      return ms_fail("argmax_rows_static: hipGetSymbolAddress on device %d: %s", device, hipGetErrorString(err));
+    g_scratch_of_device[device] = found;
+  }
+  *address = g_scratch_of_device[device];
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int ms_argmax_rows_static(const void* logits, void* out, int rows, int vocab, hipStream_t stream) {
+  MS_REQUIRE(logits != nullptr && out != nullptr, "argmax_rows_static: null operand");
+  MS_REQUIRE(vocab > 0, "argmax_rows_static: a vocabulary of %d", vocab);
+  MS_REQUIRE(rows > 0 && rows <= kStaticArgmaxMaxRows,
+             "argmax_rows_static: %d rows are outside 1..%d (the static scratch holds no more; "
+             "ms_argmax_rows takes buffers of any size)",
+             rows, kStaticArgmaxMaxRows);
+  void* base = nullptr;
+  if (int status = scratch_of_current_device(&base)) return status;
+  const int chunks = vocab < kStaticArgmaxChunks ? vocab : kStaticArgmaxChunks;
+  // Stage 1 writes every one of the rows x chunks entries that stage 2 reads, so nothing
+  // of an earlier call is seen and nothing needs clearing.
+  float* chunk_max = static_cast<float*>(base);
+  int32_t* chunk_index = reinterpret_cast<int32_t*>(static_cast<unsigned char*>(base) + kStaticArgmaxBytes / 2);
+  hipLaunchKernelGGL(argmax_chunks_kernel, dim3(chunks, rows), dim3(kArgmaxThreads), 0, stream,
+                     static_cast<const float*>(logits), chunk_max, chunk_index, vocab, chunks);
+  MS_CHECK_LAUNCH("argmax_chunks (static)");
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(ms::kWave), 0, stream, chunk_max, chunk_index,
+                     static_cast<int32_t*>(out), chunks);
+  MS_CHECK_LAUNCH("argmax_rows (static)");
   return 0;
 }
 
