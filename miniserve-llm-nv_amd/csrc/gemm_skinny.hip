@@ -95,6 +95,17 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  // The += epilogue reads the output before it adds: the first value that this thread
+  // will add to is asked for now, so that it has arrived when the sums are made (no
+  // other thread writes it).
+  float residual_ahead = 0.f;
+  if (epilogue == kAddF32 && threadIdx.x < RB * MB * 256) {
+    const int n_local = threadIdx.x & 15, m_local = (threadIdx.x >> 4) & 15, tile = threadIdx.x >> 8;
+    const int rb = tile / MB, mb = tile - rb * MB;
+    const int row_m = 16 * mb + m_local, col_n = row_start[rb] + n_local;
+    if (row_m < m && col_n < row_limit && n_local < rows) residual_ahead = out_f32[static_cast<int64_t>(row_m) * n + col_n];
+  }
+
   // NORM: this lane makes column m = r of x from row r of h, and sums its squares
   const float* h_row = NORM ? h + static_cast<int64_t>(min(r, m - 1)) * k : nullptr;
   float square_sum = 0.f;
@@ -109,17 +120,21 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) a[u][rb] = (live && r < rows) ? ms::load_bf16x8(w_row[rb] + k0) : ms::zero_bf16x8();
       if (NORM) {
-        bf16x8 made = ms::zero_bf16x8();
-        if (live && x_live[0]) {
-          const float4 lo = *reinterpret_cast<const float4*>(h_row + k0);
-          const float4 hi = *reinterpret_cast<const float4*>(h_row + k0 + 4);
-          const bf16x8 nw = ms::load_bf16x8(norm_weight + k0);
-          const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        // Loads without a branch around them (a slice past the end reads the row's last
+        // one and counts for nothing): behind a branch each would be waited for in
+        // turn, and the step would cost as many round trips as it has slices.
+        const int k_read = live ? k0 : k - 8;
+        const float4 lo = *reinterpret_cast<const float4*>(h_row + k_read);
+        const float4 hi = *reinterpret_cast<const float4*>(h_row + k_read + 4);
+        const bf16x8 nw = ms::load_bf16x8(norm_weight + k_read);
+        const bool keep = live && x_live[0];
+        const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        bf16x8 made;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            square_sum = fmaf(v[i], v[i], square_sum);
-            made[i] = static_cast<__bf16>(static_cast<float>(nw[i]) * v[i]);
-          }
+        for (int i = 0; i < 8; ++i) {
+          const float value = keep ? v[i] : 0.f;
+          square_sum = fmaf(value, value, square_sum);
+          made[i] = static_cast<__bf16>(static_cast<float>(nw[i]) * value);
         }
         b[u][0] = made;
       } else {
@@ -177,7 +192,8 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     } else if (epilogue == kStoreF32) {
       out_f32[static_cast<int64_t>(row_m) * n + col_n] = sum;
     } else if (epilogue == kAddF32) {
-      out_f32[static_cast<int64_t>(row_m) * n + col_n] += sum;
+      float* place = out_f32 + static_cast<int64_t>(row_m) * n + col_n;
+      *place = (index == static_cast<int>(threadIdx.x) ? residual_ahead : *place) + sum;
     } else {
       float up = 0.f;
 #pragma unroll

@@ -6,7 +6,7 @@ torch is the allocator and gives the stream.
 
 from __future__ import annotations
 
-import gc
+import contextlib
 
 import torch
 
@@ -317,14 +317,10 @@ def attention(
 
 
 _EPILOGUE_BF16, _EPILOGUE_F32, _EPILOGUE_ADD_F32, _EPILOGUE_SILU_MUL = 0, 1, 2, 3
-# This library's product takes up to SKINNY_KERNEL_ROWS rows.  Up to SKINNY_MAX_ROWS
-# rows and for a matrix below SKINNY_ALWAYS_BYTES it is always the faster one; beyond
-# either, which of the two products is faster depends on the matrix (on MI355X: this
-# one for the matrices of a small model, hipBLASLt for most large ones), so both are
-# timed once for a shape.
+# This library's product takes up to SKINNY_KERNEL_ROWS rows; the norm as its prologue
+# up to SKINNY_MAX_ROWS rows.
 SKINNY_MAX_ROWS = 16
 SKINNY_KERNEL_ROWS = 64
-SKINNY_ALWAYS_BYTES = 32 << 20
 
 
 _GEMM_WORKSPACE_BYTES = 64 << 20
@@ -356,87 +352,68 @@ def _library_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, a
     if workspace is None:
         workspace = _gemm_workspaces[index] = torch.empty(_GEMM_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
     m, k = x.shape
+    product_calls["library"] += 1
     call("ms_gemm_library", _ptr(x), _ptr(weight), _ptr(out), m, weight.shape[0], k, int(out.dtype == torch.float32),
          int(accumulate), _ptr(workspace), _GEMM_WORKSPACE_BYTES, _stream())
 
 
-def _use_skinny(m: int, n: int, k: int, epilogue: int) -> bool:
-    return m <= SKINNY_MAX_ROWS and bool(load().ms_gemm_skinny_supported(m, n, k, epilogue))
+# Which of the two products serves a call that both can serve is a fixed rule of the
+# shape, so that the same model gives the same logits in every run and in recorded and
+# eager steps alike.  The rule is fitted to timings on MI355X of both products inside
+# recorded graphs over matrices that no cache holds (as a decode step meets its
+# weights), for the matrices of the 0.6B, 8B and 32B sizes and 1 to 64 rows: this
+# library's product streams a small matrix faster, the more so the fewer the rows;
+# hipBLASLt streams a large one faster unless its rows are very long; the fused forms
+# (norm as prologue, activation as epilogue) save one or two kernels of some 5 us each.
+_MIB = 1 << 20
+product_calls = {"skinny": 0, "library": 0}     # calls served by each since the import
+_forced_product: str | None = None
 
 
-# (device, blocks of 16 rows, n, k, gated) -> whether this library's product served a
-# timed call faster than hipBLASLt did (for ``gated``: than hipBLASLt and the activation kernel)
-_product_choice: dict[tuple[int, int, int, int, bool], bool] = {}
-_COLD_BYTES = 768 << 20
+@contextlib.contextmanager
+def forced_product(which: str | None):
+    """Inside the block every product that both kernels can serve goes to ``which``
+    (``"skinny"``: this library's, up to ``SKINNY_KERNEL_ROWS`` rows; ``"library"``:
+    hipBLASLt, and nothing is fused into a product) instead of following the rule.
+    For tests and measurements."""
 
-
-def _recorded_us(function, calls: int, replays: int = 4) -> float:
-    """Microseconds of one of ``function(0) .. function(calls - 1)`` inside a recorded
-    graph: what the call costs the GPU where few rows are at home, in recorded decode
-    steps, without the host's share of a launch.  No collection of cycles while the
-    stream records (a free inside a recording aborts the process)."""
-
-    function(0)                     # plans and workspaces exist before the recording
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    collecting = gc.isenabled()
-    gc.disable()
+    global _forced_product
+    if which not in (None, "skinny", "library"):
+        raise ValueError("forced_product takes 'skinny', 'library' or None.")
+    previous, _forced_product = _forced_product, which
     try:
-        with torch.cuda.graph(graph):
-            for index in range(calls):
-                function(index)
+        yield
     finally:
-        if collecting:
-            gc.enable()
-    graph.replay()
-    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    begin.record()
-    for _ in range(replays):
-        graph.replay()
-    end.record()
-    end.synchronize()
-    return 1000.0 * begin.elapsed_time(end) / (replays * calls)
+        _forced_product = previous
+
+
+def prefers_skinny(m: int, n: int, k: int, *, fused: bool = False) -> bool:
+    """The rule: whether this library's product is taken for ``x [m, k] @ w [n, k]^T``
+    (``fused``: with a norm or an activation that would otherwise be kernels of their own)."""
+
+    if m > SKINNY_KERNEL_ROWS:
+        return False
+    if _forced_product is not None:
+        return _forced_product == "skinny"
+    size = 2 * n * k
+    if size <= 16 * _MIB:                       # the matrices of a small model
+        return m <= (64 if n >= 2048 else 32)
+    if m > SKINNY_MAX_ROWS:
+        return False
+    if size <= 40 * _MIB or k >= 16384:         # middle sizes; very long rows, which the library splits badly
+        return True
+    if n >= 65536:                              # a head: many short rows
+        return m <= 8
+    return fused and size <= 256 * _MIB
 
 
 def _skinny_is_faster(x: torch.Tensor, weight: torch.Tensor, gated: bool) -> bool:
-    """For up to ``SKINNY_KERNEL_ROWS`` rows: whether this library's product is the
-    faster one for this shape.  Both are timed at the first call for a shape, as
-    recorded graphs over copies of the matrix, on outputs of their own; while a stream
-    records nothing is timed and nothing is remembered, and the call is served as it
-    was before there was a choice (this library's product up to ``SKINNY_MAX_ROWS``
-    rows)."""
-
     m, k = x.shape
     n = weight.shape[0]
     epilogue = _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16
     if m > SKINNY_KERNEL_ROWS or not load().ms_gemm_skinny_supported(m, n, k, epilogue):
         return False
-    if m <= SKINNY_MAX_ROWS and (gated or weight.numel() * weight.element_size() < SKINNY_ALWAYS_BYTES):
-        return True
-    index = x.device.index if x.device.index is not None else torch.cuda.current_device()
-    key = (index, -(-m // 16), n, k, gated)
-    choice = _product_choice.get(key)
-    if choice is None:
-        if torch.cuda.is_current_stream_capturing():
-            return m <= SKINNY_MAX_ROWS
-        # As in a decode step, every call streams a matrix that no cache holds: copies
-        # of the matrix, more of them than the card's last-level cache takes.
-        calls = min(128, max(2, -(-_COLD_BYTES // (weight.numel() * weight.element_size()))))
-        try:
-            matrices = [weight] + [weight.clone() for _ in range(calls - 1)]
-            ours = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=x.device)
-            theirs = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-        except torch.OutOfMemoryError:
-            return m <= SKINNY_MAX_ROWS
-
-        def library(index: int) -> None:
-            _library_product(x, matrices[index], theirs, False)
-            if gated:
-                silu_mul(theirs)
-
-        choice = _recorded_us(lambda index: _skinny(x, matrices[index], epilogue, ours), calls) < _recorded_us(library, calls)
-        _product_choice[key] = choice
-    return choice
+    return prefers_skinny(m, n, k, fused=gated)
 
 
 def _skinny(x: torch.Tensor, weight: torch.Tensor, epilogue: int, out: torch.Tensor) -> None:
@@ -444,6 +421,7 @@ def _skinny(x: torch.Tensor, weight: torch.Tensor, epilogue: int, out: torch.Ten
     n = weight.shape[0]
     bf16_out = out if out.dtype == torch.bfloat16 else None
     f32_out = out if out.dtype == torch.float32 else None
+    product_calls["skinny"] += 1
     call("ms_gemm_skinny", _ptr(x), _ptr(weight), _ptr(bf16_out), _ptr(f32_out), m, n, k, epilogue, _stream())
 
 
@@ -457,11 +435,10 @@ def linear(
     """``x [M, K] @ weight [N, K]^T``.
 
     float32: this library's FMA kernel (true 32-bit; row results do not depend on
-    M).  bfloat16 with at most ``SKINNY_MAX_ROWS`` rows: this library's matrix-core
-    kernel that streams the weights once; more rows: the library matrix product
-    (hipBLASLt, the copy that torch has loaded); up to ``SKINNY_KERNEL_ROWS`` rows the
-    one of the two that was faster when the shape was first seen.  All with 32-bit
-    accumulation.  ``accumulate_into`` (float32
+    M).  bfloat16: this library's matrix-core kernel that streams the weights once, or
+    the library matrix product (hipBLASLt, the copy that torch has loaded), by the
+    fixed rule of :func:`prefers_skinny`; beyond ``SKINNY_KERNEL_ROWS`` rows always
+    the latter.  All with 32-bit accumulation.  ``accumulate_into`` (float32
     ``[M, N]``) receives ``+=`` and is returned; ``out_float32`` returns the
     32-bit sums without a rounding to bfloat16 in between."""
 
@@ -505,7 +482,12 @@ def can_fuse_norm(rows: int, weight: torch.Tensor, *, gated: bool = False) -> bo
 
     n, k = weight.shape
     epilogue = _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16
-    return weight.dtype == torch.bfloat16 and _use_skinny(rows, n, k, epilogue)
+    return (
+        weight.dtype == torch.bfloat16
+        and rows <= SKINNY_MAX_ROWS
+        and bool(load().ms_gemm_skinny_supported(rows, n, k, epilogue))
+        and prefers_skinny(rows, n, k, fused=True)
+    )
 
 
 def linear_normed(
@@ -525,6 +507,7 @@ def linear_normed(
     if not can_fuse_norm(m, weight, gated=gated):
         raise KernelError("linear_normed: this shape is not served by the fused kernel.")
     out = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=residual.device)
+    product_calls["skinny"] += 1
     call("ms_gemm_skinny_normed", _ptr(residual), _ptr(norm_weight), float(eps), _ptr(weight), _ptr(out), m, n, k,
          _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16, _stream())
     return out

@@ -144,7 +144,7 @@ def decoder_layer(h, weights, index, config, positions, shared_kv=None, window=N
 
 def forward_logits(
     weights: dict, config: dict, token_ids, *, dtype: torch.dtype = torch.float64,
-    order=None, windows=None, first_position: int = 0, rd=None,
+    order=None, windows=None, first_position: int = 0, rd=None, rows=None,
 ) -> torch.Tensor:
     """Logits ``[T, V]`` for one whole sequence: embed, layers, final norm, head
     (reference: miniserve/model/qwen3.py:436-448, 547-558).  The head is the
@@ -152,7 +152,8 @@ def forward_logits(
 
     ``order``: list of ``(layer, cache_from)`` (default: every layer once);
     ``windows``: per call, a window or None; ``first_position``: absolute position
-    of the first token (for the shift invariant)."""
+    of the first token (for the shift invariant); ``rows``: the positions whose
+    logits are returned (default: all), for vocabularies too large to keep whole."""
 
     weights = {name: tensor.to(dtype) for name, tensor in weights.items()}
     tokens = torch.as_tensor(token_ids, dtype=torch.long)
@@ -166,6 +167,8 @@ def forward_logits(
         shared = None if cache_from is None else kept[cache_from]
         h, kv = decoder_layer(h, weights, layer, config, positions, shared, window, rd)
         kept.append(kv)
+    if rows is not None:
+        h = h[torch.as_tensor(rows, dtype=torch.long)]
     h = rms_norm(h, weights["model.norm.weight"], config["rms_norm_eps"], rd)
     head = weights["model.embed_tokens.weight"] if config.get("tie_word_embeddings") else weights["lm_head.weight"]
     return _r(h @ head.T, rd)

@@ -530,7 +530,7 @@ def test_skinny_product_for_few_rows(ops, m, n, k, monkeypatch):
     epilogues, against float64; sizes off the tile grid in every dimension."""
 
     assert ops.load().ms_gemm_skinny_supported(m, n, k, 0)
-    monkeypatch.setattr(ops, "SKINNY_MAX_ROWS", 64)                        # the kernel itself, beyond the rows it serves
+    monkeypatch.setattr(ops, "_forced_product", "skinny")                  # the kernel itself, whatever the rule says
     x = rand(m, k, seed=m + k, dtype=torch.bfloat16)
     w = rand(n, k, seed=n, dtype=torch.bfloat16, scale=0.05)
     exact = x.cpu().double() @ w.cpu().double().T
@@ -564,48 +564,43 @@ def test_product_beyond_64_rows_uses_the_library(ops):
     torch.testing.assert_close(ops.linear_silu_mul(x, w[:32].contiguous()), ops.silu_mul(ops.linear(x, w[:32].contiguous())))
 
 
-@pytest.mark.parametrize("m,n,k", [(17, 512, 96), (40, 1024, 1024), (64, 300, 200), (8, 8192, 2048)])
-def test_the_faster_of_the_two_products_is_taken(ops, m, n, k, monkeypatch):
-    """From 17 rows on, and for a large matrix with fewer: the first call for a shape
-    times both products and remembers which was faster; either one gives the product,
-    plain and with the gated activation; a call while a stream records times nothing
-    and remembers nothing."""
+@pytest.mark.parametrize("m,n,k", [(17, 512, 96), (40, 1024, 1024), (64, 300, 200), (8, 8192, 2048), (33, 4096, 1024)])
+def test_either_product_serves_a_shape_that_both_take(ops, m, n, k):
+    """Which product serves a shape is a fixed rule; forced to either one, the call
+    gives the product, plain, in 32-bit, added into a 32-bit tensor and with the gated
+    activation, eagerly and inside a recording alike."""
 
-    monkeypatch.setattr(ops, "_product_choice", {})
     x, w = rand(m, k, seed=m, dtype=torch.bfloat16), rand(n, k, seed=n, dtype=torch.bfloat16, scale=0.1)
     exact = x.cpu().double() @ w.cpu().double().T
     scale = float(exact.abs().max())
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        recorded = ops.linear(x, w)
-    assert ops._product_choice == {}
-    graph.replay()
-    torch.cuda.synchronize()
-    torch.testing.assert_close(recorded.cpu().double(), exact, atol=scale * 2**-8, rtol=2**-7)
-
-    first = ops.linear(x, w)
-    gated_first = ops.linear_silu_mul(x, w)
-    keys = sorted(ops._product_choice)
-    # (up to 16 rows the product with the activation in its epilogue is always this library's)
-    assert [key[1:] for key in keys] == [(-(-m // 16), n, k, False)] + ([(-(-m // 16), n, k, True)] if m > 16 else [])
-    results, gated = [], []
-    for choice in (True, False):
-        for key in keys:
-            ops._product_choice[key] = choice
-        results.append(ops.linear(x, w))
-        gated.append(ops.linear_silu_mul(x, w))
-        torch.testing.assert_close(results[-1].cpu().double(), exact, atol=scale * 2**-8, rtol=2**-7)
-        wide = ops.linear(x, w, out_float32=True)
-        torch.testing.assert_close(wide.cpu().double(), exact, atol=scale * 1e-5, rtol=1e-5)
-        total = torch.ones(m, n, device=DEVICE)
-        ops.linear(x, w, accumulate_into=total)
-        torch.testing.assert_close(total.cpu().double(), 1 + exact, atol=scale * 1e-5, rtol=1e-5)
-    assert any(torch.equal(first, result) for result in results)
-    assert any(torch.equal(gated_first, result) for result in gated)
-    # the activation of the rounded product, whichever kernel made it
-    assert torch.equal(gated[0], ops.silu_mul(results[0]))
-    assert torch.equal(gated[1], ops.silu_mul(results[1] if m > 16 else results[0]))
+    by_rule = ops.linear(x, w)
+    results = {}
+    for which in ("skinny", "library"):
+        with ops.forced_product(which):
+            before = dict(ops.product_calls)
+            results[which] = ops.linear(x, w)
+            assert ops.product_calls[which] == before[which] + 1
+            assert ops.prefers_skinny(m, n, k) == (which == "skinny")
+            assert ops.can_fuse_norm(min(m, 16), w) == (which == "skinny")
+            gated = ops.linear_silu_mul(x, w)
+            assert torch.equal(gated, ops.silu_mul(results[which]))          # the activation of the rounded product
+            torch.testing.assert_close(results[which].cpu().double(), exact, atol=scale * 2**-8, rtol=2**-7)
+            wide = ops.linear(x, w, out_float32=True)
+            torch.testing.assert_close(wide.cpu().double(), exact, atol=scale * 1e-5, rtol=1e-5)
+            total = torch.ones(m, n, device=DEVICE)
+            ops.linear(x, w, accumulate_into=total)
+            torch.testing.assert_close(total.cpu().double(), 1 + exact, atol=scale * 1e-5, rtol=1e-5)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                recorded = ops.linear(x, w)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(recorded, results[which])                    # a recording takes the same kernel
+    assert torch.equal(by_rule, results["skinny" if ops.prefers_skinny(m, n, k) else "library"])
+    with pytest.raises(ValueError):
+        with ops.forced_product("other"):
+            pass
 
 
 @pytest.mark.parametrize("m,n,k", [(17, 509, 96), (65, 33, 60), (300, 1024, 200), (2048, 4096, 1024), (129, 300, 80)])
@@ -614,7 +609,7 @@ def test_library_product_for_many_rows(ops, m, n, k, monkeypatch):
     bfloat16 out, 32-bit out, and += into a 32-bit tensor; sizes off every grid; the
     same shape again takes the kept plan."""
 
-    monkeypatch.setattr(ops, "SKINNY_KERNEL_ROWS", 16)       # no choice between the two products here
+    monkeypatch.setattr(ops, "_forced_product", "library")   # no choice between the two products here
     x, w = rand(m, k, seed=m, dtype=torch.bfloat16), rand(n, k, seed=n, dtype=torch.bfloat16, scale=0.1)
     exact = x.cpu().double() @ w.cpu().double().T
     scale = float(exact.abs().max())
@@ -640,7 +635,7 @@ def test_library_product_inside_a_recorded_graph(ops, monkeypatch, m, n, k):
     what the eager call gives for the inputs of that moment: plain, and added into a
     32-bit tensor (the shapes of a decode step of 33 to 64 rows among them)."""
 
-    monkeypatch.setattr(ops, "SKINNY_KERNEL_ROWS", 16)
+    monkeypatch.setattr(ops, "_forced_product", "library")
     x = rand(m, k, seed=1, dtype=torch.bfloat16)
     w = rand(n, k, seed=2, dtype=torch.bfloat16, scale=0.1)
     base = rand(m, n, seed=3)
