@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kThreads) MS_WAVES_PER_EU(D <= 128 ? 2 : 1, 2) void
   __shared__ float l_s[kWaves][16];
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = ms::uniform(threadIdx.x >> 6);   // the same in all lanes: tile numbers and table entries are scalar work
   const int g = lane >> 4;
   const int r = lane & 15;
 

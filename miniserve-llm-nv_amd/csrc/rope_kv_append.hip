@@ -39,45 +39,61 @@ __global__ void qk_norm_rope_append_kernel(const T* __restrict__ packed, const T
   const bool is_k = !is_q && head < num_q_heads + num_kv_heads;
   const int kv_head = is_q ? 0 : (is_k ? head - num_q_heads : head - num_q_heads - num_kv_heads);
 
-  T* dst;
-  int64_t dst_stride = 1;   // distance between consecutive d
-  if (is_q) {
-    dst = q_out + (token * num_q_heads + head) * head_dim;
-  } else {
-    const int64_t slot = slot_mapping[token];
-    const int64_t page = slot / block_size;
-    const int64_t offset = slot - page * block_size;
-    if (is_k) {
-      dst = key_pool + ((page * num_kv_heads + kv_head) * block_size + offset) * head_dim;
-    } else {
-      dst = value_pool + (page * num_kv_heads + kv_head) * head_dim * block_size + offset;
-      dst_stride = block_size;
-    }
-  }
-
   // Everything the row needs is asked for at once (the row, the norm's weight, the
   // angles): one round trip to memory, not three behind one another.
   const T* weight = is_q ? q_weight : (is_k ? k_weight : nullptr);
   const bool rotate = cos_table != nullptr && (is_q || is_k);
-  float lo[kMaxPairsPerLane], hi[kMaxPairsPerLane];
-  float w_lo[kMaxPairsPerLane], w_hi[kMaxPairsPerLane], cs[kMaxPairsPerLane], sn[kMaxPairsPerLane];
+  // The loads leave their values untouched (a value that is used behind a branch is
+  // waited for behind that branch, before the next load goes out); they are turned
+  // into floats when all are on their way.
+  T raw_lo[kMaxPairsPerLane], raw_hi[kMaxPairsPerLane], raw_w_lo[kMaxPairsPerLane], raw_w_hi[kMaxPairsPerLane];
+  float cs[kMaxPairsPerLane], sn[kMaxPairsPerLane];
 #pragma unroll
   for (int c = 0; c < kMaxPairsPerLane; ++c) {
-    const int i = lane + c * ms::kWave;
-    lo[c] = hi[c] = 0.f;
-    w_lo[c] = w_hi[c] = cs[c] = 1.f;
-    sn[c] = 0.f;
-    if (i < half) {
-      lo[c] = ms::to_float(row[i]);
-      hi[c] = ms::to_float(row[i + half]);
+    const int i = min(lane + c * ms::kWave, half - 1);      // lanes past the end read the last pair and store nothing
+    if (c * ms::kWave < half) {
+      raw_lo[c] = row[i];
+      raw_hi[c] = row[i + half];
       if (weight) {
-        w_lo[c] = ms::to_float(weight[i]);
-        w_hi[c] = ms::to_float(weight[i + half]);
+        raw_w_lo[c] = weight[i];
+        raw_w_hi[c] = weight[i + half];
       }
       if (rotate) {
         cs[c] = cos_table[token * half + i];
         sn[c] = sin_table[token * half + i];
       }
+    }
+  }
+  const int slot = is_q ? 0 : slot_mapping[token];      // asked for behind the row's loads, not ahead of them
+  float lo[kMaxPairsPerLane], hi[kMaxPairsPerLane], w_lo[kMaxPairsPerLane], w_hi[kMaxPairsPerLane];
+#pragma unroll
+  for (int c = 0; c < kMaxPairsPerLane; ++c) {
+    const bool live = lane + c * ms::kWave < half;
+    const bool loaded = c * ms::kWave < half;
+    lo[c] = live ? ms::to_float(raw_lo[c]) : 0.f;
+    hi[c] = live ? ms::to_float(raw_hi[c]) : 0.f;
+    w_lo[c] = (loaded && weight) ? ms::to_float(raw_w_lo[c]) : 1.f;
+    w_hi[c] = (loaded && weight) ? ms::to_float(raw_w_hi[c]) : 1.f;
+    if (!(loaded && rotate)) {
+      cs[c] = 1.f;
+      sn[c] = 0.f;
+    }
+  }
+
+  // Where the row goes.  The slot is asked for with the row; the address is made from
+  // it only here, so that the wait for it is the wait for the row.
+  T* dst;
+  int64_t dst_stride = 1;   // distance between consecutive d
+  if (is_q) {
+    dst = q_out + (token * num_q_heads + head) * head_dim;
+  } else {
+    const int page = slot / block_size;           // 32-bit: a slot number is below 2^31
+    const int offset = slot - page * block_size;
+    if (is_k) {
+      dst = key_pool + ((static_cast<int64_t>(page) * num_kv_heads + kv_head) * block_size + offset) * head_dim;
+    } else {
+      dst = value_pool + (static_cast<int64_t>(page) * num_kv_heads + kv_head) * head_dim * block_size + offset;
+      dst_stride = block_size;
     }
   }
 
