@@ -2,10 +2,11 @@
 group, and numbered slots for per-request state of fixed size.
 
 A step is a transaction, as in the reference (miniserve/kv/manager.py:119-192,
-kv/paged.py:59-104): ``prepare_step`` reserves the missing pages tentatively and
-computes the slot of every new token, ``commit_step`` makes them part of the
-tables and advances the committed lengths, ``abort_step`` gives exactly the
-step's new pages back.  Beyond the reference: groups of calls with different
+kv/paged.py:59-104): ``prepare_step`` reserves the missing pages tentatively,
+computes the slot of every new token and keeps a copy of the requests' state rows,
+``commit_step`` makes the pages part of the tables and advances the committed
+lengths, ``abort_step`` gives exactly the step's new pages back and restores the
+state.  Beyond the reference: groups of calls with different
 needs have pools, allocators and tables of their own; a group with a window gives
 pages back as soon as no later position can read them; every live request holds a
 numbered state slot.
@@ -72,6 +73,8 @@ class StepReservation:
     step_id: int
     sequences: list[SequenceStepMeta] = field(default_factory=list)
     closed: bool = False
+    # per state tensor: (slot indices on the device, the rows as they were before the step)
+    state_before: list = field(default_factory=list)
 
 
 @dataclass
@@ -270,10 +273,32 @@ class CacheManager:
         for item in items:
             self._live[item.request_id].pending = True
         self._open = reservation
+        self._keep_state(reservation)
         return reservation
+
+    def _keep_state(self, reservation: StepReservation) -> None:
+        """Per-request state is part of the transaction: the rows of the step's
+        requests are copied before the step may write them (one small gather per state
+        tensor, in stream order behind the step before), so that an aborted step, or
+        the eager run before a recording, can be undone.  A model without state copies nothing."""
+
+        if not self.state_tensors or not reservation.sequences:
+            return
+        import torch
+
+        slots = torch.tensor([meta.state_slot for meta in reservation.sequences], dtype=torch.long,
+                             device=self.state_tensors[0].device)
+        reservation.state_before = [(slots, tensor.index_select(0, slots)) for tensor in self.state_tensors]
+
+    def restore_state(self, reservation: StepReservation) -> None:
+        """Puts the state of the step's requests back to what it was at ``prepare_step``."""
+
+        for tensor, (slots, rows) in zip(self.state_tensors, reservation.state_before):
+            tensor.index_copy_(0, slots, rows)
 
     def commit_step(self, reservation: StepReservation) -> None:
         self._close(reservation)
+        reservation.state_before = []
         for meta in reservation.sequences:
             live = self._live[meta.request_id]
             for group, table, pages in zip(self.layout.groups, live.tables, meta.new_pages):
@@ -283,7 +308,13 @@ class CacheManager:
             self._give_back_passed_pages(live)
 
     def abort_step(self, reservation: StepReservation) -> None:
+        """Gives exactly the step's new pages back and restores the state of its
+        requests; keys and values that the step wrote lie above the committed lengths
+        and are never read."""
+
         self._close(reservation)
+        self.restore_state(reservation)
+        reservation.state_before = []
         for meta in reservation.sequences:
             for allocator, pages in zip(self.allocators, meta.new_pages):
                 if pages:

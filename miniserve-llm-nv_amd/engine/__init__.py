@@ -1,4 +1,4 @@
-from .batch import StepEntry, build_step_context
+from .batch import StepEntry, build_step
 from .engine import Engine, GenerationResult, StepOutput
 from .plan import DecodeItem, ExecutionPlan, PrefillItem
 from .request import Request, SamplingParams
@@ -21,5 +21,5 @@ __all__ = [
     "SequenceView",
     "StepEntry",
     "StepOutput",
-    "build_step_context",
+    "build_step",
 ]

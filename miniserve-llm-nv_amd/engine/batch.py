@@ -10,16 +10,13 @@ is cheap and stops an allocator fault before a kernel can scribble.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Sequence
+from typing import Callable, Mapping, Sequence
 
 import numpy as np
 import torch
 
 from ..cache.manager import StepReservation
-from ..parts.base import GroupStepView, QueryTiles, StepContext
-
-
-QUERY_TILE = 64     # tokens of one sequence that one workgroup of the tiled attention kernel serves
+from ..parts.base import GroupStepView, HostBatch, StepContext
 
 
 @dataclass(frozen=True)
@@ -75,24 +72,6 @@ class BuiltStep:
         self._sent = True
 
 
-def build_step_context(
-    entries: Sequence[StepEntry],
-    reservation: StepReservation,
-    *,
-    block_size: int,
-    pool_pages: Sequence[int],
-    vocab_size: int,
-    device: torch.device | str,
-) -> tuple[StepContext, torch.Tensor | None]:
-    """The step's tensors, sent: see :func:`build_step`."""
-
-    built = build_step(
-        entries, reservation, block_size=block_size, pool_pages=pool_pages, vocab_size=vocab_size, device=device
-    )
-    built.send()
-    return built.ctx, built.rows
-
-
 def build_step(
     entries: Sequence[StepEntry],
     reservation: StepReservation,
@@ -101,10 +80,13 @@ def build_step(
     pool_pages: Sequence[int],
     vocab_size: int,
     device: torch.device | str,
+    step_tables: Callable[[HostBatch], Mapping[str, Sequence[int]]] | None = None,
 ) -> BuiltStep:
     """All integer metadata of the step is packed into one host buffer that goes to
     the device in one copy (:meth:`BuiltStep.send`); the context's tensors are views
-    of the device buffer."""
+    of the device buffer.  ``step_tables``: the model's hook that makes the integer
+    tables its parts want for this batch (tile lists of a kernel, say); they are
+    packed into the same buffer and handed to the parts as ``ctx.tables``."""
 
     if len(entries) != len(reservation.sequences):
         raise ValueError("entries and reservation disagree.")
@@ -117,15 +99,26 @@ def build_step(
     s = len(entries)
     query_lens = [len(entries[original].token_ids) for original in layout]
     n = sum(query_lens)
-    num_tiles = sum(-(-length // QUERY_TILE) for length in query_lens[decode_prefix:])
+    query_start = [0] * (s + 1)
+    for index, length in enumerate(query_lens):
+        query_start[index + 1] = query_start[index] + length
+    first_positions = [meta.before for meta in metas_in_layout]
+    part_tables: dict[str, np.ndarray] = {}
+    if step_tables is not None:
+        host_batch = HostBatch(tuple(query_lens), tuple(query_start), tuple(first_positions), decode_prefix)
+        for name, values in step_tables(host_batch).items():
+            part_tables[name] = np.asarray(values, dtype=np.int64)
+            if part_tables[name].ndim != 1 or (part_tables[name].size and (
+                    part_tables[name].min() < -(2**31) or part_tables[name].max() >= 2**31)):
+                raise ValueError(f"step table {name!r} must be a list of 32-bit integers.")
     num_rows = sum(len(entry.want) for entry in entries)
     widest = [max(1, max(len(meta.block_tables[group]) for meta in metas_in_layout)) for group in range(num_groups)]
 
     offsets: dict[str, tuple[int, int]] = {}
     total = 0
     sizes = [("token_ids", n), ("positions", n), ("seq_of_token", n), ("query_start", s + 1), ("context_lens", s),
-             ("state_slots", s), ("logit_rows", num_rows), ("tile_seq", num_tiles), ("tile_token", num_tiles),
-             ("tile_length", num_tiles)]
+             ("state_slots", s), ("logit_rows", num_rows)]
+    sizes += [(f"part:{name}", values.size) for name, values in part_tables.items()]
     for group in range(num_groups):
         sizes += [(f"slots{group}", n), (f"table{group}", s * widest[group])]
     for name, size in sizes:
@@ -146,12 +139,7 @@ def build_step(
         table_region[:] = 0
     context_lens = [meta.after for meta in metas_in_layout]
     state_slots = [meta.state_slot for meta in metas_in_layout]
-    first_positions = [meta.before for meta in metas_in_layout]
-    query_start = [0] * (s + 1)
     base_of_entry = [0] * s
-    tile_seq: list[int] = []
-    tile_token: list[int] = []
-    tile_length: list[int] = []
 
     for index, original in enumerate(layout):
         entry, meta = entries[original], metas_in_layout[index]
@@ -159,7 +147,6 @@ def build_step(
         if entry.request_id != meta.request_id or length != meta.after - meta.before:
             raise ValueError(f"entry {entry.request_id!r} does not match its reservation.")
         base = query_start[index]
-        query_start[index + 1] = base + length
         base_of_entry[original] = base
         if length == 1:
             # one token: plain integers (an array per row would cost more than it saves)
@@ -188,10 +175,6 @@ def build_step(
         run = np.arange(meta.before, meta.after, dtype=np.int64)
         positions[base : base + length] = run
         seq_of_token[base : base + length] = index
-        for start in range(0, length, QUERY_TILE):
-            tile_seq.append(index)
-            tile_token.append(base + start)
-            tile_length.append(min(QUERY_TILE, length - start))
         logical, offset = np.divmod(run, block_size)
         for group in range(num_groups):
             table = np.asarray(meta.block_tables[group], dtype=np.int64)
@@ -215,9 +198,8 @@ def build_step(
     region("context_lens")[:] = context_lens
     region("state_slots")[:] = state_slots
     region("logit_rows")[:] = logit_rows
-    region("tile_seq")[:] = tile_seq
-    region("tile_token")[:] = tile_token
-    region("tile_length")[:] = tile_length
+    for name, values in part_tables.items():
+        region(f"part:{name}")[:] = values
     buffer = torch.empty(total, dtype=torch.int32, device=device) if on_gpu else host
 
     def view(name: str) -> torch.Tensor:
@@ -244,7 +226,7 @@ def build_step(
         state_slots_host=state_slots,
         first_positions_host=first_positions,
         decode_prefix=decode_prefix,
-        tiles=QueryTiles(len(tile_seq), view("tile_seq"), view("tile_token"), view("tile_length")) if tile_seq else None,
+        tables={name: view(f"part:{name}") for name in part_tables},
     )
     rows = view("logit_rows") if logit_rows else None
     token_start = offsets["token_ids"][0]

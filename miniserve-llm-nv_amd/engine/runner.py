@@ -98,13 +98,16 @@ class DecodeGraph:
                 GroupStepView(block_table=view(f"table{g}").view(batch, width), slot_mapping=view(f"slots{g}"))
                 for g in range(groups)
             ],
+            # what holds for every replay: one token a row.  Launch decisions inside the
+            # graph go by the bound; per-request numbers live on the device only.
             query_lens=[1] * batch,
-            # launch decisions inside the graph must hold for every later step
-            context_lens_host=[runner.max_model_len] * batch,
             query_start_host=list(range(batch + 1)),
-            state_slots_host=[0] * batch,
-            first_positions_host=[0] * batch,
+            context_lens_host=None,
+            state_slots_host=None,
+            first_positions_host=None,
             decode_prefix=batch,
+            recorded=True,
+            context_bound=runner.max_model_len,
         )
         self.rows = view("logit_rows")
         # the table object that each row of the host buffer was last filled from: a request's
@@ -190,9 +193,11 @@ class DecodeGraph:
         runner = self._runner()
         model, views = runner.model, runner._call_views
         if self.graph is None:
-            # Once eagerly, so that libraries set themselves up outside the recording;
-            # running the same step twice writes the same cache slots twice.
+            # Once eagerly, so that libraries set themselves up outside the recording.  The
+            # replay below runs the same step again: cache slots are written twice with the
+            # same values, and per-request state is put back to what it was before the step.
             model.forward(self.ctx, views, self.rows)
+            runner.cache.restore_state(reservation)
             torch.cuda.synchronize(runner.device)
             self.ctx.scratch.clear()        # what the step shares between layers is made again inside the recording
             graph = torch.cuda.CUDAGraph()
@@ -397,7 +402,7 @@ class ModelRunner:
             try:
                 built = build_step(
                     entries, reservation, block_size=self.block_size, pool_pages=self.cache.num_blocks,
-                    vocab_size=self.spec.vocab_size, device=self.device,
+                    vocab_size=self.spec.vocab_size, device=self.device, step_tables=self.model.step_tables,
                 )
             except BaseException:
                 self.cache.abort_step(reservation)
@@ -464,6 +469,7 @@ class ModelRunner:
                 pool_pages=self.cache.num_blocks,
                 vocab_size=self.spec.vocab_size,
                 device=self.device,
+                step_tables=self.model.step_tables,
             )
             built.send()
             logits = self.model.forward(built.ctx, self._call_views, built.rows)

@@ -7,6 +7,8 @@ torch is the allocator and gives the stream.
 from __future__ import annotations
 
 import contextlib
+import dataclasses
+import warnings
 
 import torch
 
@@ -14,7 +16,14 @@ from .library import KernelError, call, library_path, load
 
 __all__ = [
     "KernelError",
+    "PREFILL_TILE_TOKENS",
+    "QueryTiles",
     "attention",
+    "attention_calls",
+    "forced_product",
+    "prefers_skinny",
+    "product_calls",
+    "query_tiles_host",
     "embedding_gather",
     "library_path",
     "linear",
@@ -213,6 +222,58 @@ def _value_pool_shape(key_pool: torch.Tensor) -> tuple[int, ...]:
     return (pages, kv_heads, head_dim, block_size)
 
 
+# Tokens of one sequence that one workgroup of the tiled attention kernel serves.
+PREFILL_TILE_TOKENS = 64
+
+
+@dataclasses.dataclass
+class QueryTiles:
+    """The tokens after the single-token prefix of a batch, cut into tiles of at most
+    ``PREFILL_TILE_TOKENS`` consecutive tokens of one sequence (what the tiled
+    attention kernel walks)."""
+
+    count: int
+    seq: torch.Tensor       # int32 [count]: the tile's sequence (row of the block tables)
+    token: torch.Tensor     # int32 [count]: index of the tile's first token in the batch
+    length: torch.Tensor    # int32 [count]: 1..PREFILL_TILE_TOKENS
+
+
+def query_tiles_host(query_lens, query_start, decode_prefix: int) -> tuple[list[int], list[int], list[int]]:
+    """The tiles of a batch as three lists (sequence, first token, length): every
+    sequence after the first ``decode_prefix`` is cut into runs of at most
+    ``PREFILL_TILE_TOKENS`` tokens."""
+
+    seqs: list[int] = []
+    tokens: list[int] = []
+    lengths: list[int] = []
+    for index in range(decode_prefix, len(query_lens)):
+        base, length = query_start[index], query_lens[index]
+        for start in range(0, length, PREFILL_TILE_TOKENS):
+            seqs.append(index)
+            tokens.append(base + start)
+            lengths.append(min(PREFILL_TILE_TOKENS, length - start))
+    return seqs, tokens, lengths
+
+
+# calls of attention() served by each kernel since the import; a bfloat16 call that no
+# matrix-core kernel takes is served by the generic one, many times slower, and is
+# reported once per geometry
+attention_calls = {"decode": 0, "prefill": 0, "generic": 0}
+_reported_fallbacks: set = set()
+
+
+def _report_fallback(head_dim: int, block_size: int, reason: str) -> None:
+    key = (head_dim, block_size, reason)
+    if key not in _reported_fallbacks:
+        _reported_fallbacks.add(key)
+        warnings.warn(
+            f"attention with head size {head_dim} and pages of {block_size} keys: {reason} "
+            "(correct, but far slower than the matrix-core kernels; they take head sizes in steps of 16 "
+            "up to 256 for single tokens, up to 128 for runs of tokens, and pages of a multiple of 16 keys).",
+            RuntimeWarning, stacklevel=3,
+        )
+
+
 # Workgroups that the key-split attention aims to launch: a few per compute unit
 # (the chip has 256), so that short batches still fill it.
 _DECODE_TARGET_WORKGROUPS = 512
@@ -293,7 +354,10 @@ def attention(
     if q.dtype == torch.bfloat16 and covered and lib.ms_attention_decode_supported(head_dim, block_size):
         tiled = lib.ms_attention_prefill_supported(head_dim, block_size)
         single = decode_prefix if tiled else n          # without the tiled kernel every token is served as a single one
+        if not tiled and decode_prefix < n:
+            _report_fallback(head_dim, block_size, "runs of tokens are served token by token by the single-token kernel")
         if single > 0:
+            attention_calls["decode"] += 1
             if splits is None:
                 splits = decode_splits(single, kv_heads, heads // kv_heads, max_context or max_blocks * block_size)
             partial_o = partial_ml = None
@@ -304,12 +368,16 @@ def attention(
                  _ptr(seq_of_token), _ptr(positions), _ptr(out), _ptr(partial_o), _ptr(partial_ml), single, heads,
                  kv_heads, head_dim, block_size, max_blocks, float(scale), window, int(splits), _stream())
         if tiled and decode_prefix < n:
+            attention_calls["prefill"] += 1
             for name in ("seq", "token", "length"):
                 _check(getattr(tiles, name), f"tiles.{name}", dtype=torch.int32, shape=(tiles.count,))
             call("ms_attention_prefill", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(positions),
                  _ptr(tiles.seq), _ptr(tiles.token), _ptr(tiles.length), _ptr(out), tiles.count, heads, kv_heads,
                  head_dim, block_size, max_blocks, float(scale), window, _stream())
         return out
+    attention_calls["generic"] += 1
+    if q.dtype == torch.bfloat16 and not lib.ms_attention_decode_supported(head_dim, block_size):
+        _report_fallback(head_dim, block_size, "no matrix-core kernel takes this geometry, the generic kernel serves it")
     call("ms_attention_generic", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(seq_of_token),
          _ptr(positions), _ptr(out), n, heads, kv_heads, head_dim, block_size, max_blocks, float(scale),
          window, _code(q.dtype), _stream())

@@ -15,6 +15,7 @@ import torch
 from .. import ops
 from ..config.model_spec import PartSpec
 from .base import (
+    HostBatch,
     KVCacheNeed,
     KVCacheView,
     Part,
@@ -82,6 +83,26 @@ class Attention(Part):
     def cache_need(self) -> KVCacheNeed:
         return KVCacheNeed(self.num_kv_heads, self.head_dim, self.window)
 
+    # The tiled attention kernel walks the runs of tokens of a step in tiles; the tile
+    # lists are made on the host once per step, for all attention layers, and travel to
+    # the device with the step's other numbers.
+    step_tables_key = "attention.tiles"
+
+    @staticmethod
+    def step_tables(batch: HostBatch) -> dict[str, list[int]]:
+        seqs, tokens, lengths = ops.query_tiles_host(batch.query_lens, batch.query_start, batch.decode_prefix)
+        return {"attention.tile_seq": seqs, "attention.tile_token": tokens, "attention.tile_length": lengths}
+
+    @staticmethod
+    def _tiles(ctx: StepContext):
+        if "attention.tiles" not in ctx.scratch:
+            seq = ctx.tables.get("attention.tile_seq")
+            tiles = None
+            if seq is not None and seq.numel() > 0:
+                tiles = ops.QueryTiles(seq.numel(), seq, ctx.tables["attention.tile_token"], ctx.tables["attention.tile_length"])
+            ctx.scratch["attention.tiles"] = tiles
+        return ctx.scratch["attention.tiles"]
+
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         """q, k and v rows are stacked into one matrix, q rows first, then k, then
         v, so one product gives the packed ``[N, (Hq + 2 Hkv) * D]`` row."""
@@ -138,7 +159,7 @@ class Attention(Part):
             scale=self.scale,
             window=self.window,
             decode_prefix=ctx.decode_prefix,
-            tiles=ctx.tiles,
+            tiles=self._tiles(ctx),
             max_context=ctx.max_context_len,
         )
         attended = attended.reshape(n, self.num_heads * self.head_dim)

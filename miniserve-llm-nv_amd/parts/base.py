@@ -41,8 +41,10 @@ CATEGORIES = ("norm", "position", "mixer", "feed_forward", "block", "embedding",
 class WeightSpec:
     """One checkpoint tensor that a part wants.
 
-    ``init`` picks the random-weights distribution: ``"matrix"`` ~ N(0, 0.02),
-    ``"norm"`` ~ 1 + N(0, 0.1), ``"zeros"``.  ``keep`` says how the tensor is
+    ``init`` picks the random-weights distribution: the name of a rule
+    (``"matrix"`` ~ N(0, 0.02), ``"norm"`` ~ 1 + N(0, 0.1), ``"zeros"``, or one added
+    with ``weights.register_init``) or a callable ``(shape, generator, device) ->
+    float32 tensor`` of the part's own.  ``keep`` says how the tensor is
     held: ``"compute"`` in the engine's dtype (bfloat16 or float32),
     ``"float32"`` always in 32-bit, ``"int32"`` an integer table.
     ``optional`` tensors may be absent; ``same_as`` names a tensor that an
@@ -50,7 +52,7 @@ class WeightSpec:
 
     name: str
     shape: tuple[int, ...]
-    init: str = "matrix"
+    init: str | Callable[..., torch.Tensor] = "matrix"
     keep: str = "compute"
     optional: bool = False
     same_as: str | None = None
@@ -105,15 +107,15 @@ class GroupStepView:
     slot_mapping: torch.Tensor   # int32 [N]: page * block_size + offset of each new token
 
 
-@dataclass
-class QueryTiles:
-    """The tokens after the single-token prefix of a batch, cut into tiles of at most
-    64 consecutive tokens of one sequence (what the tiled attention kernel walks)."""
+@dataclass(frozen=True)
+class HostBatch:
+    """What a part may know of a step on the host, before anything is sent: the
+    sequences in the order of the batch (those that bring one token first)."""
 
-    count: int
-    seq: torch.Tensor       # int32 [count]: the tile's sequence (row of the block tables)
-    token: torch.Tensor     # int32 [count]: index of the tile's first token in the batch
-    length: torch.Tensor    # int32 [count]: 1..64
+    query_lens: tuple[int, ...]         # tokens that each sequence brings
+    query_start: tuple[int, ...]        # index of each sequence's first token in the batch, and the total
+    first_positions: tuple[int, ...]    # absolute position of each sequence's first token
+    decode_prefix: int                  # sequences at the front that bring exactly one token
 
 
 @dataclass
@@ -121,7 +123,14 @@ class StepContext:
     """A flat ragged batch: ``N`` tokens of ``S`` sequences, each sequence's tokens
     contiguous and at consecutive absolute positions.  Sequences that bring one
     token come first (``decode_prefix`` of them), so that kernels made for single
-    tokens and kernels made for runs of tokens can each take their share."""
+    tokens and kernels made for runs of tokens can each take their share.
+
+    The host copies exist for launch decisions.  In a *recorded* step (``recorded``:
+    a graph that is replayed for many steps of single tokens) only what holds for
+    every replay is given: ``query_lens`` and ``query_start_host`` (one token each);
+    the other host copies are None, and ``max_context_len`` is the bound that no
+    request exceeds.  A part that needs per-request values there reads the device
+    tensors (``state_slots``, ``positions``, ``context_lens``)."""
 
     num_tokens: int
     num_seqs: int
@@ -134,12 +143,15 @@ class StepContext:
     groups: list[GroupStepView]
     # host copies, for launch decisions
     query_lens: list[int] = field(default_factory=list)
-    context_lens_host: list[int] = field(default_factory=list)
+    context_lens_host: list[int] | None = field(default_factory=list)
     query_start_host: list[int] = field(default_factory=list)
-    state_slots_host: list[int] = field(default_factory=list)
-    first_positions_host: list[int] = field(default_factory=list)
+    state_slots_host: list[int] | None = field(default_factory=list)
+    first_positions_host: list[int] | None = field(default_factory=list)
     decode_prefix: int = 0
-    tiles: QueryTiles | None = None
+    recorded: bool = False
+    context_bound: int | None = None      # recorded steps: the longest context any replay can have
+    # integer tables that parts asked for (``step_tables``), sent with the step's other numbers
+    tables: dict[str, torch.Tensor] = field(default_factory=dict)
     # what parts compute once per step and share between layers (position tables)
     scratch: dict = field(default_factory=dict)
 
@@ -149,6 +161,10 @@ class StepContext:
 
     @property
     def max_context_len(self) -> int:
+        if self.context_lens_host is None:
+            if self.context_bound is None:
+                raise RuntimeError("a recorded step has no per-request context lengths on the host.")
+            return self.context_bound
         return max(self.context_lens_host)
 
 

@@ -77,6 +77,30 @@ class DecoderModel:
             needs.append(CallCacheNeed(index, need, call.cache_from))
         return needs
 
+    def step_tables(self, batch) -> dict[str, list[int]]:
+        """Integer tables that parts want made on the host for this step (a
+        ``HostBatch``) and sent with its other numbers; they find them in
+        ``ctx.tables`` under the names they gave.  A mixer or feed-forward offers
+        ``step_tables(batch) -> {name: integers}`` and ``step_tables_key`` (parts with
+        the same key want the same tables: they are made once)."""
+
+        tables: dict[str, list[int]] = {}
+        seen: set = set()
+        for layer in self.layers:
+            for part in (getattr(layer, "mixer", None), getattr(layer, "feed_forward", None)):
+                provider = getattr(part, "step_tables", None)
+                if provider is None:
+                    continue
+                key = getattr(part, "step_tables_key", id(part))
+                if key in seen:
+                    continue
+                seen.add(key)
+                for name, values in provider(batch).items():
+                    if name in tables:
+                        raise ValueError(f"two parts name a step table {name!r}.")
+                    tables[name] = values
+        return tables
+
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         for part in self.parts():
             load_part_weights(part, tensors)

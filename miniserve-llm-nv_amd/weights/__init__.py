@@ -1,5 +1,5 @@
 from .loader import WeightLoadError, WeightLoadReport, load_weights, weight_files
-from .random_init import random_device_tensors, random_tensors, write_random_model
+from .random_init import random_device_tensors, random_tensors, register_init, write_random_model
 
 __all__ = [
     "WeightLoadError",
@@ -7,6 +7,7 @@ __all__ = [
     "load_weights",
     "random_device_tensors",
     "random_tensors",
+    "register_init",
     "weight_files",
     "write_random_model",
 ]

@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import json
 from pathlib import Path
-from typing import Sequence
+from typing import Callable, Sequence
 
 import torch
 
@@ -22,16 +22,34 @@ NORM_STD = 0.1
 STORE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
+# name -> rule(shape, generator, device) -> float32 tensor.  Parts name a rule in their
+# ``WeightSpec.init`` or bring a callable of the same form; ``register_init`` adds a name.
+InitRule = Callable[[tuple, torch.Generator, "torch.device | str"], torch.Tensor]
+_INIT_RULES: dict[str, InitRule] = {
+    "matrix": lambda shape, generator, device: torch.randn(shape, generator=generator, dtype=torch.float32, device=device) * MATRIX_STD,
+    "norm": lambda shape, generator, device: 1.0 + torch.randn(shape, generator=generator, dtype=torch.float32, device=device) * NORM_STD,
+    "zeros": lambda shape, generator, device: torch.zeros(shape, dtype=torch.float32, device=device),
+}
+
+
+def register_init(name: str, rule: InitRule) -> None:
+    """Adds a named rule for ``WeightSpec.init``."""
+
+    if not callable(rule):
+        raise TypeError("an init rule is a callable (shape, generator, device) -> float32 tensor.")
+    _INIT_RULES[name] = rule
+
+
 def draw_tensor(spec: WeightSpec, generator: torch.Generator, device: torch.device | str = "cpu") -> torch.Tensor:
     if spec.keep == "int32":
         return torch.zeros(spec.shape, dtype=torch.int32, device=device)
-    if spec.init == "matrix":
-        return torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device) * MATRIX_STD
-    if spec.init == "norm":
-        return 1.0 + torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device) * NORM_STD
-    if spec.init == "zeros":
-        return torch.zeros(spec.shape, dtype=torch.float32, device=device)
-    raise ValueError(f"{spec.name}: unknown init rule {spec.init!r}.")
+    rule = spec.init if callable(spec.init) else _INIT_RULES.get(spec.init)
+    if rule is None:
+        raise ValueError(f"{spec.name}: unknown init rule {spec.init!r} (known: {sorted(_INIT_RULES)}).")
+    tensor = rule(tuple(spec.shape), generator, device)
+    if tuple(tensor.shape) != tuple(spec.shape) or tensor.dtype != torch.float32:
+        raise ValueError(f"{spec.name}: its init rule must give a float32 tensor of shape {tuple(spec.shape)}.")
+    return tensor
 
 
 def random_tensors(specs: Sequence[WeightSpec], seed: int) -> dict[str, torch.Tensor]:

@@ -297,7 +297,7 @@ def attention_reference(case, scale, window=None):
 def query_tiles(case, first_sequence):
     """Tiles of at most 64 consecutive tokens for the sequences from ``first_sequence`` on."""
 
-    from miniserve_amd.parts import QueryTiles
+    from miniserve_amd.ops import QueryTiles
 
     seqs, tokens, lengths, base = [], [], [], 0
     for index, qlen in enumerate(case["query_lens"]):

@@ -31,7 +31,7 @@ def rand(*shape, seed=0):
 def step_context(query_lens, starts, block_size, *, tables=None):
     """A StepContext over one cache group, pages handed out in order (or ``tables``)."""
 
-    from miniserve_amd.parts import GroupStepView, QueryTiles, StepContext
+    from miniserve_amd.parts import GroupStepView, StepContext
 
     token_pos, seq_of, slots, table_rows = [], [], [], []
     next_page = 0
@@ -62,14 +62,14 @@ def step_context(query_lens, starts, block_size, *, tables=None):
             tile_seq.append(index)
             tile_token.append(starts_q[index] + start)
             tile_length.append(min(64, query_lens[index] - start))
-    tiles = QueryTiles(len(tile_seq), i32(tile_seq), i32(tile_token), i32(tile_length)) if tile_seq else None
+    tile_tables = {"attention.tile_seq": i32(tile_seq), "attention.tile_token": i32(tile_token), "attention.tile_length": i32(tile_length)}
     return StepContext(
         num_tokens=len(token_pos), num_seqs=len(query_lens), token_ids=i32([0] * len(token_pos)), positions=i32(token_pos),
         seq_of_token=i32(seq_of), query_start=i32(starts_q), context_lens=i32([s + q for s, q in zip(starts, query_lens)]),
         state_slots=i32(list(range(len(query_lens)))), groups=[GroupStepView(table, i32(slots))],
         query_lens=list(query_lens), context_lens_host=[s + q for s, q in zip(starts, query_lens)],
         query_start_host=starts_q, state_slots_host=list(range(len(query_lens))), first_positions_host=list(starts),
-        decode_prefix=prefix, tiles=tiles,
+        decode_prefix=prefix, tables=tile_tables if tile_seq else {},
     ), table_rows
 
 

@@ -1,8 +1,9 @@
-"""(c)'s generality: a toy mixer with state of its own and a toy architecture that
-uses it beside attention layers - one of them with a window, one named twice, one
-reading another call's cache - are defined HERE, registered, built from a model
-folder with random weights and stepped, without a change to the framework's files.
-They are no model of anyone's."""
+"""(c)'s generality: a toy mixer with state of its own, a toy feed-forward with
+routing, a toy position encoding and a toy architecture that uses them beside
+attention layers - one of them with a window, one named twice, one reading another
+call's cache - are defined HERE, registered, built from a model folder with random
+weights and stepped, without a change to the framework's files.  They are no model
+of anyone's."""
 
 from __future__ import annotations
 
@@ -19,7 +20,9 @@ from helpers import random_tokens, read_config, read_weights, tiny_a
 pytestmark = pytest.mark.gpu
 
 WINDOW = 6
-KINDS = ("attention", "running_mean", "window_attention")
+EXPERTS, EXPERT_WIDTH = 3, 40
+KINDS = ("attention", "running_mean", "window_attention")      # the mixers; layer 1 also has the routed feed-forward,
+                                                                # layer 2 the rotation of neighbouring pairs
 ORDER = ((0, None), (1, None), (2, None), (0, 0), (2, None), (1, None))    # (layer, cache_from)
 
 
@@ -47,19 +50,68 @@ def define_toy():
             return StateNeed((self.hidden + 1,), torch.float32)
 
         def forward(self, x, ctx, cache):
+            """Everything on the device, from the context's device tensors alone: a
+            recorded step gives no per-request numbers on the host."""
+
             assert isinstance(cache, StateView)
-            means = torch.empty_like(x, dtype=torch.float32)
-            for index in range(ctx.num_seqs):
-                begin, end = ctx.query_start_host[index], ctx.query_start_host[index + 1]
-                slot = ctx.state_slots_host[index]
-                state = cache.tensor[slot]
-                assert float(state[-1]) == ctx.first_positions_host[index]          # the state is this request's
-                sums = state[:-1] + torch.cumsum(x[begin:end].float(), dim=0)
-                counts = state[-1] + torch.arange(1, end - begin + 1, device=x.device, dtype=torch.float32)
-                means[begin:end] = sums / counts[:, None]
-                state[:-1] = sums[-1]
-                state[-1] = counts[-1]
-            return ops.linear(means.to(self.dtype).contiguous(), self.weight)
+            state = cache.tensor
+            seq, starts, slots = ctx.seq_of_token.long(), ctx.query_start.long(), ctx.state_slots.long()
+            running = torch.cumsum(x.double(), dim=0)
+            first = starts[seq]                                   # index of the first token of each token's sequence
+            before = running[(first - 1).clamp(min=0)] * (first > 0)[:, None]
+            kept = state[slots[seq]]
+            sums = kept[:, :-1] + (running - before).float()
+            place = torch.arange(x.shape[0], device=x.device)
+            counts = kept[:, -1] + (place - first + 1).float()
+            last = starts[1:] - 1
+            state[slots] = torch.cat([sums[last], counts[last, None]], dim=1)
+            return ops.linear((sums / counts[:, None]).to(self.dtype).contiguous(), self.weight)
+
+    class RoutedExperts(Part):
+        """A feed-forward with routing: router logits in 32-bit, the best of EXPERTS
+        experts per token, ``y = p_best * down_best(relu(up_best(x)))`` with p the softmax
+        of the router logits.  A toy: every expert runs on every row and the rows pick."""
+
+        def __init__(self, spec, dtype):
+            self.hidden, self.width, self.count = spec.params["hidden_size"], spec.params["width"], spec.params["experts"]
+            self.prefix, self.dtype = spec.prefix, dtype
+
+        def weight_specs(self):
+            decisive = lambda shape, generator, device: torch.randn(shape, generator=generator, dtype=torch.float32, device=device)
+            specs = [WeightSpec(self.prefix + "router.weight", (self.count, self.hidden), init=decisive, keep="float32")]
+            for expert in range(self.count):
+                specs.append(WeightSpec(f"{self.prefix}experts.{expert}.up.weight", (self.width, self.hidden)))
+                specs.append(WeightSpec(f"{self.prefix}experts.{expert}.down.weight", (self.hidden, self.width)))
+            return specs
+
+        def load_weights(self, tensors):
+            self.router = tensors[self.prefix + "router.weight"]
+            assert self.router.dtype == torch.float32                      # kept in 32-bit whatever the engine's dtype
+            self.up = [tensors[f"{self.prefix}experts.{e}.up.weight"] for e in range(self.count)]
+            self.down = [tensors[f"{self.prefix}experts.{e}.down.weight"] for e in range(self.count)]
+
+        def forward(self, x, ctx=None):
+            logits = ops.linear(x.float().contiguous(), self.router)      # [N, experts], true 32-bit
+            weight, chosen = torch.softmax(logits, dim=-1).max(dim=-1)
+            out = torch.zeros((x.shape[0], self.hidden), dtype=torch.float32, device=x.device)
+            for expert in range(self.count):
+                hidden = torch.relu(ops.linear(x, self.up[expert]))
+                out += (chosen == expert)[:, None] * ops.linear(hidden.contiguous(), self.down[expert]).float()
+            return (weight[:, None] * out).to(self.dtype)
+
+    class RotaryPairs(Part):
+        """Another position encoding: neighbouring pairs (2i, 2i + 1) are rotated by
+        ``position * theta^(-2i/dim)``."""
+
+        def __init__(self, spec, dtype):
+            self.dim, self.theta = spec.params["dim"], spec.params["theta"]
+
+        def apply(self, x, positions):
+            inv = 1.0 / (self.theta ** (torch.arange(0, self.dim, 2, device=x.device, dtype=torch.float32) / self.dim))
+            angle = positions.float()[:, None] * inv
+            cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+            even, odd = x[..., 0::2].float(), x[..., 1::2].float()
+            return torch.stack([even * cos - odd * sin, odd * cos + even * sin], dim=-1).reshape(x.shape).to(x.dtype)
 
     @dataclass(frozen=True)
     class ToyConfig:
@@ -87,10 +139,15 @@ def define_toy():
                 if kind == "running_mean":
                     mixer = PartSpec("test_running_mean", {"hidden_size": spec.hidden_size}, f"model.layers.{index}.mixer.")
                 elif kind == "window_attention":
-                    mixer = PartSpec("attention", {**layer.mixer.params, "window": WINDOW}, layer.mixer.prefix)
+                    position = PartSpec("test_rotary_pairs", dict(layer.mixer.params["position"].params))
+                    mixer = PartSpec("attention", {**layer.mixer.params, "window": WINDOW, "position": position}, layer.mixer.prefix)
                 else:
                     mixer = layer.mixer
-                layers.append(LayerSpec(layer.block, mixer, layer.feed_forward, layer.norms))
+                feed_forward = layer.feed_forward
+                if kind == "running_mean":
+                    feed_forward = PartSpec("test_routed_experts", {"hidden_size": spec.hidden_size, "width": EXPERT_WIDTH,
+                                                                    "experts": EXPERTS}, f"model.layers.{index}.moe.")
+                layers.append(LayerSpec(layer.block, mixer, feed_forward, layer.norms))
             return ModelSpec(
                 architecture=self.architecture, hidden_size=spec.hidden_size, vocab_size=spec.vocab_size,
                 max_positions=spec.max_positions, embedding=spec.embedding, layers=tuple(layers),
@@ -98,8 +155,41 @@ def define_toy():
             )
 
     register_part("mixer", "test_running_mean", RunningMean)
+    register_part("feed_forward", "test_routed_experts", RoutedExperts)
+    register_part("position", "test_rotary_pairs", RotaryPairs)
     register_architecture(ToyConfig.architecture, ToyConfig)
     return ToyConfig
+
+
+def pairs_attention(x, w, prefix, config, positions, window):
+    """Attention with the rotation of neighbouring pairs, from the plain parts."""
+
+    length, dim, eps = x.shape[0], config["head_dim"], config["rms_norm_eps"]
+    inv = 1.0 / (config["rope_theta"] ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))
+    angle = (positions.float()[:, None] * inv).double()
+
+    def rotate(t):          # [T, heads, dim]
+        even, odd = t[..., 0::2], t[..., 1::2]
+        cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+        return torch.stack([even * cos - odd * sin, odd * cos + even * sin], dim=-1).reshape(t.shape)
+
+    q = (x @ w[prefix + "q_proj.weight"].T).view(length, -1, dim)
+    k = (x @ w[prefix + "k_proj.weight"].T).view(length, -1, dim)
+    v = (x @ w[prefix + "v_proj.weight"].T).view(length, -1, dim)
+    q = rotate(plain.rms_norm(q, w[prefix + "q_norm.weight"], eps)).transpose(0, 1)
+    k = rotate(plain.rms_norm(k, w[prefix + "k_norm.weight"], eps)).transpose(0, 1)
+    attended = plain.causal_attention(q, k, v.transpose(0, 1), dim**-0.5, window)
+    return attended.transpose(0, 1).reshape(length, -1) @ w[prefix + "o_proj.weight"].T
+
+
+def routed_experts(x, w, prefix):
+    logits = (x.float() @ w[prefix + "router.weight"].float().T).double()      # the router's logits are 32-bit sums
+    weight, chosen = torch.softmax(logits, dim=-1).max(dim=-1)
+    out = torch.zeros_like(x)
+    for expert in range(EXPERTS):
+        y = torch.relu(x @ w[f"{prefix}experts.{expert}.up.weight"].T) @ w[f"{prefix}experts.{expert}.down.weight"].T
+        out = out + (chosen == expert)[:, None] * y
+    return weight[:, None] * out
 
 
 def toy_logits(weights, config, tokens):
@@ -117,13 +207,15 @@ def toy_logits(weights, config, tokens):
         if KINDS[layer] == "running_mean":
             mean = torch.cumsum(x, dim=0) / torch.arange(1, length + 1, dtype=torch.float64)[:, None]
             mixed = mean @ w[base + "mixer.proj.weight"].T
+        elif KINDS[layer] == "window_attention":
+            mixed = pairs_attention(x, w, base + "self_attn.", config, positions, WINDOW)
         else:
-            window = WINDOW if KINDS[layer] == "window_attention" else None
             mixed, kept[call] = plain.attention_block(
-                x, w, base + "self_attn.", config, positions, None if source is None else kept[source], window
+                x, w, base + "self_attn.", config, positions, None if source is None else kept[source], None
             )
         h = h + mixed
-        h = h + plain.swiglu(plain.rms_norm(h, w[base + "post_attention_layernorm.weight"], eps), w, base + "mlp.")
+        x = plain.rms_norm(h, w[base + "post_attention_layernorm.weight"], eps)
+        h = h + (routed_experts(x, w, base + "moe.") if KINDS[layer] == "running_mean" else plain.swiglu(x, w, base + "mlp."))
     return plain.rms_norm(h, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T
 
 
@@ -141,6 +233,8 @@ def toy(tmp_path_factory):
     assert type(load_config(folder)).__name__ == "ToyConfig"            # chosen by config.json through the registry
     yield folder
     unregister_part("mixer", "test_running_mean")
+    unregister_part("feed_forward", "test_routed_experts")
+    unregister_part("position", "test_rotary_pairs")
 
 
 def test_the_toy_model_is_built_from_its_folder(toy):
@@ -150,6 +244,8 @@ def test_the_toy_model_is_built_from_its_folder(toy):
 
     weights = read_weights(toy)
     assert "model.layers.1.mixer.proj.weight" in weights and "model.layers.1.self_attn.q_proj.weight" not in weights
+    assert "model.layers.1.moe.router.weight" in weights and "model.layers.1.mlp.gate_proj.weight" not in weights
+    assert float(weights["model.layers.1.moe.router.weight"].std()) > 0.5         # drawn by the part's own rule
     model = DecoderModel(load_config(toy).model_spec(), "float32")
     layout = CacheLayout.from_needs(model.cache_needs())
     # full attention: one cache (call 0, read again by call 3); window: two caches (calls 2, 4); two states (calls 1, 5)
@@ -206,3 +302,111 @@ def test_a_window_group_holds_few_pages_for_a_long_request(toy):
         assert 40 - free_window <= -(-WINDOW // 4) + 1                  # the window's pages, not the history's
     runner.release("long")
     assert runner.cache.capacity().free_blocks == (40, 40)
+
+
+# ---- state inside recorded steps, aborted steps and preemption ------------------------------------
+
+
+def toy_runner(toy, *, graphs, pages=24, seqs=4, block=16):
+    from miniserve_amd.config import EngineConfig
+    from miniserve_amd.engine import ModelRunner
+
+    return ModelRunner.from_folder(
+        toy, EngineConfig(dtype="float32", kv_block_size=block, num_kv_blocks=pages, max_num_seqs=seqs,
+                          enable_chunked_prefill=True, decode_graphs=graphs),
+    )
+
+
+def test_state_in_recorded_steps(toy):
+    """Single-token steps go through recorded graphs: the first step of each recorded
+    size runs eagerly and is then replayed, rows that fill a recording up use the spare
+    state slot.  Every step's logits equal the plain form's, so no state is updated
+    twice and none is mixed up."""
+
+    from miniserve_amd.engine import StepEntry
+
+    config, weights = read_config(toy), read_weights(toy)
+    requests = {f"r{i}": random_tokens(n, config["vocab_size"], 90 + i) for i, n in enumerate((21, 33, 27))}
+    expected = {rid: toy_logits(weights, config, tokens).float() for rid, tokens in requests.items()}
+    runner = toy_runner(toy, graphs=True)
+    heads = {"r0": 9, "r1": 14, "r2": 5}
+    for rid, tokens in requests.items():
+        runner.admit(rid)
+        logits = runner.step([StepEntry(rid, tuple(tokens[: heads[rid]]), (heads[rid] - 1,))])
+        assert float((logits[0].cpu() - expected[rid][heads[rid] - 1]).abs().max()) <= 2e-5
+    position = dict(heads)
+    live = list(requests)
+    steps = 0
+    while live:
+        entries = [StepEntry(rid, (requests[rid][position[rid]],), (0,)) for rid in live]
+        logits = runner.step(entries).cpu()
+        for row, rid in enumerate(live):
+            error = float((logits[row] - expected[rid][position[rid]]).abs().max())
+            assert error <= 2e-5, f"step {steps}, {rid} at {position[rid]}: {error:.3e}"
+            position[rid] += 1
+        for rid in [rid for rid in live if position[rid] == len(requests[rid])]:
+            runner.release(rid)
+            live.remove(rid)
+        steps += 1
+    assert runner.graph_steps == steps and sorted(runner._decode_graphs) == [1, 2, 4]      # three, two, one request
+
+
+def test_an_aborted_step_puts_the_state_back(toy):
+    """A step that fails after its mixers have written their state leaves no trace:
+    the same step, run again, gives the plain form's logits."""
+
+    from miniserve_amd.engine import StepEntry
+
+    config, weights = read_config(toy), read_weights(toy)
+    tokens = random_tokens(40, config["vocab_size"], 17)
+    expected = toy_logits(weights, config, tokens).float()
+    for graphs in (False, True):
+        runner = toy_runner(toy, graphs=graphs)
+        runner.admit("r")
+        runner.step([StepEntry("r", tuple(tokens[:12]), ())])
+        states_before = [tensor.clone() for tensor in runner.cache.state_tensors]
+        head_forward = runner.model.head.forward
+
+        def failing(x):
+            raise RuntimeError("the head fails")
+
+        runner.model.head.forward = failing
+        for entry in (StepEntry("r", tuple(tokens[12:20]), (7,)), StepEntry("r", (tokens[12],), (0,))):
+            with pytest.raises(RuntimeError, match="the head fails"):
+                runner.step([entry])
+            assert runner.cache.committed_tokens("r") == 12
+            for kept, tensor in zip(states_before, runner.cache.state_tensors):
+                assert torch.equal(kept, tensor)
+        runner.model.head.forward = head_forward
+        logits = runner.step([StepEntry("r", tuple(tokens[12:20]), (0, 7))]).cpu()
+        assert float((logits - expected[[12, 19]]).abs().max()) <= 2e-5
+        for place in range(20, 24):                      # single tokens: recorded steps when graphs are on
+            logits = runner.step([StepEntry("r", (tokens[place],), (0,))]).cpu()
+            assert float((logits[0] - expected[place]).abs().max()) <= 2e-5
+        runner.release("r")
+        runner.cache.assert_invariants()
+
+
+def test_a_preempted_request_builds_its_state_again(toy):
+    """With too few pages the youngest request loses its pages and its state slot and
+    is run again from its first token: the tokens are those of a roomy engine."""
+
+    from miniserve_amd.engine import SamplingParams
+    from miniserve_amd.entrypoint import LLM
+
+    config = read_config(toy)
+    prompts = [random_tokens(n, config["vocab_size"], 500 + n) for n in (30, 41, 18, 25)]
+    params = SamplingParams(max_new_tokens=24)
+    roomy = LLM(str(toy), dtype="float32", kv_block_size=16, num_kv_blocks=32, max_num_seqs=4)
+    expected = roomy.generate(prompts, params)
+    weights = read_weights(toy)
+    for prompt, tokens in zip(prompts[:2], expected[:2]):       # the roomy engine itself against the plain form
+        sequence = list(prompt)
+        for token in tokens[:6]:
+            top = torch.topk(toy_logits(weights, config, sequence)[-1], 2)
+            assert int(top.indices[0]) == token or float(top.values[0] - top.values[1]) < 1e-4
+            sequence.append(token)
+    tight = LLM(str(toy), dtype="float32", kv_block_size=16, num_kv_blocks=9, max_num_seqs=4, enable_chunked_prefill=True)
+    assert tight.generate(prompts, params) == expected
+    assert tight.engine.counters["preemptions"] > 0
+    tight.runner.cache.assert_invariants()
