@@ -37,6 +37,25 @@ class CapacitySnapshot:
     free_slots: int
     total_slots: int
     held_blocks: Mapping[str, tuple[int, ...]] = field(default_factory=dict)   # per live request, per group
+    windows: tuple[int | None, ...] = ()   # per group: the window of its layers, None = all keys are kept
+
+    def most_pages_held(self, total_tokens: int, step_tokens: int) -> tuple[int, ...]:
+        """The most pages of each group that one request of ``total_tokens`` holds at any
+        time when no step brings more than ``step_tokens``: all its pages where all keys
+        are kept; where a window has passed, only the pages from the oldest key that the
+        step's first token still sees to the step's last token (an edge page more, since
+        that span may begin anywhere inside a page)."""
+
+        whole = -(-total_tokens // self.block_size)
+        windows = self.windows or (None,) * len(self.total_blocks)
+        held = []
+        for window in windows:
+            if window is None:
+                held.append(whole)
+            else:
+                span = min(total_tokens, window - 1 + min(step_tokens, total_tokens))
+                held.append(min(whole, -(-span // self.block_size) + 1))
+        return tuple(held)
 
     def pages_for(self, before: int, after: int) -> int:
         """New pages that growing a request from ``before`` to ``after`` tokens takes in every group."""
@@ -247,11 +266,11 @@ class CacheManager:
                 live = self._live[item.request_id]
                 meta = SequenceStepMeta(item.request_id, live.state_slot, item.start, item.end, [], [], [])
                 for index, (allocator, table) in enumerate(zip(self.allocators, live.tables)):
-                    missing = table.required_blocks(item.end) - len(table.physical_block_ids)
+                    missing = table.pages_for(item.end) - len(table.pages)
                     new_pages = allocator.allocate(max(missing, 0))
                     taken.append((index, new_pages))
                     # without a new page the step reads the table's own snapshot, made once per change
-                    tentative = tuple(table.physical_block_ids + new_pages) if new_pages else table.snapshot()
+                    tentative = tuple(table.pages + new_pages) if new_pages else table.snapshot()
                     block_size = self.block_size
                     if item.end == item.start + 1:
                         logical, offset = divmod(item.start, block_size)
@@ -302,7 +321,7 @@ class CacheManager:
         for meta in reservation.sequences:
             live = self._live[meta.request_id]
             for group, table, pages in zip(self.layout.groups, live.tables, meta.new_pages):
-                table.append_blocks(pages)
+                table.extend(pages)
             live.committed = meta.after
             live.pending = False
             self._give_back_passed_pages(live)
@@ -350,6 +369,7 @@ class CacheManager:
                 request_id: tuple(table.live_count() for table in live.tables)
                 for request_id, live in self._live.items()
             },
+            windows=tuple(group.window for group in self.layout.groups),
         )
 
     def assert_invariants(self) -> None:

@@ -1,87 +1,90 @@
-"""A request's map from logical page index to physical page id, for one group
-(reference: miniserve/kv/block_table.py:9-53).  Pages that a window has passed
-are given back and their entries become ``RETURNED``."""
+"""One request's pages in one cache group, in the order of its tokens.
+
+Entry ``i`` names the page that holds positions ``i * block_size`` to
+``(i + 1) * block_size - 1``.  The pages need not be neighbours in the pool.  In a
+group with a window the oldest entries are given back while the request lives;
+they keep their place in the list as ``RETURNED`` so that positions still index it.
+(The reference's table maps positions the same way, without giving back:
+miniserve/kv/block_table.py:9-53.)
+"""
 
 from __future__ import annotations
-
-from dataclasses import dataclass, field
 
 RETURNED = -1
 
 
-def _is_int(value: object) -> bool:
-    return isinstance(value, int) and not isinstance(value, bool)
+def _whole(value: object) -> bool:
+    return type(value) is int and value >= 0
 
 
-@dataclass
 class BlockTable:
-    block_size: int
-    physical_block_ids: list[int] = field(default_factory=list)
-    first_live: int = 0          # logical index of the first page still held
-    _snapshot: tuple[int, ...] | None = field(default=None, repr=False, compare=False)   # kept until the table changes
+    def __init__(self, block_size: int, pages: list[int] | None = None) -> None:
+        if not _whole(block_size) or block_size == 0:
+            raise ValueError(f"a page holds a positive whole number of tokens, not {block_size!r}.")
+        self.block_size = block_size
+        self.pages: list[int] = []
+        self.first_live = 0                        # entries below it are RETURNED
+        self._tuple: tuple[int, ...] | None = None   # the table as a tuple, made when asked for, dropped on change
+        self.extend(list(pages or []))
 
-    def __post_init__(self) -> None:
-        if not _is_int(self.block_size) or self.block_size <= 0:
-            raise ValueError("block_size must be a positive integer.")
-        if any(not _is_int(page) or page < 0 for page in self.physical_block_ids):
-            raise ValueError("Physical block IDs must be non-negative integers.")
-        if len(self.physical_block_ids) != len(set(self.physical_block_ids)):
-            raise ValueError("One sequence block table cannot duplicate a physical ID.")
+    def pages_for(self, token_count: int) -> int:
+        """Pages that ``token_count`` tokens take."""
 
-    def required_blocks(self, token_count: int) -> int:
-        if not _is_int(token_count) or token_count < 0:
-            raise ValueError("token_count must be a non-negative integer.")
-        return (token_count + self.block_size - 1) // self.block_size
+        if not _whole(token_count):
+            raise ValueError(f"a number of tokens is a whole number, not {token_count!r}.")
+        return -(-token_count // self.block_size)
 
-    def append_blocks(self, block_ids: list[int]) -> None:
-        if isinstance(block_ids, list) and not block_ids:
-            return               # most steps of a decoding request bring no new page
-        if not isinstance(block_ids, list) or any(not _is_int(page) or page < 0 for page in block_ids):
-            raise ValueError("Appended physical block IDs must be a list of non-negative integers.")
-        if len(block_ids) != len(set(block_ids)) or set(block_ids) & set(self.live_pages()):
-            raise ValueError("Appended physical block IDs must be unique.")
-        self.physical_block_ids.extend(block_ids)
-        self._snapshot = None
+    def extend(self, new_pages: list[int]) -> None:
+        """Pages for the positions behind the last one the table covers."""
 
-    def resolve(self, token_position: int) -> tuple[int, int, int]:
-        """``(logical page, physical page, offset)`` of a position."""
+        if not new_pages:
+            return                                  # most steps of a decoding request bring no page
+        if not isinstance(new_pages, list) or not all(_whole(page) for page in new_pages):
+            raise ValueError(f"pages are named by whole numbers, in a list; got {new_pages!r}.")
+        if len(set(new_pages)) != len(new_pages) or not set(new_pages).isdisjoint(self.live_pages()):
+            raise ValueError(f"a table names a page once; {new_pages} repeats one.")
+        self.pages.extend(new_pages)
+        self._tuple = None
 
-        if not _is_int(token_position) or token_position < 0:
-            raise ValueError("token_position must be a non-negative integer.")
-        logical, offset = divmod(token_position, self.block_size)
-        if logical >= len(self.physical_block_ids):
-            raise IndexError("Token position has no reserved physical block.")
-        physical = self.physical_block_ids[logical]
-        if physical == RETURNED:
-            raise IndexError("Token position lies in a page that was given back.")
-        return logical, physical, offset
+    def locate(self, position: int) -> tuple[int, int, int]:
+        """``(entry, page, offset inside the page)`` of a token position."""
 
-    def slot(self, token_position: int) -> int:
-        _, physical, offset = self.resolve(token_position)
-        return physical * self.block_size + offset
+        if not _whole(position):
+            raise ValueError(f"a position is a whole number, not {position!r}.")
+        entry, offset = divmod(position, self.block_size)
+        if entry >= len(self.pages):
+            raise IndexError(f"position {position} lies behind the {len(self.pages)} pages of the table.")
+        if self.pages[entry] == RETURNED:
+            raise IndexError(f"position {position} lies in a page that was given back.")
+        return entry, self.pages[entry], offset
+
+    def slot(self, position: int) -> int:
+        """Where a position's key and value lie in the pool: ``page * block_size + offset``."""
+
+        _, page, offset = self.locate(position)
+        return page * self.block_size + offset
 
     def live_pages(self) -> list[int]:
-        return self.physical_block_ids[self.first_live :]
+        return self.pages[self.first_live :]
 
     def live_count(self) -> int:
-        return len(self.physical_block_ids) - self.first_live
+        return len(self.pages) - self.first_live
 
-    def give_back_before(self, token_position: int) -> list[int]:
-        """Pages whose every position is below ``token_position`` leave the table."""
+    def give_back_before(self, position: int) -> list[int]:
+        """The pages that lie wholly below ``position`` leave the table and are returned."""
 
-        limit = min(max(token_position, 0) // self.block_size, len(self.physical_block_ids))
-        returned = []
-        for logical in range(self.first_live, limit):
-            returned.append(self.physical_block_ids[logical])
-            self.physical_block_ids[logical] = RETURNED
-        self.first_live = max(self.first_live, limit)
-        if returned:
-            self._snapshot = None
-        return returned
+        end = min(max(position, 0) // self.block_size, len(self.pages))
+        gone = self.pages[self.first_live : end]
+        if gone:
+            self.pages[self.first_live : end] = [RETURNED] * len(gone)
+            self.first_live = end
+            self._tuple = None
+        return gone
 
     def snapshot(self) -> tuple[int, ...]:
-        """The table as a tuple; the same object until the table changes."""
+        """The table as a tuple; the same object until the table changes, so a reader
+        can tell by identity whether it has seen this table."""
 
-        if self._snapshot is None:
-            self._snapshot = tuple(self.physical_block_ids)
-        return self._snapshot
+        if self._tuple is None:
+            self._tuple = tuple(self.pages)
+        return self._tuple

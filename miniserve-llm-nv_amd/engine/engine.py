@@ -104,7 +104,10 @@ class Engine:
                 f"{params.max_new_tokens} exceeds max_model_len {self.max_model_len}."
             )
         capacity = self.runner.cache.capacity()
-        if capacity.pages_for(0, total) > min(capacity.total_blocks, default=1 << 60):
+        # (a preempted request runs all it holds again, so a step may bring up to total - 1 tokens or the budget)
+        step_tokens = self.max_num_batched_tokens if self.enable_chunked_prefill else total
+        needed = capacity.most_pages_held(total, step_tokens)
+        if any(pages > pool for pages, pool in zip(needed, capacity.total_blocks)):
             raise ValueError("CONTEXT_CAPACITY_EXCEEDED: the request alone needs more pages than the pool holds.")
         if any(token >= self.vocab_size for token in request.prompt_token_ids):
             raise ValueError("prompt token id is outside the vocabulary.")
@@ -165,7 +168,7 @@ class Engine:
             if state.status is RequestStatus.WAITING:
                 if not self.runner.cache.is_live(item.request_id):       # (a step planned ahead admitted it)
                     self.runner.admit(item.request_id)
-                state.begin_prefill()
+                state.admitted()
             tokens = state.tokens_between(item.token_start, item.token_end)
             final = item.token_end == state.prefill_target
             entries.append(StepEntry(item.request_id, tuple(tokens), (len(tokens) - 1,) if final else ()))
@@ -203,15 +206,15 @@ class Engine:
         self.counters["decode_tokens"] += len(plan.decode_items)
         self.counters["prefill_tokens"] += plan.scheduled_tokens - len(plan.decode_items)
         for item in plan.decode_items:
-            self._sequences[item.request_id].mark_decode_input_computed()
+            self._sequences[item.request_id].ran_pending_token()
         for item in plan.prefill_items:
-            self._sequences[item.request_id].commit_prefill(item.token_end)
+            self._sequences[item.request_id].ran_to(item.token_end)
         outputs: list[StepOutput] = []
         planned = set() if next_ahead is None else {item.request_id for item in next_ahead.plan.decode_items}
         # (the requests of its prompt portions are not sampled now and cannot end now)
         for state, sample in zip(sampled, staged):
-            state.append_sampled_token(sample.token_id)
-            reason = state.should_finish()
+            state.take_token(sample.token_id)
+            reason = state.ending()
             if reason is not None:
                 if next_ahead is not None and state.request_id in planned:
                     # a request of the step that was planned ahead ends (a stop token): that

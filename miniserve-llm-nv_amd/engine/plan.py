@@ -1,13 +1,24 @@
-"""What the scheduler decides for one step, as plain integers
-(reference: miniserve/engine/plan.py:8-84)."""
+"""What the scheduler decides for one step, as plain integers: which requests run
+a portion of their prompt, which run their pending sampled token, and which lose
+their cache first.  The plan carries no tensors and no references into the engine,
+so it can be made from views, logged, compared and replayed
+(the reference's counterpart: miniserve/engine/plan.py:8-84).
+"""
 
 from __future__ import annotations
 
 from dataclasses import dataclass
 
 
-def _is_int(value: object) -> bool:
-    return isinstance(value, int) and not isinstance(value, bool)
+def _whole_number(value: object) -> bool:
+    """A Python int that is not a bool and not negative."""
+
+    return type(value) is int and value >= 0
+
+
+def _named(request_id: object, what: str) -> None:
+    if not isinstance(request_id, str) or not request_id:
+        raise ValueError(f"a {what} needs the id of its request, got {request_id!r}.")
 
 
 @dataclass(frozen=True)
@@ -19,14 +30,15 @@ class PrefillItem:
     token_end: int
 
     def __post_init__(self) -> None:
-        if (
-            not self.request_id
-            or not _is_int(self.token_start)
-            or not _is_int(self.token_end)
-            or self.token_start < 0
-            or self.token_end <= self.token_start
-        ):
-            raise ValueError("Invalid prefill item.")
+        _named(self.request_id, "prompt portion")
+        if not (_whole_number(self.token_start) and _whole_number(self.token_end) and self.token_start < self.token_end):
+            raise ValueError(
+                f"prompt portion of {self.request_id!r}: [{self.token_start!r}, {self.token_end!r}) is no run of tokens."
+            )
+
+    @property
+    def num_tokens(self) -> int:
+        return self.token_end - self.token_start
 
 
 @dataclass(frozen=True)
@@ -38,41 +50,55 @@ class DecodeItem:
     position: int
 
     def __post_init__(self) -> None:
-        if (
-            not self.request_id
-            or not _is_int(self.input_token_id)
-            or not _is_int(self.position)
-            or self.input_token_id < 0
-            or self.position < 0
-        ):
-            raise ValueError("Invalid decode item.")
+        _named(self.request_id, "decode item")
+        if not (_whole_number(self.input_token_id) and _whole_number(self.position)):
+            raise ValueError(
+                f"decode item of {self.request_id!r}: token {self.input_token_id!r} at position {self.position!r} "
+                "must both be whole numbers."
+            )
+
+    num_tokens = 1
 
 
 @dataclass(frozen=True)
 class ExecutionPlan:
+    """One step.  ``preempted`` requests give their pages and their slot back before
+    the step runs and take no part in it; ``scheduled_tokens`` is the number of tokens
+    the step runs, kept beside the items so that a reader need not add them up and a
+    writer cannot get it wrong unnoticed."""
+
     step_id: int
     prefill_items: tuple[PrefillItem, ...] = ()
     decode_items: tuple[DecodeItem, ...] = ()
     scheduled_tokens: int = 0
-    preempted: tuple[str, ...] = ()      # requests that lose their cache before the step runs
+    preempted: tuple[str, ...] = ()
 
     def __post_init__(self) -> None:
-        if not _is_int(self.step_id) or not _is_int(self.scheduled_tokens) or self.step_id < 0 or self.scheduled_tokens < 0:
-            raise ValueError("step_id and scheduled_tokens must be non-negative.")
-        if not isinstance(self.prefill_items, tuple) or not isinstance(self.decode_items, tuple):
-            raise TypeError("ExecutionPlan items must be immutable tuples.")
-        if any(not isinstance(item, PrefillItem) for item in self.prefill_items) or any(
-            not isinstance(item, DecodeItem) for item in self.decode_items
-        ):
-            raise TypeError("ExecutionPlan contains an invalid item type.")
-        request_ids = [item.request_id for item in (*self.prefill_items, *self.decode_items)]
-        if len(request_ids) != len(set(request_ids)):
-            raise ValueError("A request may appear only once in one ExecutionPlan.")
-        if set(request_ids) & set(self.preempted):
-            raise ValueError("A preempted request cannot run in the same step.")
-        expected = sum(item.token_end - item.token_start for item in self.prefill_items) + len(self.decode_items)
-        if self.scheduled_tokens != expected:
-            raise ValueError("scheduled_tokens does not match plan items.")
+        for name, kind in (("prefill_items", PrefillItem), ("decode_items", DecodeItem)):
+            items = getattr(self, name)
+            if type(items) is not tuple:
+                raise TypeError(f"ExecutionPlan.{name} is a {type(items).__name__}; a plan is immutable and takes tuples.")
+            strangers = [type(item).__name__ for item in items if type(item) is not kind]
+            if strangers:
+                raise TypeError(f"ExecutionPlan.{name} holds {strangers[0]} where {kind.__name__} belongs.")
+        if not _whole_number(self.step_id) or not _whole_number(self.scheduled_tokens):
+            raise ValueError(f"step {self.step_id!r} with {self.scheduled_tokens!r} tokens: both must be whole numbers.")
+        running = self.request_ids
+        twice = {request_id for request_id in running if running.count(request_id) > 1}
+        if twice:
+            raise ValueError(f"requests {sorted(twice)} stand more than once in step {self.step_id}.")
+        both = set(running) & set(self.preempted)
+        if both:
+            raise ValueError(f"requests {sorted(both)} are preempted and run in the same step {self.step_id}.")
+        counted = sum(item.num_tokens for item in self.prefill_items) + len(self.decode_items)
+        if counted != self.scheduled_tokens:
+            raise ValueError(f"step {self.step_id} says {self.scheduled_tokens} tokens, its items hold {counted}.")
+
+    @property
+    def request_ids(self) -> tuple[str, ...]:
+        """The requests that run, decoding ones first (the order of the batch)."""
+
+        return tuple(item.request_id for item in (*self.decode_items, *self.prefill_items))
 
     @property
     def empty(self) -> bool:

@@ -324,6 +324,7 @@ class ModelRunner:
         """Pages that fit into 80% of the memory that is free after the weights,
         but no more than ``max_num_seqs`` full-length requests need."""
 
+        torch.cuda.empty_cache()      # what loading left behind (the unstacked matrices) goes back to the device first
         free_bytes, _ = torch.cuda.mem_get_info(self.device)
         itemsize = torch.empty((), dtype=self.dtype).element_size()
         per_block = max(layout.bytes_per_token(itemsize) * self.block_size, 1)

@@ -1,15 +1,24 @@
-"""One request's tokens and where it stands (reference: miniserve/engine/state.py:11-290).
+"""One request inside the engine: the tokens it holds and how far they have run.
 
-The invariant of the reference is kept: a DECODING request always holds exactly
-one sampled token that has not been run yet, ``total_tokens == computed_tokens + 1``.
-Beyond the reference a running request can be *preempted*: it loses its cache and
-goes back to WAITING; everything it holds so far (prompt and generated tokens) is
-then run again as one prefill of ``prefill_target`` tokens.
+Two numbers carry the whole state machine.  ``computed_tokens`` counts the tokens
+whose keys and values lie in the cache; ``prefill_target`` is how many must lie
+there before the next token may be sampled (the prompt; after a preemption,
+everything the request holds).  From them:
+
+    WAITING      nothing computed, no cache held
+    PREFILLING   computed <= target == all tokens held; nothing sampled is pending
+    DECODING     exactly one sampled token is held that has not run: computed == held - 1
+    FINISHED     as DECODING, with a reason ("stop" or "length"); the last token never runs
+    FAILED / CANCELLED   terminal, whatever the numbers were
+
+The phases and the rule of the one pending token are the reference's
+(miniserve/engine/state.py:11-290); preemption (back to WAITING with all tokens to
+run again) is this engine's own.
 """
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from enum import Enum, auto
 
 from .request import Request, SamplingParams
@@ -25,231 +34,252 @@ class RequestStatus(Enum):
 
 
 TERMINAL = frozenset({RequestStatus.FINISHED, RequestStatus.FAILED, RequestStatus.CANCELLED})
+RUNNING = frozenset({RequestStatus.PREFILLING, RequestStatus.DECODING})
+NORMAL_ENDS = ("stop", "length")
+
+
+class TransitionError(RuntimeError):
+    """A step asked a request for something its phase does not allow."""
 
 
 @dataclass(frozen=True)
 class SequenceView:
-    """What the scheduler may read; it cannot change the request through it."""
+    """The numbers of a request that the scheduler decides by.  A view is a copy: the
+    scheduler cannot change a request through it, and a view may describe a request as
+    a running step will leave it."""
 
     request_id: str
     status: RequestStatus
-    prefill_target: int        # tokens to run before the next token can be sampled
-    prefill_cursor: int
+    prefill_target: int
     computed_tokens: int
     total_tokens: int
     num_generated: int
     max_new_tokens: int
     arrival_ns: int
-    next_input_token_id: int | None
+    next_input_token_id: int | None        # DECODING: the pending token (0 where it is not known yet)
     num_preemptions: int = 0
+
+    @property
+    def age_key(self) -> tuple[int, str]:
+        """Older requests sort first; the id breaks ties of the clock."""
+
+        return (self.arrival_ns, self.request_id)
 
 
 @dataclass
 class SequenceState:
-    request_id: str
-    prompt_token_ids: tuple[int, ...]
-    generated_token_ids: list[int]
-    status: RequestStatus
-    prefill_target: int
-    prefill_cursor: int
-    computed_tokens: int
-    sampling_params: SamplingParams
-    arrival_ns: int
+    request: Request
+    generated_token_ids: list[int] = field(default_factory=list)
+    status: RequestStatus = RequestStatus.WAITING
+    computed_tokens: int = 0
+    prefill_target: int = 0
     finish_reason: str | None = None
     error_message: str | None = None
     num_preemptions: int = 0
 
     @classmethod
     def from_request(cls, request: Request) -> "SequenceState":
-        state = cls(
-            request_id=request.request_id,
-            prompt_token_ids=request.prompt_token_ids,
-            generated_token_ids=[],
-            status=RequestStatus.WAITING,
-            prefill_target=len(request.prompt_token_ids),
-            prefill_cursor=0,
-            computed_tokens=0,
-            sampling_params=request.sampling_params,
-            arrival_ns=request.arrival_ns,
-        )
-        state.assert_invariants()
-        return state
+        return cls(request=request, prefill_target=len(request.prompt_token_ids))
+
+    # ---- what it holds ----------------------------------------------------------------
+    @property
+    def request_id(self) -> str:
+        return self.request.request_id
 
     @property
-    def all_tokens(self) -> tuple[int, ...]:
-        return self.prompt_token_ids + tuple(self.generated_token_ids)
+    def prompt_token_ids(self) -> tuple[int, ...]:
+        return self.request.prompt_token_ids
 
-    def token_at(self, index: int) -> int:
-        """``all_tokens[index]`` without building the whole tuple (this is asked every step)."""
+    @property
+    def sampling_params(self) -> SamplingParams:
+        return self.request.sampling_params
 
-        prompt = len(self.prompt_token_ids)
-        return self.prompt_token_ids[index] if index < prompt else self.generated_token_ids[index - prompt]
-
-    def tokens_between(self, start: int, end: int) -> tuple[int, ...]:
-        """``all_tokens[start:end]``."""
-
-        prompt = len(self.prompt_token_ids)
-        if end <= prompt:
-            return self.prompt_token_ids[start:end]
-        if start >= prompt:
-            return tuple(self.generated_token_ids[start - prompt : end - prompt])
-        return self.prompt_token_ids[start:] + tuple(self.generated_token_ids[: end - prompt])
+    @property
+    def arrival_ns(self) -> int:
+        return self.request.arrival_ns
 
     @property
     def total_tokens(self) -> int:
-        return len(self.prompt_token_ids) + len(self.generated_token_ids)
+        return len(self.request.prompt_token_ids) + len(self.generated_token_ids)
 
-    def snapshot(self) -> SequenceView:
-        self.assert_invariants()
+    @property
+    def all_tokens(self) -> tuple[int, ...]:
+        return self.request.prompt_token_ids + tuple(self.generated_token_ids)
+
+    def token_at(self, index: int) -> int:
+        """Token ``index`` of prompt + generated, without joining the two."""
+
+        prompt = self.request.prompt_token_ids
+        return prompt[index] if index < len(prompt) else self.generated_token_ids[index - len(prompt)]
+
+    def tokens_between(self, start: int, end: int) -> tuple[int, ...]:
+        """Tokens ``[start, end)`` of prompt + generated."""
+
+        prompt = self.request.prompt_token_ids
+        from_prompt = prompt[start:end] if start < len(prompt) else ()
+        if end <= len(prompt):
+            return from_prompt
+        return from_prompt + tuple(self.generated_token_ids[max(start - len(prompt), 0) : end - len(prompt)])
+
+    # ---- views ------------------------------------------------------------------------
+    def _view(self, status: RequestStatus, computed: int, sampled_ahead: bool) -> SequenceView:
+        pending = None
+        if status is RequestStatus.DECODING:
+            pending = 0 if sampled_ahead else self.token_at(computed)
         return SequenceView(
             request_id=self.request_id,
-            status=self.status,
+            status=status,
             prefill_target=self.prefill_target,
-            prefill_cursor=self.prefill_cursor,
-            computed_tokens=self.computed_tokens,
-            total_tokens=self.total_tokens,
-            num_generated=len(self.generated_token_ids),
+            computed_tokens=computed,
+            total_tokens=self.total_tokens + int(sampled_ahead),
+            num_generated=len(self.generated_token_ids) + int(sampled_ahead),
             max_new_tokens=self.sampling_params.max_new_tokens,
             arrival_ns=self.arrival_ns,
-            next_input_token_id=(
-                self.token_at(self.computed_tokens) if self.status is RequestStatus.DECODING else None
-            ),
+            next_input_token_id=pending,
             num_preemptions=self.num_preemptions,
         )
 
-    def view_after(self, *, prefill_end: int | None = None, decoded: bool = False, sampled: bool = False) -> SequenceView:
-        """What :meth:`snapshot` will give once a running step is done: a step that ran
-        this request's prompt up to ``prefill_end``, or its pending token
-        (``decoded``), and that samples a token for it (``sampled``) which is not
-        known yet, so ``next_input_token_id`` is 0 in its place."""
+    def snapshot(self) -> SequenceView:
+        """The request as it stands."""
 
-        computed = self.computed_tokens + 1 if decoded else self.computed_tokens if prefill_end is None else prefill_end
+        self.check()
+        return self._view(self.status, self.computed_tokens, False)
+
+    def view_after(self, *, prefill_end: int | None = None, decoded: bool = False, sampled: bool = False) -> SequenceView:
+        """The request as a step that is still running will leave it: a step that runs
+        its tokens up to ``prefill_end``, or its pending token (``decoded``), and that
+        samples a token for it (``sampled``) whose id is not known yet."""
+
+        if decoded:
+            computed = self.computed_tokens + 1
+        elif prefill_end is not None:
+            computed = prefill_end
+        else:
+            computed = self.computed_tokens
         if sampled:
             status = RequestStatus.DECODING
         elif prefill_end is not None:
             status = RequestStatus.PREFILLING
         else:
             status = self.status
-        return SequenceView(
-            request_id=self.request_id,
-            status=status,
-            prefill_target=self.prefill_target,
-            prefill_cursor=self.prefill_cursor if prefill_end is None else prefill_end,
-            computed_tokens=computed,
-            total_tokens=self.total_tokens + int(sampled),
-            num_generated=len(self.generated_token_ids) + int(sampled),
-            max_new_tokens=self.sampling_params.max_new_tokens,
-            arrival_ns=self.arrival_ns,
-            next_input_token_id=(
-                0 if sampled else self.token_at(self.computed_tokens) if status is RequestStatus.DECODING else None
-            ),
-            num_preemptions=self.num_preemptions,
-        )
+        return self._view(status, computed, sampled)
 
-    # ---- transitions ------------------------------------------------------------------
-    def begin_prefill(self) -> None:
-        if self.status is not RequestStatus.WAITING:
-            raise RuntimeError("Only a waiting sequence can begin prefill.")
+    # ---- what a step does to it -----------------------------------------------------------
+    def _expect(self, *phases: RequestStatus, to: str) -> None:
+        if self.status not in phases:
+            names = " or ".join(phase.name for phase in phases)
+            raise TransitionError(f"request {self.request_id!r} is {self.status.name}; only a {names} request can {to}.")
+
+    def admitted(self) -> None:
+        """Admitted: it holds a cache slot and starts running its tokens."""
+
+        self._expect(RequestStatus.WAITING, to="be admitted")
         self.status = RequestStatus.PREFILLING
-        self.assert_invariants()
 
-    def commit_prefill(self, token_end: int) -> None:
-        """A portion of the prefill has run; a portion that does not end the prefill samples nothing."""
+    def ran_to(self, token_end: int) -> None:
+        """A step ran its tokens up to ``token_end``.  Nothing is sampled unless that is the target."""
 
-        if self.status is not RequestStatus.PREFILLING:
-            raise RuntimeError("Prompt completion requires PREFILLING state.")
-        if not self.prefill_cursor < token_end <= self.prefill_target:
-            raise RuntimeError("Prefill commit must advance within the prompt.")
-        self.prefill_cursor = token_end
+        self._expect(RequestStatus.PREFILLING, to="run a portion of its tokens")
+        if not self.computed_tokens < token_end <= self.prefill_target:
+            raise TransitionError(
+                f"request {self.request_id!r}: a portion ending at {token_end} does not move it forward from "
+                f"{self.computed_tokens} within its {self.prefill_target} tokens."
+            )
         self.computed_tokens = token_end
-        self.assert_invariants()
 
-    def mark_decode_input_computed(self) -> None:
-        if self.status is not RequestStatus.DECODING or self.computed_tokens != self.total_tokens - 1:
-            raise RuntimeError("Decode must consume exactly the pending sampled token.")
+    def ran_pending_token(self) -> None:
+        """A step ran the one pending token."""
+
+        self._expect(RequestStatus.DECODING, to="run its pending token")
+        if self.computed_tokens != self.total_tokens - 1:
+            raise TransitionError(f"request {self.request_id!r} holds no single pending token to run.")
         self.computed_tokens += 1
 
-    def append_sampled_token(self, token_id: int) -> None:
-        if self.status is not RequestStatus.PREFILLING and self.status is not RequestStatus.DECODING:
-            raise RuntimeError("A token can only be sampled after model execution.")
+    def take_token(self, token_id: int) -> None:
+        """The token sampled from the logits of its last computed position."""
+
+        self._expect(*RUNNING, to="take a sampled token")
         if self.computed_tokens != self.total_tokens:
-            raise RuntimeError("All current tokens must be computed before sampling the next token.")
-        if not isinstance(token_id, int) or isinstance(token_id, bool) or token_id < 0:
-            raise ValueError("token_id must be a non-negative integer.")
+            raise TransitionError(
+                f"request {self.request_id!r}: {self.total_tokens - self.computed_tokens} of its tokens have not run; "
+                "a token is sampled only after all of them."
+            )
+        if type(token_id) is not int or token_id < 0:
+            raise ValueError(f"a sampled token id is a whole number, not {token_id!r}.")
         self.generated_token_ids.append(token_id)
         self.status = RequestStatus.DECODING
-        self.assert_invariants()
+        self.check()
 
-    def should_finish(self) -> str | None:
-        """"stop" when the last token is a stop token (it stays in the output but is
-        never run), else "length" at ``max_new_tokens`` (reference: state.py:148-155)."""
+    def ending(self) -> str | None:
+        """Why the request ends with the token it took last, if it does: ``"stop"``
+        for a stop token (which stays in the output and never runs), ``"length"`` at
+        ``max_new_tokens``; a stop token at the length limit counts as ``"stop"``."""
 
         if not self.generated_token_ids:
             return None
-        if self.generated_token_ids[-1] in self.sampling_params.stop_token_ids:
+        params = self.sampling_params
+        if self.generated_token_ids[-1] in params.stop_token_ids:
             return "stop"
-        if len(self.generated_token_ids) >= self.sampling_params.max_new_tokens:
-            return "length"
-        return None
+        return "length" if len(self.generated_token_ids) >= params.max_new_tokens else None
 
     def finish(self, reason: str) -> None:
-        if self.status is not RequestStatus.DECODING:
-            raise RuntimeError("Only a decoding sequence can finish normally.")
-        if reason not in {"stop", "length"}:
-            raise ValueError("Normal finish reason must be 'stop' or 'length'.")
-        self.status = RequestStatus.FINISHED
-        self.finish_reason = reason
-        self.assert_invariants()
+        self._expect(RequestStatus.DECODING, to="end normally")
+        if reason not in NORMAL_ENDS:
+            raise ValueError(f"a request ends normally by one of {NORMAL_ENDS}, not {reason!r}.")
+        self.status, self.finish_reason = RequestStatus.FINISHED, reason
 
     def preempt(self) -> None:
-        """Lose the cache, keep the tokens: back to WAITING, all tokens to be run again."""
+        """It loses its cache and keeps its tokens: all of them run again, later, as one
+        prefill, after which the next token is sampled as if nothing had happened."""
 
-        if self.status not in {RequestStatus.PREFILLING, RequestStatus.DECODING}:
-            raise RuntimeError("Only a running sequence can be preempted.")
+        self._expect(*RUNNING, to="be preempted")
         self.status = RequestStatus.WAITING
         self.prefill_target = self.total_tokens
-        self.prefill_cursor = 0
         self.computed_tokens = 0
         self.num_preemptions += 1
-        self.assert_invariants()
 
     def cancel(self, reason: str = "cancelled") -> None:
         if self.status in TERMINAL:
-            raise RuntimeError("Terminal sequence cannot be cancelled again.")
-        self.status = RequestStatus.CANCELLED
-        self.finish_reason = reason
+            raise TransitionError(f"request {self.request_id!r} has ended ({self.status.name}) and cannot be cancelled.")
+        self.status, self.finish_reason = RequestStatus.CANCELLED, reason
 
     def fail(self, message: str) -> None:
         if self.status in TERMINAL:
-            raise RuntimeError("Terminal sequence cannot transition to FAILED.")
+            raise TransitionError(f"request {self.request_id!r} has ended ({self.status.name}) and cannot fail.")
         if not isinstance(message, str) or not message.strip():
-            raise ValueError("failure message must not be empty.")
-        self.status = RequestStatus.FAILED
-        self.finish_reason = "error"
-        self.error_message = message
+            raise ValueError("a failed request needs a message that says why.")
+        self.status, self.finish_reason, self.error_message = RequestStatus.FAILED, "error", message
 
-    # ---- invariants -------------------------------------------------------------------
-    def assert_invariants(self) -> None:
-        if not self.request_id or not self.prompt_token_ids:
-            raise AssertionError("Sequence identity and prompt must be non-empty.")
-        if not len(self.prompt_token_ids) <= self.prefill_target <= self.total_tokens:
-            raise AssertionError("prefill_target lies outside the sequence.")
-        if not 0 <= self.prefill_cursor <= self.prefill_target:
-            raise AssertionError("prefill_cursor is outside the prefill.")
-        if not 0 <= self.computed_tokens <= self.total_tokens:
-            raise AssertionError("computed_tokens is outside all_tokens.")
+    # ---- consistency ------------------------------------------------------------------------
+    def problems(self) -> list[str]:
+        """Everything about the numbers that does not fit the phase (empty when all is well)."""
+
+        found = []
+        held, done, target = self.total_tokens, self.computed_tokens, self.prefill_target
+        prompt = len(self.request.prompt_token_ids)
+        if not prompt <= target <= held:
+            found.append(f"target {target} lies outside prompt {prompt} .. held {held}")
+        if not 0 <= done <= held:
+            found.append(f"{done} tokens computed of {held} held")
         if len(self.generated_token_ids) > self.sampling_params.max_new_tokens:
-            raise AssertionError("generated tokens exceed max_new_tokens.")
-        status = self.status          # identity tests: hashing an enum member costs a Python call
+            found.append(f"{len(self.generated_token_ids)} tokens generated, {self.sampling_params.max_new_tokens} allowed")
+        status = self.status
+        if status is RequestStatus.WAITING and done != 0:
+            found.append(f"waiting with {done} tokens computed")
         if status is RequestStatus.WAITING or status is RequestStatus.PREFILLING:
-            if self.computed_tokens != self.prefill_cursor or self.prefill_target != self.total_tokens:
-                raise AssertionError("WAITING/PREFILLING only advances the prefill of all current tokens.")
-            if status is RequestStatus.WAITING and self.computed_tokens != 0:
-                raise AssertionError("WAITING holds no computed tokens.")
+            if target != held or done > target:
+                found.append(f"{status.name}: target {target}, held {held}, computed {done}")
         elif status is RequestStatus.DECODING or status is RequestStatus.FINISHED:
-            if not self.generated_token_ids or self.computed_tokens != self.total_tokens - 1:
-                raise AssertionError("Decode/finish must retain one sampled, uncomputed token.")
-        if status is RequestStatus.FINISHED and self.finish_reason not in {"stop", "length"}:
-            raise AssertionError("FINISHED state requires a normal finish reason.")
+            if not self.generated_token_ids or done != held - 1:
+                found.append(f"{status.name}: {done} computed of {held} held; exactly one sampled token must be pending")
+        if status is RequestStatus.FINISHED and self.finish_reason not in NORMAL_ENDS:
+            found.append(f"finished by {self.finish_reason!r}")
         if status is RequestStatus.FAILED and (self.finish_reason != "error" or not self.error_message):
-            raise AssertionError("FAILED state requires a separate diagnostic message.")
+            found.append("failed without a message")
+        return found
+
+    def check(self) -> None:
+        found = self.problems()
+        if found:
+            raise AssertionError(f"request {self.request_id!r} is inconsistent: " + "; ".join(found))
+

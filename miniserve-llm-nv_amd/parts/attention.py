@@ -24,6 +24,7 @@ from .base import (
     WeightSpec,
     build_part,
     register_part,
+    release_tensors,
     require_params,
 )
 from .norm import RMSNorm
@@ -107,12 +108,12 @@ class Attention(Part):
         """q, k and v rows are stacked into one matrix, q rows first, then k, then
         v, so one product gives the packed ``[N, (Hq + 2 Hkv) * D]`` row."""
 
-        q = tensors[self.prefix + "q_proj.weight"]
-        self.w_qkv = torch.cat(
-            [q, tensors[self.prefix + "k_proj.weight"], tensors[self.prefix + "v_proj.weight"]], dim=0
-        ).contiguous()
-        self.w_q = self.w_qkv[: q.shape[0]]
+        names = [self.prefix + part + "_proj.weight" for part in ("q", "k", "v")]
+        q_rows = tensors[names[0]].shape[0]
+        self.w_qkv = torch.cat([tensors[name] for name in names], dim=0).contiguous()
+        self.w_q = self.w_qkv[:q_rows]
         self.w_o = tensors[self.prefix + "o_proj.weight"]
+        release_tensors(tensors, names)       # the stacked copy serves from here on
 
     # -- execution ------------------------------------------------------------------
     def forward(self, x, ctx: StepContext, cache: KVCacheView, *, residual: torch.Tensor | None = None):

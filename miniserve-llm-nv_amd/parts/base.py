@@ -235,6 +235,16 @@ def require_params(spec: PartSpec, *names: str) -> Mapping[str, Any]:
     return spec.params
 
 
+def release_tensors(tensors, names) -> None:
+    """A part that has copied checkpoint tensors into a layout of its own (stacked
+    matrices) drops the originals from the mapping it was given, where the mapping
+    lets it: their memory is free before the cache pool is sized."""
+
+    if hasattr(tensors, "pop"):
+        for name in names:
+            tensors.pop(name, None)
+
+
 class Part:
     """Base of all parts: no weights, nothing to load."""
 

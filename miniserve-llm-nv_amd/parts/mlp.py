@@ -9,7 +9,7 @@ import torch
 
 from .. import ops
 from ..config.model_spec import PartSpec
-from .base import Part, PendingNorm, StepContext, WeightSpec, register_part, require_params
+from .base import Part, PendingNorm, StepContext, WeightSpec, register_part, release_tensors, require_params
 
 # activation name -> (gated activation of a packed [N, 2 I] row, the same fused with the product)
 _ACTIVATIONS = {"silu": (ops.silu_mul, ops.linear_silu_mul)}
@@ -43,10 +43,10 @@ class GatedMLP(Part):
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         """Gate rows, then up rows, in one matrix: one product gives ``[N, 2 I]``."""
 
-        self.w_gate_up = torch.cat(
-            [tensors[self.prefix + "gate_proj.weight"], tensors[self.prefix + "up_proj.weight"]], dim=0
-        ).contiguous()
+        names = [self.prefix + "gate_proj.weight", self.prefix + "up_proj.weight"]
+        self.w_gate_up = torch.cat([tensors[name] for name in names], dim=0).contiguous()
         self.w_down = tensors[self.prefix + "down_proj.weight"]
+        release_tensors(tensors, names)       # the stacked copy serves from here on
 
     def forward(self, x, ctx: StepContext | None = None, *, residual: torch.Tensor | None = None):
         """``x``: the normed input, or a ``PendingNorm`` (then the norm becomes the

@@ -55,17 +55,22 @@ def test_out_of_pages_and_invalid_release_are_atomic():
     # reference: tests/unit/test_block_allocator.py:26-37
     allocator = PageAllocator(3)
     allocator.allocate(2)
-    before = allocator.snapshot()
-    with pytest.raises(OutOfPagesError, match="OUT_OF_BLOCKS"):
+    state = lambda: (allocator.free_ids(), [allocator.refcount(page) for page in range(3)])
+    before = state()
+    with pytest.raises(OutOfPagesError, match="2 asked for, 1 of 3 free"):
         allocator.allocate(2)
-    assert allocator.snapshot() == before
-    with pytest.raises(RuntimeError, match="free block"):
-        allocator.release((2,))
-    assert allocator.snapshot() == before
-    with pytest.raises(ValueError, match="Duplicate"):
+    assert state() == before
+    with pytest.raises(RuntimeError, match="they are free"):
+        allocator.release((0, 2))           # page 0 is held, page 2 is not: neither changes
+    assert state() == before
+    with pytest.raises(ValueError, match="named twice"):
         allocator.release((0, 0))
     with pytest.raises(IndexError):
         allocator.release((3,))
+    with pytest.raises(TypeError):
+        allocator.release((True,))
+    assert state() == before
+    allocator.assert_invariants()
 
 
 def test_lowest_id_first_after_release():
@@ -79,7 +84,7 @@ def test_lowest_id_first_after_release():
 def test_allocator_rejects_coercible_or_invalid_counts(value):
     with pytest.raises((TypeError, ValueError)):
         PageAllocator(value)
-    with pytest.raises(ValueError, match="non-negative integer"):
+    with pytest.raises(ValueError, match="whole number"):
         PageAllocator(2).allocate(value)
 
 
@@ -90,7 +95,7 @@ def test_allocator_rejects_coercible_or_invalid_counts(value):
 def test_noncontiguous_block_table_boundaries(position, expected):
     # reference: tests/unit/test_block_allocator.py:66-81
     table = BlockTable(16, [5, 2, 7])
-    assert table.resolve(position) == expected
+    assert table.locate(position) == expected
     assert table.slot(position) == expected[1] * 16 + expected[2]
 
 
@@ -100,13 +105,13 @@ def test_block_table_rejects_invalid_metadata():
             BlockTable(block_size, ids)
     table = BlockTable(16, [0])
     with pytest.raises(ValueError):
-        table.append_blocks([True])
+        table.extend([True])
     with pytest.raises(ValueError):
-        table.append_blocks([0])
+        table.extend([0])
     with pytest.raises(ValueError):
-        table.resolve(1.5)
+        table.locate(1.5)
     with pytest.raises(IndexError):
-        table.resolve(16)
+        table.locate(16)
 
 
 def test_window_table_gives_pages_back():
@@ -115,9 +120,9 @@ def test_window_table_gives_pages_back():
     assert table.give_back_before(9) == [9, 8]
     assert table.snapshot() == (RETURNED, RETURNED, 7, 6) and table.live_pages() == [7, 6]
     with pytest.raises(IndexError, match="given back"):
-        table.resolve(5)
+        table.locate(5)
     assert table.give_back_before(8) == []
-    table.append_blocks([9])
+    table.extend([9])
     assert table.slot(16) == 9 * 4
 
 
@@ -125,9 +130,9 @@ def test_the_snapshot_is_one_object_until_the_table_changes():
     table = BlockTable(4, [3, 5])
     first = table.snapshot()
     assert first == (3, 5) and table.snapshot() is first
-    table.append_blocks([])
+    table.extend([])
     assert table.snapshot() is first and table.live_count() == 2
-    table.append_blocks([7])
+    table.extend([7])
     assert table.snapshot() == (3, 5, 7) and table.snapshot() is not first
     kept = table.snapshot()
     assert table.give_back_before(3) == [] and table.snapshot() is kept
@@ -258,6 +263,32 @@ def test_window_group_gives_pages_back_while_the_request_lives():
     assert length == 22                     # 6 pages of history passed through a pool of 4
     m.release("r")
     assert m.capacity().free_blocks == (16, 4)
+
+
+def test_the_most_pages_a_request_holds_follow_the_window_of_each_group():
+    """What admission compares with the pools: all pages where all keys are kept, the
+    window's span (and the step's tokens) where a window has passed; measured here on
+    a real run of the manager."""
+
+    needs = [Need(0, KVCacheNeed(1, 16)), Need(1, KVCacheNeed(1, 16, window=6))]
+    m = manager(needs, block_size=4, num_blocks=[64, 64], max_len=256)
+    capacity = m.capacity()
+    assert capacity.windows == (None, 6)
+    assert capacity.most_pages_held(200, 200) == (50, 50)          # one step brings everything
+    assert capacity.most_pages_held(200, 1) == (50, 3)             # single tokens: 6 keys over at most 3 pages
+    assert capacity.most_pages_held(200, 7) == (50, 4)
+    assert capacity.most_pages_held(3, 7) == (1, 1)
+    for step_tokens in (1, 3, 7, 16):
+        m.admit("r")
+        length, most = 0, 0
+        while length < 120:
+            step = m.prepare_step([StepItem("r", length, length + step_tokens)])
+            most = max(most, 64 - m.capacity().free_blocks[1])
+            m.commit_step(step)
+            length += step_tokens
+        assert most <= capacity.most_pages_held(120, step_tokens)[1]
+        assert most >= capacity.most_pages_held(120, step_tokens)[1] - 1        # the bound is not loose
+        m.release("r")
 
 
 @pytest.mark.parametrize("seed", range(6))

@@ -176,6 +176,79 @@ def test_whole_model_causality_and_head(models):
     )
 
 
+def test_the_attention_block_takes_the_library_routines_own_scale(models):
+    """The scale that ``attention_block`` itself chooses (no caller hands it in) is the
+    default of the library's attention, 1/sqrt(head_dim): with the output projection
+    set to the identity the block is the library routine over the normed, rotated
+    heads.  A scale of 1/head_dim, or none, fails."""
+
+    weights, config = models["a"]                     # 4 heads of 16 = the hidden size: the projection can be the identity
+    heads, kv_heads, dim = config["num_attention_heads"], config["num_key_value_heads"], config["head_dim"]
+    assert heads * dim == config["hidden_size"]
+    w = {name: tensor.to(F64) for name, tensor in weights.items()}
+    prefix = "model.layers.0.self_attn."
+    w[prefix + "o_proj.weight"] = torch.eye(heads * dim, dtype=F64)
+    generator = torch.Generator().manual_seed(12)
+    x = torch.randn(11, config["hidden_size"], generator=generator, dtype=F64)
+    positions = torch.arange(3, 14)
+    got, _ = plain.attention_block(x, w, prefix, config, positions)
+    cos, sin = plain.rope_angles(positions, dim, config["rope_theta"])
+    q = plain.rms_norm((x @ w[prefix + "q_proj.weight"].T).view(11, heads, dim), w[prefix + "q_norm.weight"], config["rms_norm_eps"])
+    k = plain.rms_norm((x @ w[prefix + "k_proj.weight"].T).view(11, kv_heads, dim), w[prefix + "k_norm.weight"], config["rms_norm_eps"])
+    v = (x @ w[prefix + "v_proj.weight"].T).view(11, kv_heads, dim)
+    q, k = plain.apply_rope(q.transpose(0, 1), cos, sin), plain.apply_rope(k.transpose(0, 1), cos, sin)
+    k, v = plain.repeat_kv(k, heads // kv_heads), plain.repeat_kv(v.transpose(0, 1), heads // kv_heads)
+    expected = F.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True)[0]     # the library's default scale
+    torch.testing.assert_close(got, expected.transpose(0, 1).reshape(11, heads * dim))
+
+
+def test_layers_that_add_nothing_leave_the_final_norm_and_the_head(models):
+    """With every output projection zero each layer adds nothing to the residual
+    stream, and the logits are the library's RMSNorm of the embeddings times the head:
+    the final norm is there, once, with the model's eps and weight, before the head."""
+
+    for name, (weights, config) in models.items():
+        w = {key: (torch.zeros_like(tensor) if key.endswith(("o_proj.weight", "down_proj.weight")) else tensor).to(F64)
+             for key, tensor in weights.items()}
+        tokens = random_tokens(9, config["vocab_size"], 2)
+        embedded = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+        normed = F.rms_norm(embedded, (config["hidden_size"],), w["model.norm.weight"], config["rms_norm_eps"])
+        head = w["model.embed_tokens.weight"] if config["tie_word_embeddings"] else w["lm_head.weight"]
+        torch.testing.assert_close(plain.forward_logits(w, config, tokens), normed @ head.T)
+
+
+def test_a_layer_norms_before_its_parts_not_after(models):
+    """Pre-norm: what a layer adds to the residual stream does not change when the
+    stream is scaled, because each part sees the stream through an RMSNorm (the eps
+    aside); the stream itself passes unnormed.  A norm after the sum, or a part fed the
+    bare stream, fails this."""
+
+    for name, (weights, config) in models.items():
+        w = {key: tensor.to(F64) for key, tensor in weights.items()}
+        generator = torch.Generator().manual_seed(3)
+        h = torch.randn(7, config["hidden_size"], generator=generator, dtype=F64)
+        positions = torch.arange(7)
+        # the mixer's share alone: the feed-forward adds nothing
+        attention_only = dict(w)
+        attention_only["model.layers.0.mlp.down_proj.weight"] = torch.zeros_like(w["model.layers.0.mlp.down_proj.weight"])
+        added = plain.decoder_layer(h, attention_only, 0, config, positions)[0] - h
+        added_scaled = plain.decoder_layer(5.0 * h, attention_only, 0, config, positions)[0] - 5.0 * h
+        torch.testing.assert_close(added_scaled, added, atol=1e-6, rtol=1e-4)       # the eps is all that differs
+        assert float(added.abs().max()) > 1e-3
+        # the feed-forward's share alone: the mixer adds nothing
+        mlp_only = dict(w)
+        mlp_only["model.layers.0.self_attn.o_proj.weight"] = torch.zeros_like(w["model.layers.0.self_attn.o_proj.weight"])
+        added = plain.decoder_layer(h, mlp_only, 0, config, positions)[0] - h
+        added_scaled = plain.decoder_layer(5.0 * h, mlp_only, 0, config, positions)[0] - 5.0 * h
+        torch.testing.assert_close(added_scaled, added, atol=1e-6, rtol=1e-4)       # the eps is all that differs
+        assert float(added.abs().max()) > 1e-3
+        # and the whole layer is the stream plus both shares, the second taken of the stream after the first
+        after_attention = plain.decoder_layer(h, attention_only, 0, config, positions)[0]
+        x = plain.rms_norm(after_attention, w["model.layers.0.post_attention_layernorm.weight"], config["rms_norm_eps"])
+        torch.testing.assert_close(plain.decoder_layer(h, w, 0, config, positions)[0],
+                                   after_attention + plain.swiglu(x, w, "model.layers.0.mlp."))
+
+
 def test_only_distances_count(models):
     """A shift of all positions leaves the logits unchanged: the rotation enters
     through q.k alone, which depends on distances."""

@@ -29,8 +29,7 @@ def view(name, status, *, target=10, cursor=0, generated=0, arrival=0, max_new=8
     computed = cursor if status is not D else target + generated - 1
     total = target if status is not D else target + generated
     return SequenceView(
-        request_id=name, status=status, prefill_target=target, prefill_cursor=cursor if status is not D else target,
-        computed_tokens=computed, total_tokens=total, num_generated=generated, max_new_tokens=max_new,
+        request_id=name, status=status, prefill_target=target, computed_tokens=computed, total_tokens=total, num_generated=generated, max_new_tokens=max_new,
         arrival_ns=arrival, next_input_token_id=7 if status is D else None,
     )
 
@@ -54,27 +53,27 @@ def request(max_new_tokens=2, stop=()):
 def test_prefill_and_decode_preserve_pending_token_invariant():
     # reference: tests/unit/test_sequence_state.py:54-71
     state = SequenceState.from_request(request())
-    state.begin_prefill()
-    state.commit_prefill(3)
-    state.append_sampled_token(42)
+    state.admitted()
+    state.ran_to(3)
+    state.take_token(42)
     assert state.status is D and state.all_tokens == (10, 20, 30, 42)
     assert state.computed_tokens == 3 and state.total_tokens == state.computed_tokens + 1
     assert state.snapshot().next_input_token_id == 42
-    state.mark_decode_input_computed()
-    state.append_sampled_token(43)
-    assert state.should_finish() == "length"
+    state.ran_pending_token()
+    state.take_token(43)
+    assert state.ending() == "length"
     state.finish("length")
     assert state.status is RequestStatus.FINISHED and state.computed_tokens == state.total_tokens - 1
 
 
 def test_tokens_are_read_without_building_the_whole_sequence():
     state = SequenceState.from_request(request(max_new_tokens=4))
-    state.begin_prefill()
-    state.commit_prefill(3)
+    state.admitted()
+    state.ran_to(3)
     for token in (42, 43):
-        state.append_sampled_token(token)
-        state.mark_decode_input_computed()
-    state.append_sampled_token(44)
+        state.take_token(token)
+        state.ran_pending_token()
+    state.take_token(44)
     everything = state.all_tokens
     assert everything == (10, 20, 30, 42, 43, 44)
     assert [state.token_at(i) for i in range(6)] == list(everything)
@@ -86,10 +85,10 @@ def test_tokens_are_read_without_building_the_whole_sequence():
 def test_stop_token_finishes_without_being_run():
     # reference: tests/unit/test_sequence_state.py:74-82
     state = SequenceState.from_request(request(max_new_tokens=4, stop=(99,)))
-    state.begin_prefill()
-    state.commit_prefill(3)
-    state.append_sampled_token(99)
-    assert state.should_finish() == "stop"
+    state.admitted()
+    state.ran_to(3)
+    state.take_token(99)
+    assert state.ending() == "stop"
     state.finish("stop")
     assert state.computed_tokens == 3 and state.total_tokens == 4
 
@@ -97,47 +96,47 @@ def test_stop_token_finishes_without_being_run():
 def test_partial_prefill_does_not_sample_and_illegal_moves_fail():
     # reference: tests/unit/test_sequence_state.py:84-104
     state = SequenceState.from_request(request())
-    with pytest.raises(RuntimeError, match="pending sampled token"):
-        state.mark_decode_input_computed()
-    state.begin_prefill()
-    state.commit_prefill(2)
-    assert state.status is P and state.prefill_cursor == state.computed_tokens == 2
-    with pytest.raises(RuntimeError, match="must be computed before sampling"):
-        state.append_sampled_token(1)
-    with pytest.raises(RuntimeError, match="advance within the prompt"):
-        state.commit_prefill(2)
-    state.commit_prefill(3)
-    state.append_sampled_token(42)
+    with pytest.raises(RuntimeError, match="only a DECODING request can run its pending token"):
+        state.ran_pending_token()
+    state.admitted()
+    state.ran_to(2)
+    assert state.status is P and state.computed_tokens == 2
+    with pytest.raises(RuntimeError, match="a token is sampled only after all of them"):
+        state.take_token(1)
+    with pytest.raises(RuntimeError, match="does not move it forward"):
+        state.ran_to(2)
+    state.ran_to(3)
+    state.take_token(42)
     assert state.status is D
 
 
 def test_preemption_keeps_tokens_and_runs_them_again():
     state = SequenceState.from_request(request(max_new_tokens=5))
-    state.begin_prefill()
-    state.commit_prefill(3)
-    state.append_sampled_token(42)
-    state.mark_decode_input_computed()
-    state.append_sampled_token(43)
+    state.admitted()
+    state.ran_to(3)
+    state.take_token(42)
+    state.ran_pending_token()
+    state.take_token(43)
     state.preempt()
     snapshot = state.snapshot()
     assert snapshot.status is W and snapshot.prefill_target == 5 and snapshot.computed_tokens == 0
     assert snapshot.num_generated == 2 and snapshot.num_preemptions == 1
-    state.begin_prefill()
-    state.commit_prefill(5)
-    state.append_sampled_token(44)
+    state.admitted()
+    state.ran_to(5)
+    state.take_token(44)
     assert state.all_tokens == (10, 20, 30, 42, 43, 44) and state.status is D
 
 
 def test_plan_checks():
     # reference: tests/unit/test_sequence_state.py:107-138
     ExecutionPlan(0, (PrefillItem("r", 0, 3),), (), 3)
-    with pytest.raises(ValueError, match="does not match"):
+    with pytest.raises(ValueError, match="its items hold"):
         ExecutionPlan(2, (PrefillItem("r", 0, 2),), (), 1)
-    with pytest.raises(TypeError, match="immutable tuples"):
+    with pytest.raises(TypeError, match="takes tuples"):
         ExecutionPlan(0, [PrefillItem("r", 0, 1)], (), 1)
-    with pytest.raises(ValueError, match="only once"):
+    with pytest.raises(ValueError, match="more than once"):
         ExecutionPlan(0, (PrefillItem("r", 0, 1),), (DecodeItem("r", 1, 1),), 2)
-    with pytest.raises(ValueError, match="same step"):
+    with pytest.raises(ValueError, match="preempted and run in the same step"):
         ExecutionPlan(0, (PrefillItem("r", 0, 1),), (), 1, preempted=("r",))
     for invalid in (True, 1.5):
         with pytest.raises(ValueError):
@@ -277,7 +276,7 @@ def test_budgets_hold_for_random_views(seed):
             pages -= -(-(v.computed_tokens + 1) // 4) - -(-v.computed_tokens // 4)
         for item in plan.prefill_items:
             v = by_id[item.request_id]
-            assert item.token_start == v.prefill_cursor and item.token_end <= v.prefill_target
+            assert item.token_start == v.computed_tokens and item.token_end <= v.prefill_target
             if not chunked:
                 assert item.token_end == v.prefill_target
             pages -= -(-item.token_end // 4) - -(-item.token_start // 4)
