@@ -1,17 +1,29 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--size 0.6B|8B|32B] [--parity]
 
 A "step" is one decode step of the engine loop (schedule, the step function over
 the paged cache, sampling) with ``--batch`` live requests, each after a prompt of
 ``--prompt-len`` random tokens.  The model has the layer sizes of Qwen3-0.6B (or
-of ``--size``) with random weights.  One JSON line is printed: decoded tokens a second, the prefill
-rate of one 2,048-token prompt with its fraction of the bf16 MFMA peak, the
-fraction of the HBM peak that the decode step reaches, decode rates at batch 1 and
-64, a mixed run (64 requests with prompts of 128 to 2,048 tokens, portions of 512
-beside decode tokens under a budget of 2,048 tokens a step, through the scheduler), and what the card reaches on a plain
-device copy and a large library product (the two fractions are given against these
-measured rates as well as against the published peaks).
+of ``--size``) with random weights.  One JSON line is printed.
+
+How the numbers are taken.  ``value`` and ``ms_per_step``: the wall clock around
+exactly ``--steps`` steps, a device synchronisation on both sides.  Beside it the
+same steps by device events (one recorded before every step): the median step and
+sixteen of the samples are kept (``decode_device``).  The prefill of one
+2,048-token prompt is timed by device events over five runs after one that is not
+counted; the median counts and all five samples are kept.  ``roofline`` and
+``points_frac``: the bytes a decode step has to read (every weight once, the cache of
+the live requests at their mean length) over its time, as a fraction of the
+published 8 TB/s.  ``mixed``: 64 requests with prompts of 128 to 2,048 tokens arrive
+at once and generate 128 tokens each, portions of 512 beside decode tokens under a
+budget of 2,048 tokens a step, through the scheduler; all tokens over the wall time,
+and by device events per step the share of steps that only decode (as a fraction
+of the HBM peak) and of steps that run prompt portions (as a fraction of the MFMA
+peak).  ``measured``: what the card reaches on a plain device copy and a large
+library product.  ``--parity`` adds a 32-bit run of the same layer sizes (two layers
+unless ``--layers`` says otherwise) against the plain float64 implementation of
+``tests/plain_qwen3.py``: a prompt whole, then 32 tokens one by one.
 """
 
 from __future__ import annotations
@@ -30,17 +42,7 @@ if ROOT not in sys.path:
 # MI355X published peaks
 HBM_GBPS = 8000.0
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}
-
-# layer sizes of the Qwen3 dense models; the default run is the first
-_COMMON = dict(head_dim=128, vocab_size=151936, max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1e6)
-SIZES = {
-    "0.6B": dict(hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16,
-                 num_key_value_heads=8, tie_word_embeddings=True, **_COMMON),
-    "8B": dict(hidden_size=4096, intermediate_size=12288, num_hidden_layers=36, num_attention_heads=32,
-               num_key_value_heads=8, tie_word_embeddings=False, **_COMMON),
-    "32B": dict(hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64,
-                num_key_value_heads=8, tie_word_embeddings=False, **_COMMON),
-}
+SIZES = ("0.6B", "8B", "32B")       # layer sizes that ship as config presets (qwen3-<size>)
 
 
 def parse_args():
@@ -51,7 +53,7 @@ def parse_args():
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--prompt-len", type=int, default=2048)
     parser.add_argument("--context", type=int, default=4096)
-    parser.add_argument("--size", default="0.6B", choices=tuple(SIZES), help="layer sizes of this Qwen3 model")
+    parser.add_argument("--size", default="0.6B", choices=SIZES, help="layer sizes of this Qwen3 model")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--prefill-tokens", type=int, default=2048)
@@ -59,6 +61,8 @@ def parse_args():
     parser.add_argument("--mixed-requests", type=int, default=64, help="requests of the mixed continuous-batching run")
     parser.add_argument("--mixed-new-tokens", type=int, default=128, help="tokens each of them generates")
     parser.add_argument("--eager", action="store_true", help="no HIP graphs for decode steps")
+    parser.add_argument("--parity", action="store_true",
+                        help="also run these layer sizes in 32-bit against the plain float64 implementation")
     return parser.parse_args()
 
 
@@ -80,6 +84,14 @@ def weight_bytes(model, itemsize):
     return total
 
 
+def per_token_flops(config):
+    """Matrix products of all layers on one row of the batch (without attention and head)."""
+
+    h, i, layers = config.hidden_size, config.intermediate_size, config.num_hidden_layers
+    q, kv = config.num_attention_heads * config.head_dim, config.num_key_value_heads * config.head_dim
+    return layers * 2 * (h * (q + 2 * kv) + q * h + 3 * h * i)
+
+
 def prefill_flops(config, tokens):
     """Matrix products of the layers and of the head on one row, plus causal attention
     (2 * heads * head_dim * T^2 per layer: two products over the lower triangle)."""
@@ -91,6 +103,57 @@ def prefill_flops(config, tokens):
         2 * h * config.vocab_size
 
 
+def parity_run(sizes, layers, device, prompt_len=300, tail=32):
+    """The same layer sizes in true 32-bit against the plain float64 implementation of
+    the tests: a model folder with random weights, a prompt whole and ``tail`` tokens
+    one by one; the largest difference of a logit, the largest logit, and whether the
+    tokens decoded one by one gave the logits of the whole run to the bit."""
+
+    import tempfile
+
+    import torch
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import plain_qwen3
+
+    from miniserve_amd.config import EngineConfig, config_from_dict
+    from miniserve_amd.engine import ModelRunner, StepEntry
+    from miniserve_amd.weights import write_random_model
+
+    data = dict(sizes)
+    data["num_hidden_layers"] = layers
+    data["max_position_embeddings"] = 1024
+    generator = torch.Generator().manual_seed(1)
+    tokens = torch.randint(0, data["vocab_size"], (prompt_len + tail,), generator=generator).tolist()
+    places = list(range(0, prompt_len, 25)) + list(range(prompt_len - 1, prompt_len + tail))
+    with tempfile.TemporaryDirectory() as folder:
+        write_random_model(config_from_dict(data), folder, seed=2, store_dtype="bfloat16")
+        from safetensors.torch import load_file
+
+        weights = {name: tensor.double() for name, tensor in load_file(os.path.join(folder, "model.safetensors")).items()}
+        exact = plain_qwen3.forward_logits(weights, data, tokens, rows=places).float()
+        del weights
+        engine_config = EngineConfig(dtype="float32", kv_block_size=16, num_kv_blocks=2 * (len(tokens) // 16 + 2),
+                                     max_num_seqs=2, enable_chunked_prefill=True, decode_graphs=False)
+        runner = ModelRunner.from_folder(folder, engine_config, device=device)
+        runner.admit("whole")
+        whole = runner.step([StepEntry("whole", tuple(tokens), tuple(places))]).cpu()
+        runner.release("whole")
+        runner.admit("cut")
+        head_places = [place for place in places if place < prompt_len]
+        rows = [runner.step([StepEntry("cut", tuple(tokens[:prompt_len]), tuple(head_places))]).cpu()]
+        for position in range(prompt_len, prompt_len + tail):
+            rows.append(runner.step([StepEntry("cut", (tokens[position],), (0,))]).cpu())
+        cut = torch.cat(rows)
+        del runner
+        torch.cuda.empty_cache()
+    return {
+        "dtype": "fp32", "layers": layers, "tokens": len(tokens), "compared_positions": len(places),
+        "max_abs_diff": float((whole - exact).abs().max()), "max_abs_logit": float(exact.abs().max()),
+        "decoded_equals_whole_bitwise": bool(torch.equal(whole, cut)),
+    }
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -98,14 +161,14 @@ def main() -> int:
         return 2
     import torch
 
-    from miniserve_amd.config import EngineConfig, Qwen3Config
+    from miniserve_amd.config import EngineConfig, config_dict_from_preset_or_file, config_from_dict
     from miniserve_amd.engine import Engine, ModelRunner, SamplingParams, StepEntry
 
-    sizes = dict(SIZES[args.size])
+    sizes = config_dict_from_preset_or_file(f"qwen3-{args.size}")
     full_layers = sizes["num_hidden_layers"]
     if args.layers is not None:
         sizes["num_hidden_layers"] = args.layers
-    config = Qwen3Config(**sizes)
+    config = config_from_dict(sizes)
     device = "cuda:0"
     itemsize = 2 if args.dtype == "bfloat16" else 4
     generator = torch.Generator().manual_seed(0)
@@ -122,8 +185,15 @@ def main() -> int:
         )
         return ModelRunner.from_random(config, engine_config, seed=0, device=device)
 
+    def thin(samples, keep=16):
+        """At most ``keep`` of the samples, evenly spaced, in milliseconds."""
+
+        stride = max(1, len(samples) // keep)
+        return [round(value, 4) for value in samples[::stride][:keep]]
+
     def decode_rate(batch, steps, warmup):
-        """(tokens a second, ms a step, mean context) of ``steps`` decode steps at ``batch``."""
+        """``steps`` decode steps at ``batch``: tokens a second and ms a step by the wall
+        clock around all of them, the mean context, and the single steps by device events."""
 
         runner = make_runner(batch)
         engine = Engine(runner)
@@ -135,16 +205,24 @@ def main() -> int:
         for _ in range(warmup):
             engine.step()
         start_context = args.prompt_len + 1 + warmup + 1
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
         torch.cuda.synchronize()
         begin = time.perf_counter()
-        for _ in range(steps):
+        for index in range(steps):
+            marks[index].record()
             out = engine.step()
+        marks[steps].record()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - begin
         assert len(out) == batch and engine.last_plan.prefill_items == ()
+        by_device = [marks[index].elapsed_time(marks[index + 1]) for index in range(steps)]
         del engine, runner
         torch.cuda.empty_cache()
-        return batch * steps / elapsed, 1000 * elapsed / steps, start_context + steps / 2
+        device = {"median_ms": round(statistics.median(by_device), 4), "samples_ms": thin(by_device), "steps": steps}
+        return batch * steps / elapsed, 1000 * elapsed / steps, start_context + steps / 2, device
+
+    def step_bytes_of(batch, context, model_bytes, kv_bytes_per_token):
+        return model_bytes + batch * context * kv_bytes_per_token
 
     def mixed_rate(requests, new_tokens, chunk=512):
         """Continuous batching as a server sees it: ``requests`` prompts of 128 to
@@ -165,52 +243,100 @@ def main() -> int:
             decode_graphs=not args.eager,
         )
         runner = ModelRunner.from_random(config, engine_config, seed=0, device=device)
+        model_bytes = weight_bytes(runner.model, itemsize)
+        kv_bytes_per_token = runner.cache.layout.bytes_per_token(itemsize)
         params = SamplingParams(max_new_tokens=new_tokens)
         for prompts in rounds:
             engine = Engine(runner)
             for index, prompt in enumerate(prompts):
                 engine.add_request(f"m{index}", prompt, params, arrival_ns=index)
+            marks, plans = [], []
             torch.cuda.synchronize()
             begin = time.perf_counter()
-            mixed_steps = 0
             while engine.has_unfinished():
+                mark = torch.cuda.Event(enable_timing=True)
+                mark.record()
+                marks.append(mark)
                 engine.step()
-                mixed_steps += bool(engine.last_plan.prefill_items and engine.last_plan.decode_items)
+                plans.append(engine.last_plan)
+            mark = torch.cuda.Event(enable_timing=True)
+            mark.record()
+            marks.append(mark)
             torch.cuda.synchronize()
             elapsed = time.perf_counter() - begin
             counters = dict(engine.counters)
+        # the last round by phase: steps of single tokens only against the HBM peak (their weights once and
+        # the cache they read), steps with prompt portions against the MFMA peak (their products and attention)
+        decode_only = {"steps": 0, "ms": 0.0, "bytes": 0.0}
+        with_prompts = {"steps": 0, "ms": 0.0, "flops": 0.0, "tokens": 0}
+        per_token = per_token_flops(config)
+        for index, plan in enumerate(plans):
+            if plan.empty:
+                continue
+            ms = marks[index].elapsed_time(marks[index + 1])
+            if plan.prefill_items:
+                flops = per_token * plan.scheduled_tokens
+                for item in plan.prefill_items:
+                    keys = item.num_tokens * (item.token_start + (item.num_tokens + 1) / 2)
+                    flops += config.num_hidden_layers * 4 * config.num_attention_heads * config.head_dim * keys
+                for item in plan.decode_items:
+                    flops += config.num_hidden_layers * 4 * config.num_attention_heads * config.head_dim * (item.position + 1)
+                with_prompts["steps"] += 1
+                with_prompts["ms"] += ms
+                with_prompts["flops"] += flops
+                with_prompts["tokens"] += plan.scheduled_tokens
+            else:
+                cache_tokens = sum(item.position + 1 for item in plan.decode_items)
+                decode_only["steps"] += 1
+                decode_only["ms"] += ms
+                decode_only["bytes"] += model_bytes + cache_tokens * kv_bytes_per_token
+        mixed_steps = sum(1 for plan in plans if plan.prefill_items and plan.decode_items)
         del engine, runner
         torch.cuda.empty_cache()
         total = counters["prefill_tokens"] + counters["decode_tokens"]
+        phases = {}
+        if decode_only["steps"]:
+            phases["decode_only"] = {
+                "steps": decode_only["steps"], "ms": round(decode_only["ms"], 1),
+                "frac_hbm": round(decode_only["bytes"] / (decode_only["ms"] / 1000) / 1e9 / HBM_GBPS, 4),
+            }
+        if with_prompts["steps"]:
+            phases["with_prompts"] = {
+                "steps": with_prompts["steps"], "ms": round(with_prompts["ms"], 1), "tokens": with_prompts["tokens"],
+                "frac_mfma": round(with_prompts["flops"] / (with_prompts["ms"] / 1000) / (PEAK_TFLOPS[args.dtype] * 1e12), 4),
+            }
         return {
             "value": round(total / elapsed, 1), "unit": "tokens/s, prompt and generated", "requests": requests,
             "prompt_tokens": counters["prefill_tokens"], "generated_tokens": counters["decode_tokens"] + requests,
             "steps": counters["steps"], "steps_with_both": mixed_steps, "chunk": chunk,
             "token_budget": engine_config.max_num_batched_tokens, "ms": round(1000 * elapsed, 1),
-            "preemptions": counters.get("preemptions", 0),
+            "preemptions": counters.get("preemptions", 0), "phases": phases,
         }
 
-    value, ms_per_step, mean_context = decode_rate(args.batch, args.steps, args.warmup)
+    value, ms_per_step, mean_context, decode_device = decode_rate(args.batch, args.steps, args.warmup)
 
     # ---- roofline of the decode step --------------------------------------------------
     runner = make_runner(1)
     model_bytes = weight_bytes(runner.model, itemsize)
     kv_bytes_per_token = runner.cache.layout.bytes_per_token(itemsize)
-    step_bytes = model_bytes + args.batch * mean_context * kv_bytes_per_token
+    step_bytes = step_bytes_of(args.batch, mean_context, model_bytes, kv_bytes_per_token)
     achieved = step_bytes / (ms_per_step / 1000) / 1e9
 
-    # ---- prefill of one prompt -----------------------------------------------------------
+    # ---- prefill of one prompt: device events, the median of five runs after one uncounted ----
     prompt = random_prompts(1, args.prefill_tokens)[0]
-    times = []
-    for repeat in range(4):
+    prefill_samples = []
+    for repeat in range(6):
         runner.admit("p")
+        before, after = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        begin = time.perf_counter()
+        before.record()
         runner.step([StepEntry("p", tuple(prompt), (len(prompt) - 1,))])
+        after.record()
         torch.cuda.synchronize()
-        times.append(time.perf_counter() - begin)
+        prefill_samples.append(before.elapsed_time(after))
         runner.release("p")
-    prefill_s = statistics.median(times[1:])
+    prefill_samples = prefill_samples[1:]
+    prefill_s = statistics.median(prefill_samples) / 1000
     flops = prefill_flops(config, args.prefill_tokens)
     del runner
     torch.cuda.empty_cache()
@@ -237,11 +363,13 @@ def main() -> int:
     del a, b
     torch.cuda.empty_cache()
 
-    points = {}
+    points, points_frac = {}, {}
     if not args.no_points:
         for batch in (1, 64):
-            rate, _, _ = decode_rate(batch, max(16, args.steps // 4), min(args.warmup, 4))
-            points[f"decode_b{batch}"] = round(rate, 1)
+            point_rate, point_ms, point_context, _ = decode_rate(batch, max(16, args.steps // 4), min(args.warmup, 4))
+            points[f"decode_b{batch}"] = round(point_rate, 1)
+            point_bytes = step_bytes_of(batch, point_context, model_bytes, kv_bytes_per_token)
+            points_frac[f"decode_b{batch}"] = round(point_bytes / (point_ms / 1000) / 1e9 / HBM_GBPS, 4)
     mixed = None
     if not args.no_points:
         mixed = mixed_rate(args.mixed_requests, args.mixed_new_tokens)
@@ -278,10 +406,12 @@ def main() -> int:
             "kv_block_size": 16,
             "decode_graphs": not args.eager,
         },
+        "decode_device": decode_device,
         "prefill": {
             "value": round(args.prefill_tokens / prefill_s, 1),
             "tokens": args.prefill_tokens,
             "ms": round(1000 * prefill_s, 3),
+            "samples_ms": [round(sample, 3) for sample in prefill_samples],
             "frac": round(flops / prefill_s / (PEAK_TFLOPS[args.dtype] * 1e12), 5),
             "frac_of_measured_gemm": round(flops / prefill_s / (gemm_tflops * 1e12), 5),
         },
@@ -294,9 +424,12 @@ def main() -> int:
             "frac_of_measured_copy": round(achieved / copy_gbps, 5),
         },
         "points": points,
+        "points_frac": points_frac,
         "mixed": mixed,
         "measured": {"copy_GBps": round(copy_gbps, 1), "library_gemm_8192_TFLOPs": round(gemm_tflops, 1)},
     }
+    if args.parity:
+        line["parity"] = parity_run(sizes, args.layers if args.layers is not None else 2, device)
     print(json.dumps(line))
     return 0
 

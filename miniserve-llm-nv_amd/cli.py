@@ -2,6 +2,7 @@
 
     python -m miniserve_amd.cli --model DIR --prompt-ids 1,2,3 --max-new-tokens 8
     python -m miniserve_amd.cli --random-weights config.json --seed 0 --prompt-len 32
+    python -m miniserve_amd.cli --random-weights qwen3-0.6b --layers 4 --prompt-len 32
 
 Engine options carry the names of the reference's launcher
 (miniserve/api/server.py:350-397); per-request options the names of its request
@@ -14,15 +15,16 @@ from __future__ import annotations
 import argparse
 import json
 import sys
-import tempfile
-from pathlib import Path
 
 
 def build_cli_parser() -> argparse.ArgumentParser:
     parser = argparse.ArgumentParser(prog="miniserve-generate", description=__doc__.split("\n\n")[0])
     source = parser.add_mutually_exclusive_group(required=True)
     source.add_argument("--model", help="folder with config.json and safetensors")
-    source.add_argument("--random-weights", metavar="CONFIG_JSON", help="a config.json; weights are drawn from --seed")
+    source.add_argument("--random-weights", metavar="PRESET|CONFIG_JSON",
+                        help="layer sizes by name (qwen3-0.6b, qwen3-8b, qwen3-32b) or a config.json; weights are drawn from --seed")
+    parser.add_argument("--layers", type=int, default=None,
+                        help="with --random-weights: this many layers instead of the configuration's own number")
     parser.add_argument("--seed", type=int, default=0, help="seed of the random weights and of sampling")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--max-model-len", type=int, default=None)
@@ -53,20 +55,23 @@ def main(argv: list[str] | None = None) -> int:
     args = parser.parse_args(argv)
     import torch
 
-    from .config import config_from_dict
+    from .config import config_dict_from_preset_or_file, config_from_dict
     from .engine import SamplingParams
     from .entrypoint import LLM
-    from .weights import write_random_model
 
-    scratch = None
     model_dir = args.model
     if args.random_weights:
-        config = config_from_dict(json.loads(Path(args.random_weights).read_text()))
-        scratch = tempfile.TemporaryDirectory()
-        model_dir = str(write_random_model(config, scratch.name, seed=args.seed))
+        try:
+            data = config_dict_from_preset_or_file(args.random_weights)
+        except FileNotFoundError as exc:
+            parser.error(str(exc))
+        if args.layers is not None:
+            data["num_hidden_layers"] = args.layers
+        model_dir = config_from_dict(data)        # a configuration: the weights are drawn on the device
     try:
         llm = LLM(
             model_dir,
+            seed=args.seed,
             dtype=args.dtype,
             max_model_len=args.max_model_len,
             num_kv_blocks=args.num_kv_blocks,
@@ -100,8 +105,6 @@ def main(argv: list[str] | None = None) -> int:
     ]
     for prompt, tokens in zip(prompts, llm.generate(prompts, params)):
         print(json.dumps({"prompt_token_ids": prompt, "token_ids": tokens}))
-    if scratch is not None:
-        scratch.cleanup()
     return 0
 
 

@@ -1,7 +1,14 @@
 from .engine_config import DTYPES, EngineConfig
 from .fields import ConfigError
 from .model_spec import LayerCall, LayerSpec, ModelSpec, PartSpec
-from .registry import config_from_dict, load_config, register_architecture, registered_architectures
+from .registry import (
+    config_dict_from_preset_or_file,
+    config_from_dict,
+    load_config,
+    preset_names,
+    register_architecture,
+    registered_architectures,
+)
 from .qwen3 import Qwen3Config
 
 __all__ = [
@@ -13,8 +20,10 @@ __all__ = [
     "ModelSpec",
     "PartSpec",
     "Qwen3Config",
+    "config_dict_from_preset_or_file",
     "config_from_dict",
     "load_config",
+    "preset_names",
     "register_architecture",
     "registered_architectures",
 ]

@@ -61,3 +61,29 @@ def load_config(model_dir: str | Path) -> ArchitectureConfig:
     if not isinstance(data, dict):
         raise ConfigError("config.json must hold a JSON object.")
     return config_from_dict(data)
+
+
+PRESET_DIR = Path(__file__).resolve().parent / "presets"
+
+
+def preset_names() -> tuple[str, ...]:
+    """Names of the ``config.json`` files that ship with the package: the layer sizes
+    of served models, for runs with random weights."""
+
+    return tuple(sorted(path.stem for path in PRESET_DIR.glob("*.json")))
+
+
+def config_dict_from_preset_or_file(name_or_path: str) -> dict[str, Any]:
+    """The ``config.json`` mapping of a preset (by name, any case) or of a file."""
+
+    path = Path(name_or_path)
+    if not path.is_file():
+        path = PRESET_DIR / f"{name_or_path.lower()}.json"
+        if not path.is_file():
+            raise FileNotFoundError(
+                f"{name_or_path!r} is neither a config.json nor one of the presets {', '.join(preset_names())}."
+            )
+    data = json.loads(path.read_text(encoding="utf-8"))
+    if not isinstance(data, dict):
+        raise ConfigError(f"{path} must hold a JSON object.")
+    return data

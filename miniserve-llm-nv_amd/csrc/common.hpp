@@ -5,21 +5,7 @@
 #include <stdint.h>
 
 // Occupancy hint for a kernel: the register budget is set for `lo`..`hi` waves per SIMD.
-#ifndef MS_WAVES_PER_EU
 #define MS_WAVES_PER_EU(lo, hi) __attribute__((amdgpu_waves_per_eu(lo, hi)))
-#endif
-
-#ifndef MS_FAST_EXP2
-#define MS_FAST_EXP2(x) __builtin_amdgcn_exp2f(x)
-#define MS_UNIFORM(v) __builtin_amdgcn_readfirstlane(v)
-#endif
-
-// max of a value with that of the lane 32 further (or back): one swap of the wave's
-// halves on gfx950 instead of a trip through the LDS crossbar.
-#ifndef MS_MAX_XOR32
-#define MS_MAX_XOR32(v) ms::max_swap32(v)
-#define MS_HAS_SWAP32 1
-#endif
 
 namespace ms {
 
@@ -64,25 +50,25 @@ __device__ __forceinline__ float round_to(float v) {
   return to_float(from_float<T>(v));
 }
 
-#ifdef MS_HAS_SWAP32
+// max of a value with that of the lane 32 further (or back): one swap of the wave's
+// halves on gfx950 instead of a trip through the LDS crossbar.
 __device__ __forceinline__ float max_swap32(float v) {
   const auto halves = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   return fmaxf(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
 }
-#endif
 
 // 2^x by the hardware instruction alone (no handling of results below the smallest
 // normal number, which are zero weights anyway).
-__device__ __forceinline__ float fast_exp2(float x) { return MS_FAST_EXP2(x); }
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // A value that is the same in every lane of the wave, moved to a scalar register so
 // that what is computed from it is scalar work and branches on it are scalar branches.
-__device__ __forceinline__ int uniform(int v) { return MS_UNIFORM(v); }
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // Butterfly reductions over the 64 lanes of a wave; every lane gets the result
 // and the order of additions is fixed, so a row's result never depends on what
 // else is in the launch.
-__device__ __forceinline__ float max_xor32(float v) { return MS_MAX_XOR32(v); }
+__device__ __forceinline__ float max_xor32(float v) { return max_swap32(v); }
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -10,6 +10,7 @@ as it does in the reference (miniserve/api/adapter.py:73-80).
 
 from __future__ import annotations
 
+import os
 from typing import Sequence
 
 from .config import EngineConfig
@@ -19,7 +20,7 @@ from .engine import Engine, ModelRunner, SamplingParams
 class LLM:
     def __init__(
         self,
-        model: str,
+        model,
         *,
         dtype: str = "bfloat16",
         max_model_len: int | None = None,
@@ -32,6 +33,7 @@ class LLM:
         prefill_chunk_size: int | None = None,
         decode_graphs: bool = True,
         device: str = "cuda:0",
+        seed: int = 0,
     ) -> None:
         self.engine_config = EngineConfig(
             dtype=dtype,
@@ -45,8 +47,20 @@ class LLM:
             max_pending_requests=max_pending_requests,
             decode_graphs=decode_graphs,
         )
-        self.runner = ModelRunner.from_folder(model, self.engine_config, device=device)
+        if isinstance(model, (str, os.PathLike)):
+            self.runner = ModelRunner.from_folder(model, self.engine_config, device=device)
+        else:
+            # a configuration object: random weights, drawn on the device from ``seed``
+            self.runner = ModelRunner.from_random(model, self.engine_config, seed=seed, device=device)
         self.engine = Engine(self.runner)
+
+    @classmethod
+    def from_random(cls, config, *, seed: int = 0, **options) -> "LLM":
+        """An engine over random weights of ``config`` (a configuration object of a
+        registered architecture), drawn on the device: for sizes that should not
+        pass through a file.  ``options`` as for the constructor."""
+
+        return cls(config, seed=seed, **options)
 
     def generate(
         self,

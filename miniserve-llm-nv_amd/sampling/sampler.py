@@ -68,15 +68,15 @@ class Sampler:
         from .. import ops
 
         if logits.ndim != 2 or logits.shape[0] != len(requests) or logits.shape[1] == 0:
-            raise ValueError("logits must have shape [requests, vocab].")
+            raise ValueError(f"{len(requests)} requests need logits [{len(requests)}, vocab], not {tuple(logits.shape)}.")
         if not logits.is_floating_point():
-            raise TypeError("logits must use a floating-point dtype.")
+            raise TypeError(f"logits are floating-point numbers, not {logits.dtype}.")
         vocab = logits.shape[1]
         states: list[torch.Tensor | None] = []
         uniforms: list[float] = []
         for request_id, params in requests:
             if params.top_k > vocab:
-                raise ValueError("top_k must not exceed the vocabulary size.")
+                raise ValueError(f"request {request_id!r}: top_k {params.top_k} is more than the {vocab} tokens of the vocabulary.")
             if params.temperature == 0:
                 states.append(None)
                 uniforms.append(0.0)
@@ -110,7 +110,7 @@ class Sampler:
         tokens, requests, states = launched
         token_ids = tokens.tolist()
         if any(token < 0 for token in token_ids):
-            raise NonFiniteLogitsError("logits must contain only finite values.")
+            raise NonFiniteLogitsError("a row of logits holds a value that is not finite; no token can be chosen from it.")
         return tuple(
             StagedSample(request_id, int(token), state)
             for (request_id, _), token, state in zip(requests, token_ids, states)

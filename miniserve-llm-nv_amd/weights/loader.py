@@ -10,6 +10,7 @@ must equal the embedding bit for bit.  All findings are reported in ONE error.
 from __future__ import annotations
 
 import json
+import re
 from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Sequence
@@ -127,6 +128,13 @@ def load_weights(
         for name, spec in wanted.items()
         if name in shapes and shapes[name] != tuple(spec.shape)
     )
+    # An unexpected tensor of a layer that the model does not have most often means a
+    # checkpoint of a deeper model; it gets a line of its own (reference: weight_map.py:49-59).
+    layer_of = re.compile(r"(?:^|\.)layers\.(\d+)\.")
+    depth = 1 + max((int(found.group(1)) for found in map(layer_of.search, wanted) if found), default=-1)
+    beyond = sorted({int(found.group(1)) for found in map(layer_of.search, unexpected) if found and int(found.group(1)) >= depth})
+    if depth > 0 and beyond:
+        other.append(f"tensors of layers {beyond} are stored, the model has layers 0..{depth - 1}")
     if missing or unexpected or wrong_shape or other:
         raise WeightLoadError(missing, unexpected, wrong_shape, other)
 

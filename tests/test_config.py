@@ -154,3 +154,20 @@ def test_engine_config_rules():
             EngineConfig(**{name: value}).validate(max_positions=512)
     assert EngineConfig().resolved_max_num_batched_tokens(512) == 512
     assert EngineConfig().resolved_max_num_batched_tokens(40960) == 4096
+
+
+def test_presets_are_config_files_of_registered_architectures(tmp_path):
+    from miniserve_amd.config import config_dict_from_preset_or_file, config_from_dict, preset_names
+
+    assert preset_names() == ("qwen3-0.6b", "qwen3-32b", "qwen3-8b")
+    for name in preset_names():
+        config = config_from_dict(config_dict_from_preset_or_file(name.upper()))       # names in any case
+        spec = config.model_spec()
+        assert spec.vocab_size == 151936 and len(spec.layers) == config.num_hidden_layers
+    small = config_from_dict(config_dict_from_preset_or_file("qwen3-0.6b"))
+    assert (small.hidden_size, small.num_attention_heads, small.num_key_value_heads, small.tie_word_embeddings) == (1024, 16, 8, True)
+    path = tmp_path / "config.json"
+    path.write_text(json.dumps({**config_dict_from_preset_or_file("qwen3-8b"), "num_hidden_layers": 3}))
+    assert config_from_dict(config_dict_from_preset_or_file(str(path))).num_hidden_layers == 3
+    with pytest.raises(FileNotFoundError, match="neither a config.json nor one of the presets"):
+        config_dict_from_preset_or_file("qwen3-7b")

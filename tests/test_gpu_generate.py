@@ -39,7 +39,7 @@ def check_greedy(got, prompt, weights, config, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_tiny_a(dtype, model_folders):
-    """BASELINE configuration Tiny A: prompts of 5, 17 and 33 tokens, 8 greedy tokens each."""
+    """The first tiny configuration: prompts of 5, 17 and 33 tokens, 8 greedy tokens each."""
 
     from miniserve_amd.engine import SamplingParams
     from miniserve_amd.entrypoint import LLM
@@ -84,7 +84,7 @@ def test_greedy_generation_with_wide_heads_through_recorded_steps(model_folders)
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_chunked_prefill_mixed_with_decode_tiny_b(dtype, model_folders):
-    """BASELINE configuration Tiny B: prompts of 1, 9, 24 and 40 tokens, portions of
+    """The second tiny configuration: prompts of 1, 9, 24 and 40 tokens, portions of
     7 mixed with decoding; greedy, then temperature 0.8 from seed 0."""
 
     from miniserve_amd.engine import SamplingParams
@@ -232,6 +232,30 @@ def test_command_line(model_folders):
     assert [line["prompt_token_ids"] for line in lines] == [[5, 9, 200, 31], [7]]
     for line in lines:
         assert check_greedy(line["token_ids"], line["prompt_token_ids"], weights, config, "float32") == 5
+
+
+def test_command_line_with_layer_sizes_by_name():
+    """Random weights of a named size (fewer layers, so that it takes seconds): the same
+    seed gives the same tokens, another seed other weights and other tokens."""
+
+    def run(seed):
+        process = subprocess.run(
+            [sys.executable, str(ROOT / "bin" / "miniserve-generate"), "--random-weights", "qwen3-0.6B", "--layers", "2",
+             "--seed", str(seed), "--max-model-len", "256", "--num-kv-blocks", "32", "--prompt-ids", "5,9,200,31",
+             "--max-new-tokens", "6"],
+            capture_output=True, text=True, timeout=300,
+        )
+        assert process.returncode == 0, process.stderr[-2000:]
+        return json.loads(process.stdout.strip().splitlines()[-1])["token_ids"]
+
+    first = run(3)
+    assert len(first) == 6 and all(0 <= token < 151936 for token in first)
+    assert run(3) == first and run(4) != first
+    process = subprocess.run(
+        [sys.executable, str(ROOT / "bin" / "miniserve-generate"), "--random-weights", "qwen3-7b", "--prompt-len", "4"],
+        capture_output=True, text=True, timeout=300,
+    )
+    assert process.returncode != 0 and "qwen3-0.6b, qwen3-32b, qwen3-8b" in process.stderr
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -66,6 +66,29 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     text = str(error)
     for needle in ("missing tensors (2)", "unexpected tensors (2)", "(16, 64)", "(32, 64)", "surprise.bias"):
         assert needle in text
+    # a tensor of a layer that the model does not have is named as such (a checkpoint of a deeper model)
+    assert "tensors of layers [7] are stored, the model has layers 0..1" in text
+
+
+def test_init_rules_are_open(tmp_path):
+    """A part names a rule that another package registered, or brings a callable."""
+
+    from miniserve_amd.parts import WeightSpec
+    from miniserve_amd.weights import register_init
+
+    register_init("test_ones", lambda shape, generator, device: torch.ones(shape, dtype=torch.float32, device=device))
+    specs = [
+        WeightSpec("a", (2, 3), init="test_ones"),
+        WeightSpec("b", (4,), init=lambda shape, generator, device: torch.full(shape, 7.0, device=device)),
+        WeightSpec("c", (2, 2)),
+    ]
+    drawn = random_tensors(specs, seed=1)
+    assert torch.equal(drawn["a"], torch.ones(2, 3)) and torch.equal(drawn["b"], torch.full((4,), 7.0))
+    assert 0 < float(drawn["c"].abs().max()) < 0.2
+    with pytest.raises(ValueError, match="unknown init rule"):
+        random_tensors([WeightSpec("d", (1,), init="nobody")], seed=1)
+    with pytest.raises(ValueError, match="float32 tensor of shape"):
+        random_tensors([WeightSpec("e", (2,), init=lambda shape, generator, device: torch.zeros(3))], seed=1)
 
 
 def test_tied_head_in_the_file_must_equal_the_embedding(tmp_path):
