@@ -11,6 +11,12 @@
 // summed through LDS in a fixed order; every output element is written by one
 // workgroup: results do not depend on anything but their own row of x and of W.
 //
+// With more than 16 rows of x and a matrix of few rows the launch is cut along M as well
+// (blockIdx.y): a workgroup takes 16 rows of x against its rows of W, so that what it
+// reads of x (from the caches) stays near what it streams of W; the workgroups that
+// share rows of W stand 'gridDim.x' apart in the launch order, which puts them on the
+// same die and lets all but the first find those rows in its cache.
+//
 // Epilogues (what the reference does in separate torch calls):
 //   0  out = bf16(C)                                   nn.Linear (qwen3.py:174-176)
 //   1  out_f32 = C                                     logits (qwen3.py:558)
@@ -80,11 +86,12 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     const int row = local + (epilogue == kSiluMul && rb >= RB / 2 ? half : 0);
     w_row[rb] = w + static_cast<int64_t>(row) * k;
   }
+  const int m_base = blockIdx.y * (16 * MB);      // the workgroup's first row of x
   const bf16* x_row[MB];
   bool x_live[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    const int row = 16 * mb + r;
+    const int row = m_base + 16 * mb + r;
     x_live[mb] = row < m;
     x_row[mb] = NORM ? nullptr : x + static_cast<int64_t>(min(row, m - 1)) * k;
   }
@@ -102,7 +109,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
   if (epilogue == kAddF32 && threadIdx.x < RB * MB * 256) {
     const int n_local = threadIdx.x & 15, m_local = (threadIdx.x >> 4) & 15, tile = threadIdx.x >> 8;
     const int rb = tile / MB, mb = tile - rb * MB;
-    const int row_m = 16 * mb + m_local, col_n = row_start[rb] + n_local;
+    const int row_m = m_base + 16 * mb + m_local, col_n = row_start[rb] + n_local;
     if (row_m < m && col_n < row_limit && n_local < rows) residual_ahead = out_f32[static_cast<int64_t>(row_m) * n + col_n];
   }
 
@@ -173,7 +180,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     const int m_local = (index >> 4) & 15;
     const int tile = index >> 8;
     const int rb = tile / MB, mb = tile - rb * MB;
-    const int row_m = 16 * mb + m_local;
+    const int row_m = m_base + 16 * mb + m_local;
     const int col_n = row_start[rb] + n_local;
     if (row_m >= m || col_n >= row_limit || n_local >= rows) continue;
     float sum = 0.f;
@@ -211,21 +218,22 @@ void launch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, 
             hipStream_t stream, const void* h = nullptr, const void* norm_weight = nullptr, float eps = 0.f) {
   const int out_rows = epilogue == kSiluMul ? n / 2 : n;
   const int blocks_per_group = epilogue == kSiluMul ? RB / 2 : RB;
+  const int m_tiles = (m + 16 * MB - 1) / (16 * MB);
   // A matrix of few rows gives 8 or 4 rows instead of 16 to a workgroup: one workgroup
   // streams less, and there are 256 compute units to feed.
   int rows = 16;
   if (RB == 1 && epilogue != kSiluMul) {
-    while (rows > 4 && (out_rows + rows - 1) / rows < 256) rows /= 2;
+    while (rows > 4 && ((out_rows + rows - 1) / rows) * m_tiles < 256) rows /= 2;
   }
   const int groups = (out_rows + rows * blocks_per_group - 1) / (rows * blocks_per_group);
   // rows of 2048 elements and more: eight k-steps in flight a wave (where the registers allow it)
   if (k >= 2048 && MB * RB <= 2) {
-    hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 8>), dim3(groups), dim3(kGroupThreads), 0, stream,
+    hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 8>), dim3(groups, m_tiles), dim3(kGroupThreads), 0, stream,
                        static_cast<const bf16*>(x), static_cast<const float*>(h),
                        static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
                        static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue, rows);
   } else {
-    hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 4>), dim3(groups), dim3(kGroupThreads), 0, stream,
+    hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 4>), dim3(groups, m_tiles), dim3(kGroupThreads), 0, stream,
                        static_cast<const bf16*>(x), static_cast<const float*>(h),
                        static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
                        static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue, rows);
@@ -250,14 +258,20 @@ extern "C" int ms_gemm_skinny(const void* x, const void* w, void* out_bf16, void
   MS_REQUIRE((epilogue == kStoreBf16 || epilogue == kSiluMul) ? out_bf16 != nullptr : out_f32 != nullptr,
              "gemm_skinny: the output of epilogue %d is null", epilogue);
   const int mb = (m + 15) / 16;
-  const bool many_rows = (epilogue == kSiluMul ? n / 2 : n) >= 32768;   // the head: larger tiles, fewer workgroups
-  if (epilogue == kSiluMul) {
-    if (mb == 1) launch<1, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-    else if (mb == 2) launch<2, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-    else launch<4, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-  } else if (mb == 1) {
-    if (many_rows) launch<1, 4>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+  const int out_rows = epilogue == kSiluMul ? n / 2 : n;
+  const bool many_rows = out_rows >= 32768;   // the head: larger tiles, fewer workgroups
+  if (mb == 1) {
+    if (epilogue == kSiluMul) launch<1, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+    else if (many_rows) launch<1, 4>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
     else launch<1, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+  } else if (out_rows <= 2048 && epilogue != kSiluMul) {
+    // More than 16 rows against a matrix of few rows: a workgroup that took all rows of x
+    // would read far more of x than of W.  The launch is cut along M too: 16 rows of x
+    // against 16 (or fewer) rows of W a workgroup.
+    launch<1, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+  } else if (epilogue == kSiluMul) {
+    if (mb == 2) launch<2, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
+    else launch<4, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
   } else if (mb == 2) {
     if (many_rows) launch<2, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
     else launch<2, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);

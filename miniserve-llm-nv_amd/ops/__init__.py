@@ -465,7 +465,7 @@ def prefers_skinny(m: int, n: int, k: int, *, fused: bool = False) -> bool:
         return _forced_product == "skinny"
     size = 2 * n * k
     if size <= 16 * _MIB:                       # the matrices of a small model
-        return m <= (64 if n >= 2048 else 32)
+        return True
     if m > SKINNY_MAX_ROWS:
         return False
     if size <= 40 * _MIB or k >= 16384:         # middle sizes; very long rows, which the library splits badly

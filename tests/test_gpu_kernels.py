@@ -438,6 +438,24 @@ def test_tiled_kernel_sizes_portions_and_windows(ops, heads, kv_heads, dim, bloc
         torch.testing.assert_close(out.cpu().double(), expected, atol=ATTENTION_BF16, rtol=ATTENTION_BF16, msg=lambda m: f"window {window}: {m}")
 
 
+@pytest.mark.parametrize("contexts,query_lens,heads,kv_heads,dim", [
+    ([2048], [2048], 16, 8, 128),                 # a prompt of the served sizes: 32 tiles, the last walks 2,048 keys
+    ([1100, 1200], [1100, 1200], 32, 8, 64),      # two prompts, two workgroups of heads to a kv head
+    ([700, 300, 40], [500, 33, 40], 4, 1, 32),    # portions with history, an odd tail
+    ([1500] * 3, [1000] * 3, 4, 4, 48),           # one head a workgroup
+])
+def test_tiled_kernel_over_long_prompts(ops, contexts, query_lens, heads, kv_heads, dim):
+    """Prompts of a thousand tokens and more (dozens of tiles, walks of thousands of
+    keys), against the plain attention, with a window as well."""
+
+    case = paged_case(contexts, heads, kv_heads, dim, 16, torch.bfloat16, query_lens=query_lens, seed=dim)
+    for window in (None, 300):
+        out = run_attention(ops, case, dim**-0.5, window=window)
+        expected = attention_reference(case, dim**-0.5, window=window)
+        torch.testing.assert_close(out.cpu().double(), expected, atol=ATTENTION_BF16, rtol=ATTENTION_BF16,
+                                   msg=lambda m: f"window {window}: {m}")
+
+
 def test_tiled_kernel_ignores_stale_values(ops):
     case = paged_case([37, 70], 8, 2, 64, 16, torch.bfloat16, query_lens=[20, 70], seed=4)   # unused slots hold NaN
     assert torch.isnan(case["value_pool"]).any()

@@ -15,7 +15,7 @@ def test_the_rule_for_the_two_products():
     for n, k in small.values():
         assert ops.prefers_skinny(1, n, k) and ops.prefers_skinny(16, n, k) and ops.prefers_skinny(32, n, k)
         assert not ops.prefers_skinny(65, n, k)
-    assert ops.prefers_skinny(64, *small["qkv"]) and not ops.prefers_skinny(64, *small["down"])
+    assert ops.prefers_skinny(64, *small["qkv"]) and ops.prefers_skinny(64, *small["down"])
     assert ops.prefers_skinny(8, 151936, 1024) and not ops.prefers_skinny(16, 151936, 1024)      # the head
     assert ops.prefers_skinny(16, 4096, 4096) and not ops.prefers_skinny(17, 4096, 4096)         # 32 MiB
     assert not ops.prefers_skinny(8, 24576, 4096) and ops.prefers_skinny(8, 24576, 4096, fused=True)
@@ -26,13 +26,13 @@ def test_the_rule_for_the_two_products():
 def test_a_forced_product_overrides_the_rule_and_is_undone():
     from miniserve_amd import ops
 
-    assert not ops.prefers_skinny(64, 1024, 3072)
+    assert not ops.prefers_skinny(64, 4096, 4096)
     with ops.forced_product("skinny"):
-        assert ops.prefers_skinny(64, 1024, 3072) and not ops.prefers_skinny(65, 1024, 3072)
+        assert ops.prefers_skinny(64, 4096, 4096) and not ops.prefers_skinny(65, 4096, 4096)
         with ops.forced_product("library"):
             assert not ops.prefers_skinny(1, 4096, 1024)
-        assert ops.prefers_skinny(64, 1024, 3072)
-    assert not ops.prefers_skinny(64, 1024, 3072) and ops.prefers_skinny(1, 4096, 1024)
+        assert ops.prefers_skinny(64, 4096, 4096)
+    assert not ops.prefers_skinny(64, 4096, 4096) and ops.prefers_skinny(1, 4096, 1024)
     with pytest.raises(ValueError):
         with ops.forced_product("fastest"):
             pass
