@@ -29,15 +29,16 @@ class CacheError(RuntimeError):
 
 @dataclass(frozen=True)
 class CapacitySnapshot:
-    """What the scheduler may know: numbers only (reference: miniserve/kv/base.py:14-36)."""
+    """What the scheduler may know: numbers only (reference: miniserve/kv/base.py:14-36).
+    Everything is per cache group; a group has its own page size."""
 
-    block_size: int
-    total_blocks: tuple[int, ...]      # per group
-    free_blocks: tuple[int, ...]       # per group
+    block_sizes: tuple[int, ...]       # tokens a page holds
+    total_blocks: tuple[int, ...]
+    free_blocks: tuple[int, ...]
     free_slots: int
     total_slots: int
-    held_blocks: Mapping[str, tuple[int, ...]] = field(default_factory=dict)   # per live request, per group
-    windows: tuple[int | None, ...] = ()   # per group: the window of its layers, None = all keys are kept
+    held_blocks: Mapping[str, tuple[int, ...]] = field(default_factory=dict)   # per live request
+    windows: tuple[int | None, ...] = ()   # the window of the group's layers, None = all keys are kept
 
     def most_pages_held(self, total_tokens: int, step_tokens: int) -> tuple[int, ...]:
         """The most pages of each group that one request of ``total_tokens`` holds at any
@@ -46,21 +47,31 @@ class CapacitySnapshot:
         step's first token still sees to the step's last token (an edge page more, since
         that span may begin anywhere inside a page)."""
 
-        whole = -(-total_tokens // self.block_size)
         windows = self.windows or (None,) * len(self.total_blocks)
         held = []
-        for window in windows:
+        for block_size, window in zip(self.block_sizes, windows):
+            whole = -(-total_tokens // block_size)
             if window is None:
                 held.append(whole)
             else:
                 span = min(total_tokens, window - 1 + min(step_tokens, total_tokens))
-                held.append(min(whole, -(-span // self.block_size) + 1))
+                held.append(min(whole, -(-span // block_size) + 1))
         return tuple(held)
 
-    def pages_for(self, before: int, after: int) -> int:
-        """New pages that growing a request from ``before`` to ``after`` tokens takes in every group."""
+    def pages_for(self, before: int, after: int) -> tuple[int, ...]:
+        """New pages of each group that growing a request from ``before`` to ``after`` tokens takes."""
 
-        return -(-after // self.block_size) - -(-before // self.block_size)
+        return tuple(-(-after // size) - -(-before // size) for size in self.block_sizes)
+
+    def room_for(self, before: int, free_pages: Sequence[int]) -> int:
+        """Tokens that a request of ``before`` tokens can grow by with ``free_pages``
+        new pages per group: the rest of its last page and the free pages, in the
+        group where that is least."""
+
+        return min(
+            ((-before) % size + max(free, 0) * size for size, free in zip(self.block_sizes, free_pages)),
+            default=1 << 60,
+        )
 
     @property
     def min_free_blocks(self) -> int:
@@ -118,8 +129,17 @@ class CacheManager:
         if block_size <= 0 or max_num_seqs <= 0 or max_model_len <= 0:
             raise ValueError("block_size, max_num_seqs and max_model_len must be positive.")
         self.layout = layout
-        self.block_size = block_size
-        counts = [num_blocks] * len(layout.groups) if isinstance(num_blocks, int) else list(num_blocks)
+        self.block_size = block_size          # the engine's page size; a group's need may name its own
+        self.block_sizes = tuple(
+            block_size if group.need.block_size is None else group.need.block_size for group in layout.groups
+        )
+        if any(type(size) is not int or size <= 0 for size in self.block_sizes):
+            raise ValueError(f"page sizes must be positive whole numbers, not {self.block_sizes}.")
+        if isinstance(num_blocks, int):
+            # one number: pages of the engine's size; a group with pages of its own size gets as many tokens
+            counts = [max(1, num_blocks * block_size // size) for size in self.block_sizes]
+        else:
+            counts = list(num_blocks)
         if len(counts) != len(layout.groups):
             raise ValueError("num_blocks must give one count per cache group.")
         self.num_blocks = tuple(counts)
@@ -150,14 +170,10 @@ class CacheManager:
         import torch
 
         self.key_pools, self.value_pools, self.state_tensors = [], [], []
-        for group, count in zip(self.layout.groups, self.num_blocks):
+        for group, count, page in zip(self.layout.groups, self.num_blocks, self.block_sizes):
             heads, dim = group.need.num_kv_heads, group.need.head_dim
-            self.key_pools.append(
-                torch.empty((len(group.calls), count + 1, heads, self.block_size, dim), dtype=dtype, device=device)
-            )
-            self.value_pools.append(
-                torch.empty((len(group.calls), count + 1, heads, dim, self.block_size), dtype=dtype, device=device)
-            )
+            self.key_pools.append(torch.empty((len(group.calls), count + 1, heads, page, dim), dtype=dtype, device=device))
+            self.value_pools.append(torch.empty((len(group.calls), count + 1, heads, dim, page), dtype=dtype, device=device))
         for need in self.layout.states:
             self.state_tensors.append(torch.zeros((self.max_num_seqs + 1, *need.shape), dtype=need.dtype, device=device))
 
@@ -183,7 +199,7 @@ class CacheManager:
                         group=placement.group,
                         key=self.key_pools[placement.group][placement.index],
                         value=self.value_pools[placement.group][placement.index],
-                        block_size=self.block_size,
+                        block_size=self.block_sizes[placement.group],
                         write=placement.write,
                     )
                 )
@@ -203,7 +219,7 @@ class CacheManager:
             raise CacheError("NO_FREE_SLOT: every state slot is taken.")
         slot = self._free_slots.pop()
         self._live[request_id] = _Live(
-            request_id, slot, tables=[BlockTable(self.block_size) for _ in self.layout.groups]
+            request_id, slot, tables=[BlockTable(size) for size in self.block_sizes]
         )
         for tensor in self.state_tensors:
             tensor[slot].zero_()
@@ -271,7 +287,7 @@ class CacheManager:
                     taken.append((index, new_pages))
                     # without a new page the step reads the table's own snapshot, made once per change
                     tentative = tuple(table.pages + new_pages) if new_pages else table.snapshot()
-                    block_size = self.block_size
+                    block_size = self.block_sizes[index]
                     if item.end == item.start + 1:
                         logical, offset = divmod(item.start, block_size)
                         slots = (tentative[logical] * block_size + offset,)
@@ -360,7 +376,7 @@ class CacheManager:
     # ---- accounting -------------------------------------------------------------------
     def capacity(self) -> CapacitySnapshot:
         return CapacitySnapshot(
-            block_size=self.block_size,
+            block_sizes=self.block_sizes,
             total_blocks=self.num_blocks,
             free_blocks=tuple(allocator.free_count() for allocator in self.allocators),
             free_slots=len(self._free_slots),

@@ -76,7 +76,7 @@ def build_step(
     entries: Sequence[StepEntry],
     reservation: StepReservation,
     *,
-    block_size: int,
+    block_sizes: Sequence[int],
     pool_pages: Sequence[int],
     vocab_size: int,
     device: torch.device | str,
@@ -156,8 +156,9 @@ def build_step(
             token_ids[base] = token
             positions[base] = meta.before
             seq_of_token[base] = index
-            logical, offset = divmod(meta.before, block_size)
             for group in range(num_groups):
+                block_size = block_sizes[group]
+                logical, offset = divmod(meta.before, block_size)
                 table = meta.block_tables[group]
                 slot = meta.slot_mappings[group][0]
                 page = table[logical]
@@ -175,8 +176,9 @@ def build_step(
         run = np.arange(meta.before, meta.after, dtype=np.int64)
         positions[base : base + length] = run
         seq_of_token[base : base + length] = index
-        logical, offset = np.divmod(run, block_size)
         for group in range(num_groups):
+            block_size = block_sizes[group]
+            logical, offset = np.divmod(run, block_size)
             table = np.asarray(meta.block_tables[group], dtype=np.int64)
             slots = np.asarray(meta.slot_mappings[group], dtype=np.int64)
             pages = table[logical]

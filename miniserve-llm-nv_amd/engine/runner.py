@@ -67,11 +67,11 @@ class DecodeGraph:
         # and not at some later collection of cycles
         self._runner = weakref.ref(runner)
         groups = len(runner.cache.layout.groups)
-        width = runner.max_blocks_per_seq
+        widths = runner.max_blocks_per_seq          # per group: pages of the longest request the engine admits
         sizes = [("token_ids", batch), ("positions", batch), ("seq_of_token", batch), ("query_start", batch + 1),
                  ("context_lens", batch), ("state_slots", batch), ("logit_rows", batch)]
         for group in range(groups):
-            sizes += [(f"slots{group}", batch), (f"table{group}", batch * width)]
+            sizes += [(f"slots{group}", batch), (f"table{group}", batch * widths[group])]
         self.offsets: dict[str, tuple[int, int]] = {}
         total = 0
         for name, size in sizes:
@@ -83,7 +83,7 @@ class DecodeGraph:
         self.hosts_np = [host.numpy() for host in self.hosts]
         self._turn = 0
         self.meta = torch.zeros(total, dtype=torch.int32, device=runner.device)
-        self.width = width
+        self.widths = widths
         view = lambda name: self.meta[self.offsets[name][0] : self.offsets[name][0] + self.offsets[name][1]]
         self.ctx = StepContext(
             num_tokens=batch,
@@ -95,7 +95,7 @@ class DecodeGraph:
             context_lens=view("context_lens"),
             state_slots=view("state_slots"),
             groups=[
-                GroupStepView(block_table=view(f"table{g}").view(batch, width), slot_mapping=view(f"slots{g}"))
+                GroupStepView(block_table=view(f"table{g}").view(batch, widths[g]), slot_mapping=view(f"slots{g}"))
                 for g in range(groups)
             ],
             # what holds for every replay: one token a row.  Launch decisions inside the
@@ -125,7 +125,7 @@ class DecodeGraph:
     def _fill(self, reservation, which: int) -> None:
         """Everything of the step but its token ids, into host buffer ``which``."""
 
-        host, offsets, batch, width = self.hosts_np[which], self.offsets, self.batch, self.width
+        host, offsets, batch = self.hosts_np[which], self.offsets, self.batch
 
         def put(name: str, values) -> None:
             start, size = offsets[name]
@@ -136,7 +136,6 @@ class DecodeGraph:
         if spare < 0:
             raise ValueError(f"{len(metas)} requests do not fit a recorded step of {batch}.")
         runner = self._runner()
-        block_size = runner.block_size
         put("positions", [meta.before for meta in metas] + [0] * spare)
         put("seq_of_token", range(batch))
         put("query_start", range(batch + 1))
@@ -145,6 +144,7 @@ class DecodeGraph:
         put("logit_rows", range(batch))
         for group in range(len(runner.cache.layout.groups)):
             pool_pages = runner.cache.num_blocks[group]
+            block_size, width = runner.cache.block_sizes[group], self.widths[group]
             slots = []
             start, _ = offsets[f"table{group}"]
             row_tables = self._row_tables[which][group]
@@ -280,7 +280,7 @@ class ModelRunner:
         )
         self.cache.allocate_storage(self.dtype, self.device)
         self._call_views = self.cache.call_views()
-        self.max_blocks_per_seq = -(-self.max_model_len // self.block_size)
+        self.max_blocks_per_seq = tuple(-(-self.max_model_len // size) for size in self.cache.block_sizes)
         self._decode_graphs: dict[int, DecodeGraph] = {}
         self._graph_pool = None
         self.steps_run = 0
@@ -402,7 +402,7 @@ class ModelRunner:
             reservation = self._open_step(entries)
             try:
                 built = build_step(
-                    entries, reservation, block_size=self.block_size, pool_pages=self.cache.num_blocks,
+                    entries, reservation, block_sizes=self.cache.block_sizes, pool_pages=self.cache.num_blocks,
                     vocab_size=self.spec.vocab_size, device=self.device, step_tables=self.model.step_tables,
                 )
             except BaseException:
@@ -466,7 +466,7 @@ class ModelRunner:
             built = build_step(
                 entries,
                 reservation,
-                block_size=self.block_size,
+                block_sizes=self.cache.block_sizes,
                 pool_pages=self.cache.num_blocks,
                 vocab_size=self.spec.vocab_size,
                 device=self.device,

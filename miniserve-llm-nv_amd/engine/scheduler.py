@@ -43,15 +43,15 @@ class _Ledger:
         self.preempted: list[str] = []
         self.planned: set[str] = set()
 
-    def holds(self, pages: int) -> bool:
-        return all(pages <= free for free in self.free_pages)
+    def holds(self, pages: Sequence[int]) -> bool:
+        return all(wanted <= free for wanted, free in zip(pages, self.free_pages))
 
-    def spend(self, view: SequenceView, tokens: int, pages: int) -> None:
+    def spend(self, view: SequenceView, tokens: int, pages: Sequence[int]) -> None:
         self.planned.add(view.request_id)
         self.tokens -= tokens
-        self.free_pages = [free - pages for free in self.free_pages]
+        self.free_pages = [free - wanted for free, wanted in zip(self.free_pages, pages)]
 
-    def preempt_for(self, view: SequenceView, pages: int) -> bool:
+    def preempt_for(self, view: SequenceView, pages: Sequence[int]) -> bool:
         """Takes the caches of the youngest running requests that are younger than
         ``view`` and not part of this step, one by one, until ``pages`` fit.  False
         when there is nobody left to take from (what was taken stays taken: those
@@ -148,7 +148,6 @@ class Scheduler:
 
     def _plan_prompts(self, prompts: list[SequenceView], ledger: _Ledger) -> list[PrefillItem]:
         items = []
-        block_size = ledger.capacity.block_size
         for view in prompts:
             if view.request_id in ledger.preempted or ledger.tokens <= 0:
                 continue
@@ -169,8 +168,7 @@ class Scheduler:
                 if not self.enable_chunked_prefill:
                     continue
                 # as much as the free pages hold: the rest of its last page and every free page
-                room = (-start) % block_size + max(min(ledger.free_pages, default=0), 0) * block_size
-                tokens = min(tokens, room)
+                tokens = min(tokens, ledger.capacity.room_for(start, ledger.free_pages))
                 if tokens <= 0:
                     continue
                 pages = ledger.capacity.pages_for(start, start + tokens)

@@ -49,6 +49,10 @@ class Attention(Part):
         if window is not None and (not isinstance(window, int) or window <= 0):
             raise ValueError("attention window must be a positive integer or None.")
         self.window = window
+        page = params.get("block_size")
+        if page is not None and (not isinstance(page, int) or page <= 0):
+            raise ValueError("attention block_size (tokens a page of its cache holds) must be a positive integer or None.")
+        self.block_size = page
         self.dtype = dtype
         self.prefix = spec.prefix
         self.q_norm = build_part("norm", params["q_norm"], dtype) if params.get("q_norm") else None
@@ -82,7 +86,7 @@ class Attention(Part):
         ]
 
     def cache_need(self) -> KVCacheNeed:
-        return KVCacheNeed(self.num_kv_heads, self.head_dim, self.window)
+        return KVCacheNeed(self.num_kv_heads, self.head_dim, self.window, self.block_size)
 
     # The tiled attention kernel walks the runs of tokens of a step in tiles; the tile
     # lists are made on the host once per step, for all attention layers, and travel to

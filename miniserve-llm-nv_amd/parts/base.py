@@ -63,11 +63,14 @@ class WeightSpec:
 @dataclass(frozen=True)
 class KVCacheNeed:
     """Keys and values in pages.  ``window`` None: all keys are kept; an int: only
-    the last ``window`` keys of a position are ever read, older pages go back."""
+    the last ``window`` keys of a position are ever read, older pages go back.
+    ``block_size``: tokens a page of this mixer's group holds; None = the engine's
+    ``kv_block_size`` (a mixer with a short window may want smaller pages)."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    block_size: int | None = None
 
 
 @dataclass(frozen=True)

@@ -265,6 +265,35 @@ def test_window_group_gives_pages_back_while_the_request_lives():
     assert m.capacity().free_blocks == (16, 4)
 
 
+def test_groups_with_page_sizes_of_their_own():
+    """A mixer may ask for pages of another size than the engine's: its group has its
+    own pool, tables and slots; one number of pages for the engine means as many tokens
+    in every group."""
+
+    needs = [Need(0, KVCacheNeed(1, 16)), Need(1, KVCacheNeed(1, 16, window=6, block_size=2)), Need(2, KVCacheNeed(1, 16))]
+    m = manager(needs, block_size=8, num_blocks=6, max_len=64)
+    assert m.block_sizes == (8, 2) and m.num_blocks == (6, 24)          # 48 tokens each
+    assert [g.calls for g in m.layout.groups] == [[0, 2], [1]]
+    capacity = m.capacity()
+    assert capacity.block_sizes == (8, 2) and capacity.pages_for(0, 9) == (2, 5) and capacity.pages_for(9, 10) == (0, 0)
+    assert capacity.most_pages_held(40, 1) == (5, 4) and capacity.room_for(9, (1, 1)) == 3     # 1 + 2 in the small pages
+    m.admit("r")
+    step = m.prepare_step([StepItem("r", 0, 11)])
+    meta = step.sequences[0]
+    assert [len(table) for table in meta.block_tables] == [2, 6]
+    for group, size in enumerate((8, 2)):
+        assert list(meta.slot_mappings[group]) == [
+            meta.block_tables[group][position // size] * size + position % size for position in range(11)
+        ]
+    m.commit_step(step)
+    m.assert_invariants()
+    assert m.capacity().free_blocks == (4, 24 - 3)                       # positions 6..10 of the window: pages 3, 4, 5
+    m.release("r")
+    assert m.capacity().free_blocks == (6, 24)
+    with pytest.raises(ValueError, match="page sizes"):
+        manager([Need(0, KVCacheNeed(1, 16, block_size=0))])
+
+
 def test_the_most_pages_a_request_holds_follow_the_window_of_each_group():
     """What admission compares with the pools: all pages where all keys are kept, the
     window's span (and the step's tokens) where a window has passed; measured here on

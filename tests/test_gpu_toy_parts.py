@@ -20,6 +20,7 @@ from helpers import random_tokens, read_config, read_weights, tiny_a
 pytestmark = pytest.mark.gpu
 
 WINDOW = 6
+WINDOW_PAGE = 32        # the window layers keep pages of their own size (the engine's are 16 or 4 below)
 EXPERTS, EXPERT_WIDTH = 3, 40
 KINDS = ("attention", "running_mean", "window_attention")      # the mixers; layer 1 also has the routed feed-forward,
                                                                 # layer 2 the rotation of neighbouring pairs
@@ -140,7 +141,8 @@ def define_toy():
                     mixer = PartSpec("test_running_mean", {"hidden_size": spec.hidden_size}, f"model.layers.{index}.mixer.")
                 elif kind == "window_attention":
                     position = PartSpec("test_rotary_pairs", dict(layer.mixer.params["position"].params))
-                    mixer = PartSpec("attention", {**layer.mixer.params, "window": WINDOW, "position": position}, layer.mixer.prefix)
+                    mixer = PartSpec("attention", {**layer.mixer.params, "window": WINDOW, "position": position,
+                                                   "block_size": WINDOW_PAGE}, layer.mixer.prefix)
                 else:
                     mixer = layer.mixer
                 feed_forward = layer.feed_forward
@@ -249,7 +251,7 @@ def test_the_toy_model_is_built_from_its_folder(toy):
     model = DecoderModel(load_config(toy).model_spec(), "float32")
     layout = CacheLayout.from_needs(model.cache_needs())
     # full attention: one cache (call 0, read again by call 3); window: two caches (calls 2, 4); two states (calls 1, 5)
-    assert [(g.need.window, g.calls) for g in layout.groups] == [(None, [0]), (WINDOW, [2, 4])]
+    assert [(g.need.window, g.need.block_size, g.calls) for g in layout.groups] == [(None, None, [0]), (WINDOW, WINDOW_PAGE, [2, 4])]
     assert len(layout.states) == 2
     assert [p.kind for p in layout.placements] == ["kv", "state", "kv", "kv", "kv", "state"]
     assert layout.placements[3].write is False and layout.placements[3].index == 0
@@ -265,7 +267,7 @@ def test_the_toy_model_steps_like_its_plain_form(toy, shape, tmp_path):
     requests = {f"r{i}": random_tokens(n, config["vocab_size"], 60 + i) for i, n in enumerate((37, 52, 19, 44, 30, 26))}
     steps = getattr(shapes, shape)(requests, **({"seed": 2} if shape == "mixed" else {}))
     pages_full = -(-shapes.max_live_tokens(steps) // 16)
-    window_pages = 4 * (-(-(WINDOW + 21) // 16) + 1)
+    window_pages = 4 * 2 * (WINDOW_PAGE // 16)         # four live requests, two of the window layers' own pages each
     runner = ModelRunner.from_folder(
         toy, EngineConfig(dtype="float32", kv_block_size=16, num_kv_blocks=max(pages_full, window_pages), max_num_seqs=4,
                           enable_chunked_prefill=True, decode_graphs=False),
@@ -291,6 +293,8 @@ def test_a_window_group_holds_few_pages_for_a_long_request(toy):
         toy, EngineConfig(dtype="float32", kv_block_size=4, num_kv_blocks=40, max_num_seqs=2, enable_chunked_prefill=True,
                           decode_graphs=False),
     )
+    window_pool = 40 * 4 // WINDOW_PAGE            # as many tokens as the engine's 40 pages of 4, in pages of its own size
+    assert runner.cache.num_blocks == (40, window_pool) and runner.cache.block_sizes == (4, WINDOW_PAGE)
     tokens = random_tokens(120, config["vocab_size"], 1)
     runner.admit("long")
     position = 0
@@ -299,9 +303,9 @@ def test_a_window_group_holds_few_pages_for_a_long_request(toy):
         position += size
         free_full, free_window = runner.cache.capacity().free_blocks
         assert free_full == 40 - -(-position // 4)
-        assert 40 - free_window <= -(-WINDOW // 4) + 1                  # the window's pages, not the history's
+        assert window_pool - free_window <= -(-WINDOW // WINDOW_PAGE) + 1        # the window's pages, not the history's
     runner.release("long")
-    assert runner.cache.capacity().free_blocks == (40, 40)
+    assert runner.cache.capacity().free_blocks == (40, window_pool)
 
 
 # ---- state inside recorded steps, aborted steps and preemption ------------------------------------

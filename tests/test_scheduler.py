@@ -35,7 +35,7 @@ def view(name, status, *, target=10, cursor=0, generated=0, arrival=0, max_new=8
 
 
 def capacity(free, *, total=64, block_size=4, free_slots=4, slots=8, held=None) -> CapacitySnapshot:
-    return CapacitySnapshot(block_size, (total,), (free,), free_slots, slots, held or {})
+    return CapacitySnapshot((block_size,), (total,), (free,), free_slots, slots, held or {})
 
 
 def scheduler(**options) -> Scheduler:
