@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     if (epilogue == kSiluMul) {
       // RB is even: blocks 0..RB/2-1 are gate rows, the others the matching up rows
       const int pair = rb % (RB / 2 > 0 ? RB / 2 : 1);
-      row_start[rb] = (blockIdx.x * (RB / 2 > 0 ? RB / 2 : 1) + pair) * 16 + (rb >= RB / 2 ? half : 0);
+      row_start[rb] = (blockIdx.x * (RB / 2 > 0 ? RB / 2 : 1) + pair) * rows + (rb >= RB / 2 ? half : 0);
     } else {
       row_start[rb] = (blockIdx.x * RB + rb) * rows;
     }
@@ -219,11 +219,24 @@ void launch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, 
   const int out_rows = epilogue == kSiluMul ? n / 2 : n;
   const int blocks_per_group = epilogue == kSiluMul ? RB / 2 : RB;
   const int m_tiles = (m + 16 * MB - 1) / (16 * MB);
-  // A matrix of few rows gives 8 or 4 rows instead of 16 to a workgroup: one workgroup
-  // streams less, and there are 256 compute units to feed.
+  // How many of the 16 rows of a block a workgroup takes.  The chip has 256 compute
+  // units; the launch lasts as long as the unit with the most to stream, that is
+  // ceil(workgroups / 256) times a workgroup's rows: 6144 rows in blocks of 16 are 384
+  // workgroups, two for half of the units and one for the others; in blocks of 12 they are
+  // 512, two for each, and a quarter less to stream for the busiest.  Fewest rows on the
+  // busiest unit wins, more rows a workgroup among equals (fewer workgroups, less of x read).
   int rows = 16;
-  if (RB == 1 && epilogue != kSiluMul) {
-    while (rows > 4 && ((out_rows + rows - 1) / rows) * m_tiles < 256) rows /= 2;
+  if (RB <= 2) {
+    int64_t best = INT64_MAX;
+    for (int candidate = 16; candidate >= 4; --candidate) {
+      const int64_t workgroups =
+          static_cast<int64_t>((out_rows + candidate * blocks_per_group - 1) / (candidate * blocks_per_group)) * m_tiles;
+      const int64_t busiest = ((workgroups + 255) / 256) * candidate;
+      if (busiest < best) {
+        best = busiest;
+        rows = candidate;
+      }
+    }
   }
   const int groups = (out_rows + rows * blocks_per_group - 1) / (rows * blocks_per_group);
   // rows of 2048 elements and more: eight k-steps in flight a wave (where the registers allow it)
