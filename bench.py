@@ -24,6 +24,11 @@ peak).  ``measured``: what the card reaches on a plain device copy and a large
 library product.  ``--parity`` adds a 32-bit run of the same layer sizes (two layers
 unless ``--layers`` says otherwise) against the plain float64 implementation of
 ``tests/plain_qwen3.py``: a prompt whole, then 32 tokens one by one.
+
+``--account-trace FILE`` runs nothing on the GPU: it reads the kernel trace
+(``*_kernel_trace.csv``) that ``rocprofv3 --kernel-trace --output-format csv`` wrote
+for a run of this program and prints, kernel by kernel, the time of a decode step,
+of the prefill step and of the mixed run's steps (medians over the steps).
 """
 
 from __future__ import annotations
@@ -63,6 +68,8 @@ def parse_args():
     parser.add_argument("--eager", action="store_true", help="no HIP graphs for decode steps")
     parser.add_argument("--parity", action="store_true",
                         help="also run these layer sizes in 32-bit against the plain float64 implementation")
+    parser.add_argument("--account-trace", metavar="KERNEL_TRACE_CSV", default=None,
+                        help="no run: the per-step kernel times of a rocprofv3 kernel trace of this program")
     return parser.parse_args()
 
 
@@ -154,8 +161,75 @@ def parity_run(sizes, layers, device, prompt_len=300, tail=32):
     }
 
 
+def account_trace(path: str) -> None:
+    """Per-step kernel times from a rocprofv3 kernel trace of this program.  A step
+    begins with the embedding kernel.  Decode steps are those of the most frequent
+    kernel count (the first four are left out as warm-up), the prefill steps the last
+    three that bring neither that count nor single-token attention, the mixed steps
+    the later half (the timed run) of those that hold both attention kernels."""
+
+    import collections
+    import csv
+    import re
+
+    with open(path, newline="") as handle:
+        rows = sorted(csv.DictReader(handle), key=lambda row: int(row["Start_Timestamp"]))
+
+    def short(name: str) -> str:
+        name = name.replace("void ", "").replace("(anonymous namespace)::", "")
+        library = re.match(r"(Custom_)?Cijk_\w*?(MT\d+x\d+x\d+)", name)
+        return "hipBLASLt " + library.group(2) if library else re.sub(r"\(.*", "", name)
+
+    names = [short(row["Kernel_Name"]) for row in rows]
+    begin = [int(row["Start_Timestamp"]) / 1e3 for row in rows]
+    length = [(int(row["End_Timestamp"]) - int(row["Start_Timestamp"])) / 1e3 for row in rows]
+    starts = [index for index, name in enumerate(names) if name.startswith("embedding_gather")] + [len(rows)]
+    steps = list(zip(starts[:-1], starts[1:]))
+    if not steps:
+        print("no step (no embedding kernel) in this trace")
+        return
+
+    def table(chosen, title):
+        if not chosen:
+            return
+        busy = [sum(length[a:b]) for a, b in chosen]
+        span = [begin[b - 1] + length[b - 1] - begin[a] for a, b in chosen]
+        print(f"\n{title}: {len(chosen)} steps, {statistics.median(b - a for a, b in chosen):.0f} kernels a step; "
+              f"kernel time {statistics.median(busy):.1f} us, first start to last end {statistics.median(span):.1f} us (medians)")
+        print(f"{'kernel':58s} {'calls':>5s} {'us/step':>8s} {'avg us':>7s} {'in steps':>8s}")
+        per_kernel = collections.defaultdict(list)
+        for a, b in chosen:
+            inside = collections.defaultdict(list)
+            for name, us in zip(names[a:b], length[a:b]):
+                inside[name].append(us)
+            for name, values in inside.items():
+                per_kernel[name].append((len(values), sum(values)))
+        for name, seen in sorted(per_kernel.items(), key=lambda item: -statistics.median(x[1] for x in item[1])):
+            if len(seen) * 8 < len(chosen):
+                continue                      # a library product of a row count that few steps had
+            calls = statistics.median(x[0] for x in seen)
+            us = statistics.median(x[1] for x in seen)
+            print(f"{name[:58]:58s} {calls:5.0f} {us:8.1f} {us / calls:7.2f} {len(seen):8d}")
+
+    def holds(step, prefix):
+        return any(name.startswith(prefix) for name in names[step[0]:step[1]])
+
+    count = collections.Counter(b - a for a, b in steps if not holds((a, b), "attention_prefill")).most_common(1)
+    decode = [s for s in steps if count and s[1] - s[0] == count[0][0] and not holds(s, "attention_prefill")][4:]
+    mixed = [s for s in steps if holds(s, "attention_prefill") and holds(s, "attention_decode")]
+    prefill = [s for s in steps if holds(s, "attention_prefill") and not holds(s, "attention_decode")
+               and not holds(s, "at::native")][-3:]
+    table(decode, "decode step")
+    table(prefill, "prefill step")
+    if len(mixed) >= 8:                       # fewer: the prompts of the decode runs, not the mixed run
+        table(mixed[len(mixed) // 2:], "step with prompt portions beside decode tokens")
+
+
 def main() -> int:
     args = parse_args()
+    if args.account_trace:
+        account_trace(args.account_trace)
+        return 0
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine does not span GPUs).")
         return 2

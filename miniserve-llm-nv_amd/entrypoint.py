@@ -55,11 +55,22 @@ class LLM:
         self.engine = Engine(self.runner)
 
     @classmethod
-    def from_random(cls, config, *, seed: int = 0, **options) -> "LLM":
-        """An engine over random weights of ``config`` (a configuration object of a
-        registered architecture), drawn on the device: for sizes that should not
-        pass through a file.  ``options`` as for the constructor."""
+    def from_random(cls, config, *, seed: int = 0, layers: int | None = None, **options) -> "LLM":
+        """An engine over random weights, drawn on the device: for sizes that should
+        not pass through a file.  ``config`` is a configuration object of a
+        registered architecture, the name of a preset (``"qwen3-0.6b"``) or the path
+        of a ``config.json``; ``layers`` replaces the number of layers of a preset or
+        file.  ``options`` as for the constructor."""
 
+        if isinstance(config, (str, os.PathLike)):
+            from .config import config_dict_from_preset_or_file, config_from_dict
+
+            data = config_dict_from_preset_or_file(os.fspath(config))
+            if layers is not None:
+                data["num_hidden_layers"] = layers
+            config = config_from_dict(data)
+        elif layers is not None:
+            raise ValueError("layers= goes with a preset's name or a config.json; a configuration object names its own.")
         return cls(config, seed=seed, **options)
 
     def generate(

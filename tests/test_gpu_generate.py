@@ -258,6 +258,26 @@ def test_command_line_with_layer_sizes_by_name():
     assert process.returncode != 0 and "qwen3-0.6b, qwen3-32b, qwen3-8b" in process.stderr
 
 
+def test_entry_point_with_layer_sizes_by_name():
+    """``LLM.from_random`` with a preset's name draws what the command line draws for the
+    same seed, and refuses ``layers=`` beside a configuration object."""
+
+    from miniserve_amd.config import config_dict_from_preset_or_file, config_from_dict
+    from miniserve_amd.engine import SamplingParams
+    from miniserve_amd.entrypoint import LLM
+
+    options = dict(max_model_len=256, num_kv_blocks=32, seed=3)
+    by_name = LLM.from_random("qwen3-0.6b", layers=2, **options)
+    tokens = by_name.generate([[5, 9, 200, 31]], SamplingParams(max_new_tokens=6))[0]
+    del by_name
+    data = config_dict_from_preset_or_file("qwen3-0.6b")
+    data["num_hidden_layers"] = 2
+    by_object = LLM.from_random(config_from_dict(data), **options)
+    assert by_object.generate([[5, 9, 200, 31]], SamplingParams(max_new_tokens=6))[0] == tokens
+    with pytest.raises(ValueError, match="layers="):
+        LLM.from_random(config_from_dict(data), layers=1)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_graphs_replay_like_eager_steps(dtype, model_folders):
     """Decode steps recorded as HIP graphs, replayed many times with eager steps
