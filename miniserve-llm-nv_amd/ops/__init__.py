@@ -389,6 +389,10 @@ _EPILOGUE_BF16, _EPILOGUE_F32, _EPILOGUE_ADD_F32, _EPILOGUE_SILU_MUL = 0, 1, 2, 
 # up to SKINNY_MAX_ROWS rows.
 SKINNY_MAX_ROWS = 16
 SKINNY_KERNEL_ROWS = 64
+# The largest matrices whose product takes the norm as its prologue (plain, and with the
+# gated activation as its epilogue); beyond them the norm is a kernel of its own.
+FUSED_NORM_BYTES = 64 << 20
+FUSED_NORM_GATED_BYTES = 48 << 20
 
 
 _GEMM_WORKSPACE_BYTES = 64 << 20
@@ -431,8 +435,10 @@ def _library_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, a
 # recorded graphs over matrices that no cache holds (as a decode step meets its
 # weights), for the matrices of the 0.6B, 8B and 32B sizes and 1 to 64 rows: this
 # library's product streams a small matrix faster, the more so the fewer the rows;
-# hipBLASLt streams a large one faster unless its rows are very long; the fused forms
-# (norm as prologue, activation as epilogue) save one or two kernels of some 5 us each.
+# hipBLASLt, with the fastest of its candidates for the shape, streams a large one
+# faster; the fused forms (norm as prologue, activation as epilogue) save one or two
+# kernels of some 5 us each.  (Which candidate the library runs is timed once per
+# process and shape; its candidates differ in the order of their 32-bit sums only.)
 _MIB = 1 << 20
 product_calls = {"skinny": 0, "library": 0}     # calls served by each since the import
 _forced_product: str | None = None
@@ -468,7 +474,7 @@ def prefers_skinny(m: int, n: int, k: int, *, fused: bool = False) -> bool:
         return True
     if m > SKINNY_MAX_ROWS:
         return False
-    if size <= 40 * _MIB or k >= 16384:         # middle sizes; very long rows, which the library splits badly
+    if size <= 40 * _MIB:                       # middle sizes
         return True
     if n >= 65536:                              # a head: many short rows
         return m <= 8
@@ -546,10 +552,17 @@ def can_accumulate(rows: int, weight: torch.Tensor) -> bool:
 
 
 def can_fuse_norm(rows: int, weight: torch.Tensor, *, gated: bool = False) -> bool:
-    """Whether :func:`linear_normed` runs as one kernel for this many rows."""
+    """Whether :func:`linear_normed` runs as one kernel for this many rows.  The norm as
+    a prologue makes every workgroup read the 32-bit rows and the norm's weight beside its
+    share of the matrix, which costs more than a norm kernel of its own once the matrix
+    is large (measured on MI355X at 8 rows, fused against product + norm kernel: 48 MiB,
+    16 us against 13 + 5; 100 MiB, 38 against 23 + 7; with the gated activation 48 MiB,
+    17.5 against 12 + 5; 95 MiB, 39 against 24 + 5; 192 MiB, 50 against 42 + 5)."""
 
     n, k = weight.shape
     epilogue = _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16
+    if _forced_product is None and 2 * n * k > (FUSED_NORM_GATED_BYTES if gated else FUSED_NORM_BYTES):
+        return False
     return (
         weight.dtype == torch.bfloat16
         and rows <= SKINNY_MAX_ROWS

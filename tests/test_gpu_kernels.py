@@ -542,7 +542,8 @@ def test_linear_bfloat16_and_fused_projection_rows(ops):
 
 
 @pytest.mark.parametrize("m", [1, 8, 15, 16, 17, 33, 64])
-@pytest.mark.parametrize("n,k", [(16, 32), (509, 96), (100, 200), (4096, 1024), (1024, 3072), (72, 2056), (40, 4104), (40000, 64)])
+@pytest.mark.parametrize("n,k", [(16, 32), (509, 96), (100, 200), (4096, 1024), (1024, 3072), (72, 2056), (40, 4104), (40000, 64),
+                                 (5130, 72), (6144, 2048)])       # from 5120 rows on two blocks a workgroup
 def test_skinny_product_for_few_rows(ops, m, n, k, monkeypatch):
     """The matrix-core product that decoding uses (at most 64 rows), with its four
     epilogues, against float64; sizes off the tile grid in every dimension."""
@@ -889,3 +890,31 @@ def test_product_with_the_norm_as_its_prologue(ops, m, n, k):
     assert float(ratio) <= 1.0, f"unfused: error / bound = {float(ratio):.2f}"
     assert not ops.can_fuse_norm(17, weight)
     assert not ops.can_fuse_norm(m, weight.float())
+
+
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("n,k", [(5128, 64), (6144, 2048), (5120, 4104)])
+def test_product_with_the_norm_as_its_prologue_against_many_rows(ops, m, n, k):
+    """From 5120 rows of the matrix on a workgroup takes two blocks of rows.  Against the
+    norm and the product in float64 with nothing rounded: the one rounding of a normed
+    input to bfloat16 is at most 2^-8 of it (uniform, so 2^-8 / sqrt(3) in the mean), the
+    roundings of the k inputs are independent, and the result is rounded once more;
+    six standard deviations, and every row bit-equal to the same row alone."""
+
+    residual = rand(m, k, seed=m + n, scale=2.0)
+    norm_weight = (1 + 0.1 * rand(k, seed=5)).to(torch.bfloat16)
+    weight = rand(n, k, seed=n + k, dtype=torch.bfloat16, scale=0.05)
+    wide = residual.cpu().double()
+    inputs = wide / (wide.pow(2).mean(-1, keepdim=True) + 1e-5).sqrt() * norm_weight.cpu().double()
+    exact = inputs @ weight.cpu().double().T
+    deviation = 2**-8 / 3**0.5 * (inputs.pow(2) @ weight.cpu().double().pow(2).T).sqrt()
+    bound = 6 * deviation + 2**-8 * exact.abs() + 1e-6
+    with ops.forced_product("skinny"):
+        fused = ops.linear_normed(residual, norm_weight, 1e-5, weight)
+        ratio = ((fused.cpu().double() - exact).abs() / bound).max()
+        assert float(ratio) <= 1.0, f"error / bound = {float(ratio):.2f}"
+        alone = ops.linear_normed(residual[m // 2 : m // 2 + 1].contiguous(), norm_weight, 1e-5, weight)
+        assert torch.equal(alone[0], fused[m // 2])
+        if n % 2 == 0:
+            gated = ops.linear_normed(residual, norm_weight, 1e-5, weight, gated=True)
+            assert torch.equal(gated, ops.silu_mul(fused))       # the same sums, rounded, then the activation

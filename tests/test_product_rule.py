@@ -20,7 +20,36 @@ def test_the_rule_for_the_two_products():
     assert ops.prefers_skinny(16, 4096, 4096) and not ops.prefers_skinny(17, 4096, 4096)         # 32 MiB
     assert not ops.prefers_skinny(8, 24576, 4096) and ops.prefers_skinny(8, 24576, 4096, fused=True)
     assert not ops.prefers_skinny(8, 51200, 5120, fused=True)                                    # 500 MiB
-    assert ops.prefers_skinny(16, 5120, 25600) and not ops.prefers_skinny(17, 5120, 25600)       # very long rows
+    assert not ops.prefers_skinny(8, 5120, 25600)            # 250 MiB of very long rows: the library's timed choice splits them
+
+
+def test_the_norm_is_a_prologue_only_of_small_and_middle_matrices(monkeypatch):
+    """The norm as the product's prologue pays up to 64 MiB (48 MiB with the gated
+    activation); larger matrices get a norm kernel of their own."""
+
+    import torch
+
+    from miniserve_amd import ops
+
+    class Library:
+        @staticmethod
+        def ms_gemm_skinny_supported(m, n, k, epilogue):
+            return 1
+
+    monkeypatch.setattr(ops, "load", lambda: Library)
+
+    def weight(n, k):
+        return torch.empty((n, k), dtype=torch.bfloat16, device="meta")
+
+    assert ops.can_fuse_norm(8, weight(4096, 1024)) and ops.can_fuse_norm(8, weight(6144, 1024), gated=True)   # 0.6B
+    assert ops.can_fuse_norm(16, weight(4096, 4096)) and not ops.can_fuse_norm(17, weight(4096, 4096))
+    assert ops.can_fuse_norm(8, weight(6144, 4096))                     # 48 MiB: the q/k/v matrix of the 8B sizes
+    assert not ops.can_fuse_norm(8, weight(10240, 5120))                # 100 MiB: that of the 32B sizes
+    assert not ops.can_fuse_norm(8, weight(24576, 4096), gated=True)    # 192 MiB: its gate and up matrix
+    assert ops.can_fuse_norm(8, weight(12288, 2048), gated=True)        # 48 MiB, gated
+    assert ops.prefers_skinny(8, 24576, 4096, fused=True)               # the activation stays that product's epilogue
+    with ops.forced_product("skinny"):
+        assert ops.can_fuse_norm(8, weight(10240, 5120))                # tests may still ask for the fused kernel
 
 
 def test_a_forced_product_overrides_the_rule_and_is_undone():
