@@ -42,7 +42,13 @@ constexpr int kWaveColumns = 32;      // columns (token, head) of one wave
 constexpr float kMaxSlack = 6.0f;
 
 // Keys and values of one pair of tiles in LDS.  Rows are padded so that lanes that
-// read different rows spread over the banks.
+// read different rows spread over the banks (16 lanes that read 16 bytes each of
+// consecutive rows touch every bank once, for keys and for values).
+//
+// A row of values holds the 16 keys of its tile in the order in which the product
+// P.V wants them: the scores' product leaves lane half h with the keys 4h..4h+3 and
+// 8+4h..8+4h+3 of a tile, so the groups of four keys lie in the order 0, 2, 1, 3 and a
+// lane reads its eight values as one 16-byte word.
 template <int D>
 struct alignas(16) PairBuffer {
   static constexpr int kKeyRow = D + 8;      // elements; 16-byte aligned rows
@@ -78,24 +84,48 @@ struct ChunkPlace {
   }
 };
 
-template <int D, int THREADS>
-__device__ __forceinline__ void stage_load(StagedPair<D, THREADS>& staged, int thread, int tile, int end_tile,
-                                           const int32_t* __restrict__ table, const bf16* __restrict__ key_pool,
-                                           const bf16* __restrict__ value_pool, int num_kv_heads, int kv_head,
-                                           int block_size) {
-  // No branch stands around a load: the counters that order the loads stay exact.  A
-  // pair past the end repeats the last one and a missing second tile repeats the
+// Where the two tiles of a pair lie in the cache: the page of each and the offset of its
+// first key in the page.  The same in every lane (scalar registers); looked up from the
+// block table two rounds before the pair's loads are issued, so that nothing waits for
+// the table.
+struct PairPages {
+  int32_t page[2];
+  int offset[2];
+};
+
+__device__ __forceinline__ PairPages find_pair(int tile, int end_tile, const int32_t* __restrict__ table,
+                                               int block_size) {
+  // A pair past the end repeats the last one and a missing second tile repeats the
   // first; what they hold lies beyond the last key and is masked.
   tile = min(tile, end_tile - 1);
+  PairPages pages;
 #pragma unroll
   for (int side = 0; side < 2; ++side) {
-    const int first_key = (side == 1 && tile + 1 < end_tile ? tile + 1 : tile) * kTileKeys;
-    // the same in every lane: scalar arithmetic
-    const int64_t page = ms::uniform(table[first_key / block_size]);
-    const int offset = first_key % block_size;
-    const int64_t slab = page * num_kv_heads + kv_head;
-    const bf16* keys = key_pool + (slab * block_size + offset) * D;
-    const bf16* values = value_pool + slab * D * block_size + offset;
+    const int this_tile = side == 1 && tile + 1 < end_tile ? tile + 1 : tile;
+    if (block_size == kTileKeys) {      // a page is a tile: no division
+      pages.page[side] = ms::uniform(table[this_tile]);
+      pages.offset[side] = 0;
+    } else {
+      const int first_key = this_tile * kTileKeys;
+      pages.page[side] = ms::uniform(table[first_key / block_size]);
+      pages.offset[side] = first_key % block_size;
+    }
+  }
+  return pages;
+}
+
+// page_stride: elements of one page of a pool (all its kv heads); head_base: where the
+// workgroup's kv head begins in a page.  Both are the same for keys and values.
+template <int D, int THREADS>
+__device__ __forceinline__ void stage_load(StagedPair<D, THREADS>& staged, int thread, const PairPages& pages,
+                                           const bf16* __restrict__ key_pool, const bf16* __restrict__ value_pool,
+                                           int64_t page_stride, int head_base, int block_size) {
+  // No branch stands around a load: the counters that order the loads stay exact.
+#pragma unroll
+  for (int side = 0; side < 2; ++side) {
+    const int64_t slab = pages.page[side] * page_stride + head_base;
+    const bf16* keys = key_pool + slab + pages.offset[side] * D;
+    const bf16* values = value_pool + slab + pages.offset[side];
 #pragma unroll
     for (int j = 0; j < StagedPair<D, THREADS>::kPerTile; ++j) {
       const ChunkPlace<D, THREADS> place(thread, j);
@@ -113,7 +143,11 @@ __device__ __forceinline__ void stage_store(const StagedPair<D, THREADS>& staged
     for (int j = 0; j < StagedPair<D, THREADS>::kPerTile; ++j) {
       const ChunkPlace<D, THREADS> place(thread, j);
       *reinterpret_cast<bf16x8*>(&buffer.k[side * kTileKeys + place.key][8 * place.part]) = staged.k[side][j];
-      *reinterpret_cast<bf16x8*>(&buffer.v[side][place.d][8 * place.half]) = staged.v[side][j];
+      // keys 8 half .. 8 half + 7: the groups 2 half and 2 half + 1, which lie at 4 half and 8 + 4 half
+      const bf16x8 values = staged.v[side][j];
+      *reinterpret_cast<bf16x4*>(&buffer.v[side][place.d][4 * place.half]) = bf16x4{values[0], values[1], values[2], values[3]};
+      *reinterpret_cast<bf16x4*>(&buffer.v[side][place.d][8 + 4 * place.half]) =
+          bf16x4{values[4], values[5], values[6], values[7]};
     }
 }
 
@@ -127,11 +161,14 @@ struct PrefillState {
   float run_sum;    // of this lane's keys only; the two lanes are added at the end
 };
 
-// One pair of key tiles (32 keys from `key0`) against the wave's 32 columns.
-template <int D, bool MASKED>
+// One pair of key tiles (32 keys from `key0`) against the wave's 32 columns.  `masked`
+// (the same in all lanes): some key of the pair is hidden from some column, or lies
+// beyond what the sequence has written.  One body serves both cases, so that the
+// outputs stay in the same registers whichever way a step goes.
+template <int D>
 __device__ __forceinline__ void consume_pair(PrefillState<D>& st, const PairBuffer<D>& buffer,
                                              const bf16x8 (&q_reg)[D / 16], int key0, int lo, int pos, int last_key,
-                                             float scale_log2, int h, int column) {
+                                             float scale_log2, int h, int column, bool masked) {
   constexpr int KS = D / 16, CS = PrefillState<D>::CS;
   floatx16 s;
 #pragma unroll
@@ -141,16 +178,36 @@ __device__ __forceinline__ void consume_pair(PrefillState<D>& st, const PairBuff
     const bf16x8 keys = *reinterpret_cast<const bf16x8*>(&buffer.k[column][16 * step + 8 * h]);
     s = ms::mfma_32x32x16(keys, q_reg[step], s);
   }
-  // register v: key0 + 8 (v / 4) + 4 h + v % 4
-  float tile_max = -INFINITY;
+  // The values of the step are asked for now; they arrive while the weights are made.
+  // slot x of the contraction index of half j: key0 + 16 j + 8 (x / 4) + 4 h + x % 4,
+  // for P (registers 8 j + x below) and for V alike.
+  bf16x8 values[CS][2];
 #pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    if (MASKED) {
+  for (int c = 0; c < CS; ++c) {
+    const int d = (D % 32 == 0) ? 32 * c + column : min(32 * c + column, D - 1);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) values[c][j] = *reinterpret_cast<const bf16x8*>(&buffer.v[j][d][8 * h]);
+  }
+  // register v: key0 + 8 (v / 4) + 4 h + v % 4
+  if (masked) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
       const int key = key0 + 8 * (v / 4) + 4 * h + (v % 4);
       s[v] = (key >= lo && key <= pos) ? s[v] : -INFINITY;
     }
-    tile_max = fmaxf(tile_max, s[v]);
+    // A stale value (a slot beyond what the sequence has written) times a zero weight
+    // must not become NaN: such slots exist only in steps that are masked.
+#pragma unroll
+    for (int c = 0; c < CS; ++c)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int x = 0; x < 8; ++x)
+          if (key0 + 16 * j + 8 * (x / 4) + 4 * h + (x % 4) > last_key) values[c][j][x] = static_cast<__bf16>(0.0f);
   }
+  float tile_max = -INFINITY;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) tile_max = fmaxf(tile_max, s[v]);
   tile_max = ms::max_xor32(tile_max) * scale_log2;
   // the maximum moves only when it is exceeded by more than the slack (or is still unset)
   const bool move = tile_max > st.run_max + kMaxSlack;
@@ -175,28 +232,10 @@ __device__ __forceinline__ void consume_pair(PrefillState<D>& st, const PairBuff
   }
   st.run_sum += tile_sum;
   st.run_max = new_max;
-
-  // slot x of the contraction index of half j: key0 + 16 j + 8 (x / 4) + 4 h + x % 4,
-  // for P (registers 8 j + x above) and for V alike
 #pragma unroll
-  for (int c = 0; c < CS; ++c) {
-    const int d = (D % 32 == 0) ? 32 * c + column : min(32 * c + column, D - 1);
+  for (int c = 0; c < CS; ++c)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      bf16x4 near = *reinterpret_cast<const bf16x4*>(&buffer.v[j][d][4 * h]);
-      bf16x4 far = *reinterpret_cast<const bf16x4*>(&buffer.v[j][d][8 + 4 * h]);
-      if (MASKED) {
-        // A stale value (a slot beyond what the sequence has written) times a zero
-        // weight must not become NaN: such slots exist only in steps that are masked.
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (key0 + 16 * j + 4 * h + e > last_key) near[e] = static_cast<__bf16>(0.0f);
-          if (key0 + 16 * j + 8 + 4 * h + e > last_key) far[e] = static_cast<__bf16>(0.0f);
-        }
-      }
-      st.o[c] = ms::mfma_32x32x16(ms::concat(near, far), p[j], st.o[c]);
-    }
-  }
+    for (int j = 0; j < 2; ++j) st.o[c] = ms::mfma_32x32x16(values[c][j], p[j], st.o[c]);
 }
 
 // What the second half of a workgroup hands to the first at the end: every register
@@ -291,30 +330,37 @@ __global__ __launch_bounds__(256 * HB) MS_WAVES_PER_EU(2, 2) void attention_pref
   st.run_max = -INFINITY;
   st.run_sum = 0.f;
 
-  // One pair in flight in registers, two buffers in LDS for each half: the loads of
-  // the half's next pair are issued before the current one is consumed.  No branch
-  // stands between a load and its use; both halves make the same number of rounds.
-  StagedPair<D, HALF_THREADS> staged;
-  stage_load<D, HALF_THREADS>(staged, thread, t0 + 2 * half_id, t1, table, key_pool, value_pool, num_kv_heads, kv_head,
-                              block_size);
-  int parity = 0;
-  for (int round_tile = t0; round_tile < t1; round_tile += 4) {
-    const int t = round_tile + 2 * half_id;
-    PairBuffer<D>& buffer = buffers[2 * parity + half_id];
-    stage_store<D, HALF_THREADS>(staged, thread, buffer);
-    stage_load<D, HALF_THREADS>(staged, thread, t + 4, t1, table, key_pool, value_pool, num_kv_heads, kv_head,
-                                block_size);
-    __syncthreads();    // the pair is in LDS; every wave is done with the other buffers' previous content
-    if (t < t1 && t * kTileKeys <= wave_last_key && (t + 2) * kTileKeys > wave_first_lo) {
-      // every key of the pair visible to every column of the wave: no masks
-      const bool all_visible = (t + 2) * kTileKeys - 1 <= wave_first_pos && t * kTileKeys >= wave_last_lo;
-      if (all_visible) {
-        consume_pair<D, false>(st, buffer, q_reg, t * kTileKeys, lo, pos, last_key, scale_log2, h, column);
-      } else {
-        consume_pair<D, true>(st, buffer, q_reg, t * kTileKeys, lo, pos, last_key, scale_log2, h, column);
+  // Two pairs in flight in registers, two buffers in LDS for each half: the loads of a
+  // pair are issued two rounds before it is consumed (a round is shorter than the way
+  // to memory and back).  No branch stands between a load and its use; both halves make
+  // the same number of rounds, two to a turn of the loop so that each pair in flight has
+  // registers of its own.
+  StagedPair<D, HALF_THREADS> ahead[2];
+  PairPages pages[2];
+  const int64_t page_stride = static_cast<int64_t>(num_kv_heads) * block_size * D;
+  const int head_base = kv_head * block_size * D;
+#pragma unroll
+  for (int parity = 0; parity < 2; ++parity) {
+    stage_load<D, HALF_THREADS>(ahead[parity], thread, find_pair(t0 + 2 * half_id + 4 * parity, t1, table, block_size),
+                                key_pool, value_pool, page_stride, head_base, block_size);
+    pages[parity] = find_pair(t0 + 2 * half_id + 4 * parity + 8, t1, table, block_size);
+  }
+  for (int round_tile = t0; round_tile < t1; round_tile += 8) {
+#pragma unroll
+    for (int parity = 0; parity < 2; ++parity) {
+      const int t = round_tile + 4 * parity + 2 * half_id;
+      PairBuffer<D>& buffer = buffers[2 * parity + half_id];
+      stage_store<D, HALF_THREADS>(ahead[parity], thread, buffer);
+      stage_load<D, HALF_THREADS>(ahead[parity], thread, pages[parity], key_pool, value_pool, page_stride, head_base,
+                                  block_size);
+      pages[parity] = find_pair(t + 16, t1, table, block_size);
+      __syncthreads();    // the pair is in LDS; every wave is done with the other buffers' previous content
+      if (t < t1 && t * kTileKeys <= wave_last_key && (t + 2) * kTileKeys > wave_first_lo) {
+        // every key of the pair visible to every column of the wave: no masks
+        const bool all_visible = (t + 2) * kTileKeys - 1 <= wave_first_pos && t * kTileKeys >= wave_last_lo;
+        consume_pair<D>(st, buffer, q_reg, t * kTileKeys, lo, pos, last_key, scale_log2, h, column, !all_visible);
       }
     }
-    parity ^= 1;
   }
 
   // The second half hands over; the two states of a column are joined as two steps
@@ -423,6 +469,8 @@ extern "C" int ms_attention_prefill(const void* q, const void* key_pool, const v
              "is not supported",
              head_dim, block_size);
   MS_REQUIRE(max_blocks > 0 && window >= 0, "attention_prefill: bad table width or window");
+  MS_REQUIRE(static_cast<int64_t>(num_kv_heads) * block_size * head_dim < (int64_t{1} << 31),
+             "attention_prefill: a page of %d kv heads x %d keys x %d is too large", num_kv_heads, block_size, head_dim);
   const int group = num_q_heads / num_kv_heads;
   const int hb = group >= 2 ? 2 : 1;   // query heads of one workgroup
   MS_REQUIRE(num_kv_heads * ((group + hb - 1) / hb) <= 65535, "attention_prefill: too many heads");
