@@ -5,7 +5,11 @@
 // query heads that share a kv head: 64 * HB columns, 32 to a wave (16 tokens of two
 // heads, or 32 tokens of one).  It walks the keys 0 .. (its last token's position) in
 // pairs of tiles of 16; its threads load a pair together (16 bytes a thread) into an
-// LDS buffer, and every wave reads its matrix-core operands from there.  With
+// LDS buffer, and every wave reads its matrix-core operands from there.  The keys are
+// dealt out to PARTS parts of the workgroup (two parts of two heads, or four parts of
+// one head: eight waves either way, two to a SIMD), which are joined through LDS at
+// the end.  A workgroup may take two tiles one after the other, a long one and a short
+// one, so that all workgroups of a launch have about the same number of keys to walk.  With
 // 32x32x16 products
 //
 //   S^T[key, column]  = K[key, :] . Q[column, :]       A = 32 keys, B = Q^T
@@ -30,6 +34,8 @@ using ms::floatx16;
 using ms::kTileKeys;
 
 constexpr int kTileTokens = 64;       // query tokens of a workgroup at most
+constexpr int kComputeUnits = 256;    // of the chip: a launch wants a workgroup for each
+constexpr int kPairedFrom = 2 * kComputeUnits - kComputeUnits / 4;   // workgroups from which they are handed out in pairs
 constexpr int kWaveColumns = 32;      // columns (token, head) of one wave
 
 // Softmax arithmetic runs in base 2: the scale and log2(e) enter the exponent's
@@ -49,12 +55,23 @@ constexpr float kMaxSlack = 6.0f;
 // P.V wants them: the scores' product leaves lane half h with the keys 4h..4h+3 and
 // 8+4h..8+4h+3 of a tile, so the groups of four keys lie in the order 0, 2, 1, 3 and a
 // lane reads its eight values as one 16-byte word.
+//
+// Key rows of 128 elements are not padded (eight buffers of them must fit the LDS):
+// the 16-byte chunk c of row r lies at chunk c ^ (r & 15) instead.
 template <int D>
 struct alignas(16) PairBuffer {
-  static constexpr int kKeyRow = D + 8;      // elements; 16-byte aligned rows
-  static constexpr int kValueRow = 24;       // 16 keys of one value column + padding
+  static constexpr bool kSwizzled = D == 128;
+  static constexpr int kKeyRow = kSwizzled ? D : D + 8;      // elements; 16-byte aligned rows
+  static constexpr int kValueRow = 24;                       // 16 keys of one value column + padding
   bf16 k[2 * kTileKeys][kKeyRow];
   bf16 v[2][D][kValueRow];
+  // where the 8 elements from d = 8 * chunk of key row `row` lie
+  __device__ __forceinline__ bf16* key_chunk(int row, int chunk) {
+    return &k[row][8 * (kSwizzled ? (chunk ^ (row & 15)) : chunk)];
+  }
+  __device__ __forceinline__ const bf16* key_chunk(int row, int chunk) const {
+    return &k[row][8 * (kSwizzled ? (chunk ^ (row & 15)) : chunk)];
+  }
 };
 
 // The share of one thread in the cooperative load of a pair: 16-byte chunks, the
@@ -142,7 +159,7 @@ __device__ __forceinline__ void stage_store(const StagedPair<D, THREADS>& staged
 #pragma unroll
     for (int j = 0; j < StagedPair<D, THREADS>::kPerTile; ++j) {
       const ChunkPlace<D, THREADS> place(thread, j);
-      *reinterpret_cast<bf16x8*>(&buffer.k[side * kTileKeys + place.key][8 * place.part]) = staged.k[side][j];
+      *reinterpret_cast<bf16x8*>(buffer.key_chunk(side * kTileKeys + place.key, place.part)) = staged.k[side][j];
       // keys 8 half .. 8 half + 7: the groups 2 half and 2 half + 1, which lie at 4 half and 8 + 4 half
       const bf16x8 values = staged.v[side][j];
       *reinterpret_cast<bf16x4*>(&buffer.v[side][place.d][4 * place.half]) = bf16x4{values[0], values[1], values[2], values[3]};
@@ -175,7 +192,7 @@ __device__ __forceinline__ void consume_pair(PrefillState<D>& st, const PairBuff
   for (int v = 0; v < 16; ++v) s[v] = 0.f;
 #pragma unroll
   for (int step = 0; step < KS; ++step) {
-    const bf16x8 keys = *reinterpret_cast<const bf16x8*>(&buffer.k[column][16 * step + 8 * h]);
+    const bf16x8 keys = *reinterpret_cast<const bf16x8*>(buffer.key_chunk(column, 2 * step + h));
     s = ms::mfma_32x32x16(keys, q_reg[step], s);
   }
   // The values of the step are asked for now; they arrive while the weights are made.
@@ -238,139 +255,147 @@ __device__ __forceinline__ void consume_pair(PrefillState<D>& st, const PairBuff
     for (int j = 0; j < 2; ++j) st.o[c] = ms::mfma_32x32x16(values[c][j], p[j], st.o[c]);
 }
 
-// What the second half of a workgroup hands to the first at the end: every register
-// of the state, lane by lane.
+// What a part of a workgroup hands to the first part at the end: every register of the
+// state, lane by lane.
 template <int D>
 struct MergeSlot {
   float value[PrefillState<D>::CS * 16 + 2][ms::kWave];
 };
 
-constexpr int kMergeWaves = 4;   // slots of one round of the hand-over
-
-template <int D>
+template <int D, int HB, int PARTS>
 constexpr size_t prefill_lds_bytes() {
-  return 4 * sizeof(PairBuffer<D>) > kMergeWaves * sizeof(MergeSlot<D>) ? 4 * sizeof(PairBuffer<D>)
-                                                                          : kMergeWaves * sizeof(MergeSlot<D>);
+  constexpr size_t buffers = 2 * PARTS * sizeof(PairBuffer<D>);
+  constexpr size_t slots = (PARTS - 1) * 2 * HB * sizeof(MergeSlot<D>);
+  return buffers > slots ? buffers : slots;
 }
 
-template <int D, int HB>
-__global__ __launch_bounds__(256 * HB) MS_WAVES_PER_EU(2, 2) void attention_prefill_kernel(
+template <int D, int HB, int PARTS>
+__global__ __launch_bounds__(128 * HB * PARTS) MS_WAVES_PER_EU(2, 2) void attention_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ key_pool, const bf16* __restrict__ value_pool,
     const int32_t* __restrict__ block_table, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_token, const int32_t* __restrict__ tile_count,
-    bf16* __restrict__ out, int num_q_heads, int num_kv_heads, int block_size, int max_blocks, float scale,
-    int window) {
-  // The workgroup is two halves of 2 HB waves.  Both hold the same 64 HB columns; the
-  // first takes the pairs of key tiles 0, 2, 4, ... of the tile's range and the second
-  // the pairs 1, 3, 5, ...: two waves on every SIMD, one in the matrix cores while the
-  // other is in its softmax, and half as many steps for the longest tile.  Each half
-  // loads its own pairs into its own LDS buffers; at the end the second hands its
-  // state to the first through LDS.
-  constexpr int HALF_THREADS = 128 * HB;
-  constexpr int HALF_WAVES = 2 * HB;
+    bf16* __restrict__ out, int num_tiles, int paired, int num_q_heads, int num_kv_heads, int block_size,
+    int max_blocks, float scale, int window) {
+  // The workgroup is PARTS parts of 2 HB waves.  All hold the same 64 HB columns; part p
+  // takes the pairs of key tiles p, p + PARTS, p + 2 PARTS, ... of the tile's range: two
+  // waves on every SIMD, one in the matrix cores while the other is in its softmax, and
+  // 1 / PARTS of the steps for the longest tile.  Each part loads its own pairs into its
+  // own LDS buffers; at the end the others hand their states to the first through LDS.
+  constexpr int PART_THREADS = 128 * HB;
+  constexpr int PART_WAVES = 2 * HB;
   constexpr int KS = D / 16, CS = PrefillState<D>::CS;
-  __shared__ __align__(16) unsigned char lds[prefill_lds_bytes<D>()];
-  PairBuffer<D>* buffers = reinterpret_cast<PairBuffer<D>*>(lds);        // [parity][half]
-  MergeSlot<D>* slots = reinterpret_cast<MergeSlot<D>*>(lds);
+  __shared__ __align__(16) unsigned char lds[prefill_lds_bytes<D, HB, PARTS>()];
+  PairBuffer<D>* buffers = reinterpret_cast<PairBuffer<D>*>(lds);        // [parity][part]
+  MergeSlot<D>* slots = reinterpret_cast<MergeSlot<D>*>(lds);            // [part - 1][wave]
 
   const int lane = threadIdx.x & 63;
   const int wave_of_group = ms::uniform(threadIdx.x >> 6);   // the same in all lanes: kept in a scalar register
-  const int half_id = wave_of_group / HALF_WAVES;
-  const int wave = wave_of_group - half_id * HALF_WAVES;
-  const int thread = threadIdx.x - half_id * HALF_THREADS;
+  const int part_id = wave_of_group / PART_WAVES;
+  const int wave = wave_of_group - part_id * PART_WAVES;
+  const int thread = threadIdx.x - part_id * PART_THREADS;
   const int h = lane >> 5;
   const int column = lane & 31;
 
-  // long tiles (late in their sequences) first
-  const int tile_index = gridDim.x - 1 - blockIdx.x;
   const int group = num_q_heads / num_kv_heads;
   const int head_blocks = (group + HB - 1) / HB;
   const int kv_head = blockIdx.y / head_blocks;
   const int head0 = kv_head * group + (blockIdx.y - kv_head * head_blocks) * HB;
   const int heads_here = min(HB, kv_head * group + group - head0);
-
-  // The workgroup's tile: up to 64 consecutive tokens of one sequence.
-  const int token0 = tile_token[tile_index];
-  const int count = tile_count[tile_index];
-  const int32_t* table = block_table + static_cast<int64_t>(tile_seq[tile_index]) * max_blocks;
-  const int first_pos = positions[token0];
-  const int last_key = first_pos + count - 1;          // all keys up to it are written
-  const int first_lo = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
-  const int t0 = first_lo / kTileKeys;
-  const int t1 = last_key / kTileKeys + 1;
-
-  // The wave's columns: with one head 32 tokens, else 16 tokens of two heads.
-  const int wave_token = HB == 1 ? kWaveColumns * wave : 16 * wave;
-  const int wave_span = HB == 1 ? kWaveColumns : 16;
-  const int my_head = HB == 1 ? 0 : (column >> 4);
-  const int my_local = HB == 1 ? column : (column & 15);
-  const int my_count = max(0, min(wave_span, count - wave_token));
-  // a column past the wave's tokens repeats the last one and is not stored
-  const int64_t my_token = token0 + (my_count > 0 ? wave_token + min(my_local, my_count - 1) : 0);
-  const bool head_live = my_head < heads_here;
-  const int pos = positions[my_token];
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int wave_first_pos = first_pos + wave_token;
-  const int wave_last_key = my_count > 0 ? wave_first_pos + my_count - 1 : -1;
-  const int wave_first_lo = (window > 0 && wave_first_pos - window + 1 > 0) ? wave_first_pos - window + 1 : 0;
-  const int wave_last_lo = (window > 0 && wave_last_key - window + 1 > 0) ? wave_last_key - window + 1 : 0;
   const float scale_log2 = scale * 1.4426950408889634f;
-
-  bf16x8 q_reg[KS];
-#pragma unroll
-  for (int step = 0; step < KS; ++step)
-    q_reg[step] = head_live ? ms::load_bf16x8(q + (my_token * num_q_heads + head0 + my_head) * D + 16 * step + 8 * h)
-                            : ms::zero_bf16x8();
-
-  PrefillState<D> st;
-#pragma unroll
-  for (int c = 0; c < CS; ++c)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) st.o[c][v] = 0.f;
-  st.run_max = -INFINITY;
-  st.run_sum = 0.f;
-
-  // Two pairs in flight in registers, two buffers in LDS for each half: the loads of a
-  // pair are issued two rounds before it is consumed (a round is shorter than the way
-  // to memory and back).  No branch stands between a load and its use; both halves make
-  // the same number of rounds, two to a turn of the loop so that each pair in flight has
-  // registers of its own.
-  StagedPair<D, HALF_THREADS> ahead[2];
-  PairPages pages[2];
   const int64_t page_stride = static_cast<int64_t>(num_kv_heads) * block_size * D;
   const int head_base = kv_head * block_size * D;
+
+  // The tiles come sorted by the keys they walk, fewest first.  Long tiles go out first;
+  // a paired workgroup takes the b-th longest and then the b-th shortest.
+  const int passes = (paired && static_cast<int>(blockIdx.x) != num_tiles - 1 - static_cast<int>(blockIdx.x)) ? 2 : 1;
+#pragma unroll 1
+  for (int pass = 0; pass < passes; ++pass) {
+    const int tile_index = pass == 0 ? num_tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x);
+    if (pass > 0) __syncthreads();      // the hand-over of the tile before is read
+
+    // The workgroup's tile: up to 64 consecutive tokens of one sequence.
+    const int token0 = tile_token[tile_index];
+    const int count = tile_count[tile_index];
+    const int32_t* table = block_table + static_cast<int64_t>(tile_seq[tile_index]) * max_blocks;
+    const int first_pos = positions[token0];
+    const int last_key = first_pos + count - 1;          // all keys up to it are written
+    const int first_lo = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+    const int t0 = first_lo / kTileKeys;
+    const int t1 = last_key / kTileKeys + 1;
+
+    // The wave's columns: with one head 32 tokens, else 16 tokens of two heads.
+    const int wave_token = HB == 1 ? kWaveColumns * wave : 16 * wave;
+    const int wave_span = HB == 1 ? kWaveColumns : 16;
+    const int my_head = HB == 1 ? 0 : (column >> 4);
+    const int my_local = HB == 1 ? column : (column & 15);
+    const int my_count = max(0, min(wave_span, count - wave_token));
+    // a column past the wave's tokens repeats the last one and is not stored
+    const int64_t my_token = token0 + (my_count > 0 ? wave_token + min(my_local, my_count - 1) : 0);
+    const bool head_live = my_head < heads_here;
+    const int pos = positions[my_token];
+    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int wave_first_pos = first_pos + wave_token;
+    const int wave_last_key = my_count > 0 ? wave_first_pos + my_count - 1 : -1;
+    const int wave_first_lo = (window > 0 && wave_first_pos - window + 1 > 0) ? wave_first_pos - window + 1 : 0;
+    const int wave_last_lo = (window > 0 && wave_last_key - window + 1 > 0) ? wave_last_key - window + 1 : 0;
+
+    bf16x8 q_reg[KS];
 #pragma unroll
-  for (int parity = 0; parity < 2; ++parity) {
-    stage_load<D, HALF_THREADS>(ahead[parity], thread, find_pair(t0 + 2 * half_id + 4 * parity, t1, table, block_size),
-                                key_pool, value_pool, page_stride, head_base, block_size);
-    pages[parity] = find_pair(t0 + 2 * half_id + 4 * parity + 8, t1, table, block_size);
-  }
-  for (int round_tile = t0; round_tile < t1; round_tile += 8) {
+    for (int step = 0; step < KS; ++step)
+      q_reg[step] = head_live ? ms::load_bf16x8(q + (my_token * num_q_heads + head0 + my_head) * D + 16 * step + 8 * h)
+                              : ms::zero_bf16x8();
+
+    PrefillState<D> st;
 #pragma unroll
-    for (int parity = 0; parity < 2; ++parity) {
-      const int t = round_tile + 4 * parity + 2 * half_id;
-      PairBuffer<D>& buffer = buffers[2 * parity + half_id];
-      stage_store<D, HALF_THREADS>(ahead[parity], thread, buffer);
-      stage_load<D, HALF_THREADS>(ahead[parity], thread, pages[parity], key_pool, value_pool, page_stride, head_base,
-                                  block_size);
-      pages[parity] = find_pair(t + 16, t1, table, block_size);
-      __syncthreads();    // the pair is in LDS; every wave is done with the other buffers' previous content
-      if (t < t1 && t * kTileKeys <= wave_last_key && (t + 2) * kTileKeys > wave_first_lo) {
-        // every key of the pair visible to every column of the wave: no masks
-        const bool all_visible = (t + 2) * kTileKeys - 1 <= wave_first_pos && t * kTileKeys >= wave_last_lo;
-        consume_pair<D>(st, buffer, q_reg, t * kTileKeys, lo, pos, last_key, scale_log2, h, column, !all_visible);
+    for (int c = 0; c < CS; ++c)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) st.o[c][v] = 0.f;
+    st.run_max = -INFINITY;
+    st.run_sum = 0.f;
+
+    // Pairs in flight in registers, two buffers in LDS for each part: the loads of a pair
+    // are issued kDepth rounds before it is consumed (a round is shorter than the way to
+    // memory and back), two where the registers hold two (a part of 128 threads stages
+    // twice as much a thread, and two pairs would spill).  No branch stands between a load
+    // and its use; all parts make the same number of rounds, two to a turn of the loop so
+    // that each buffer and each pair in flight is named at compile time.  A round is
+    // 2 PARTS tiles of keys.
+    constexpr int kRound = 2 * PARTS;
+    constexpr int kDepth = StagedPair<D, PART_THREADS>::kPerTile > 1 ? 1 : 2;
+    StagedPair<D, PART_THREADS> ahead[kDepth];
+    PairPages pages[kDepth];
+#pragma unroll
+    for (int i = 0; i < kDepth; ++i) {
+      const int first = t0 + 2 * part_id + kRound * i;
+      stage_load<D, PART_THREADS>(ahead[i], thread, find_pair(first, t1, table, block_size), key_pool, value_pool,
+                                  page_stride, head_base, block_size);
+      pages[i] = find_pair(first + kDepth * kRound, t1, table, block_size);
+    }
+    for (int round_tile = t0; round_tile < t1; round_tile += 2 * kRound) {
+#pragma unroll
+      for (int parity = 0; parity < 2; ++parity) {
+        constexpr int kUnused = 0;
+        const int i = kDepth == 2 ? parity : kUnused;
+        const int t = round_tile + kRound * parity + 2 * part_id;
+        PairBuffer<D>& buffer = buffers[PARTS * parity + part_id];
+        stage_store<D, PART_THREADS>(ahead[i], thread, buffer);
+        stage_load<D, PART_THREADS>(ahead[i], thread, pages[i], key_pool, value_pool, page_stride, head_base,
+                                    block_size);
+        pages[i] = find_pair(t + 2 * kDepth * kRound, t1, table, block_size);
+        __syncthreads();    // the pair is in LDS; every wave is done with the other buffers' previous content
+        if (t < t1 && t * kTileKeys <= wave_last_key && (t + 2) * kTileKeys > wave_first_lo) {
+          // every key of the pair visible to every column of the wave: no masks
+          const bool all_visible = (t + 2) * kTileKeys - 1 <= wave_first_pos && t * kTileKeys >= wave_last_lo;
+          consume_pair<D>(st, buffer, q_reg, t * kTileKeys, lo, pos, last_key, scale_log2, h, column, !all_visible);
+        }
       }
     }
-  }
 
-  // The second half hands over; the two states of a column are joined as two steps
-  // of the online softmax are.
-#pragma unroll 1
-  for (int first_wave = 0; first_wave < HALF_WAVES; first_wave += kMergeWaves) {
+    // The other parts hand over; the states of a column are joined as steps of the
+    // online softmax are.
     __syncthreads();    // everybody is done with what the memory held before
-    const bool in_round = wave >= first_wave && wave < first_wave + kMergeWaves;
-    MergeSlot<D>& slot = slots[wave - first_wave];
-    if (in_round && half_id == 1) {
+    if (part_id > 0) {
+      MergeSlot<D>& slot = slots[(part_id - 1) * PART_WAVES + wave];
 #pragma unroll
       for (int c = 0; c < CS; ++c)
 #pragma unroll
@@ -379,67 +404,71 @@ __global__ __launch_bounds__(256 * HB) MS_WAVES_PER_EU(2, 2) void attention_pref
       slot.value[16 * CS + 1][lane] = st.run_sum;
     }
     __syncthreads();
-    if (in_round && half_id == 0) {
+    if (part_id > 0) continue;
+#pragma unroll 1
+    for (int other = 1; other < PARTS; ++other) {
+      const MergeSlot<D>& slot = slots[(other - 1) * PART_WAVES + wave];
       const float other_max = slot.value[16 * CS][lane];
       const float joint = fmaxf(st.run_max, other_max);
-      // a half may have seen no key of a column: its share is zero
+      // a part may have seen no key of a column: its share is zero
       const float mine = st.run_max == -INFINITY ? 0.f : ms::fast_exp2(st.run_max - joint);
       const float theirs = other_max == -INFINITY ? 0.f : ms::fast_exp2(other_max - joint);
       st.run_sum = st.run_sum * mine + slot.value[16 * CS + 1][lane] * theirs;
+      st.run_max = joint;
 #pragma unroll
       for (int c = 0; c < CS; ++c)
 #pragma unroll
         for (int v = 0; v < 16; ++v) st.o[c][v] = st.o[c][v] * mine + slot.value[16 * c + v][lane] * theirs;
     }
-  }
-  if (half_id == 1) return;
 
-  // this lane: column's rows d = 32 c + 8 (v / 4) + 4 h + v % 4; its sum is shared with lane + 32
-  const float total = st.run_sum + __shfl_xor(st.run_sum, 32, ms::kWave);
-  const float inv = 1.0f / total;
-  if (!head_live || my_local >= my_count) return;
-  bf16* dst = out + (my_token * num_q_heads + head0 + my_head) * D;
+    // this lane: column's rows d = 32 c + 8 (v / 4) + 4 h + v % 4; its sum is shared with lane + 32
+    const float total = st.run_sum + __shfl_xor(st.run_sum, 32, ms::kWave);
+    const float inv = 1.0f / total;
+    if (!head_live || my_local >= my_count) continue;
+    bf16* dst = out + (my_token * num_q_heads + head0 + my_head) * D;
 #pragma unroll
-  for (int c = 0; c < CS; ++c)
+    for (int c = 0; c < CS; ++c)
 #pragma unroll
-    for (int quad = 0; quad < 4; ++quad) {
-      const int d = 32 * c + 8 * quad + 4 * h;
-      if (D % 32 != 0 && d >= D) continue;
-      const uint32_t low = static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad] * inv)) |
-                           (static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 1] * inv)) << 16);
-      const uint32_t high = static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 2] * inv)) |
-                            (static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 3] * inv)) << 16);
-      *reinterpret_cast<uint2*>(dst + d) = make_uint2(low, high);
-    }
+      for (int quad = 0; quad < 4; ++quad) {
+        const int d = 32 * c + 8 * quad + 4 * h;
+        if (D % 32 != 0 && d >= D) continue;
+        const uint32_t low = static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad] * inv)) |
+                             (static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 1] * inv)) << 16);
+        const uint32_t high = static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 2] * inv)) |
+                              (static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 3] * inv)) << 16);
+        *reinterpret_cast<uint2*>(dst + d) = make_uint2(low, high);
+      }
+  }
 }
 
-template <int D, int HB>
+template <int D, int HB, int PARTS>
 void launch_prefill(const void* q, const void* key_pool, const void* value_pool, const void* block_table,
                     const void* positions, const void* tile_seq, const void* tile_token, const void* tile_count,
-                    void* out, int num_tiles, int num_q_heads, int num_kv_heads, int block_size, int max_blocks,
-                    float scale, int window, hipStream_t stream) {
+                    void* out, int num_tiles, int paired, int num_q_heads, int num_kv_heads, int block_size,
+                    int max_blocks, float scale, int window, hipStream_t stream) {
   const int head_blocks = (num_q_heads / num_kv_heads + HB - 1) / HB;
-  const dim3 grid(num_tiles, num_kv_heads * head_blocks);
-  hipLaunchKernelGGL((attention_prefill_kernel<D, HB>), grid, dim3(256 * HB), 0, stream, static_cast<const bf16*>(q),
-                     static_cast<const bf16*>(key_pool), static_cast<const bf16*>(value_pool),
-                     static_cast<const int32_t*>(block_table), static_cast<const int32_t*>(positions),
-                     static_cast<const int32_t*>(tile_seq), static_cast<const int32_t*>(tile_token),
-                     static_cast<const int32_t*>(tile_count), static_cast<bf16*>(out), num_q_heads, num_kv_heads,
-                     block_size, max_blocks, scale, window);
+  const dim3 grid(paired ? (num_tiles + 1) / 2 : num_tiles, num_kv_heads * head_blocks);
+  hipLaunchKernelGGL((attention_prefill_kernel<D, HB, PARTS>), grid, dim3(128 * HB * PARTS), 0, stream,
+                     static_cast<const bf16*>(q), static_cast<const bf16*>(key_pool),
+                     static_cast<const bf16*>(value_pool), static_cast<const int32_t*>(block_table),
+                     static_cast<const int32_t*>(positions), static_cast<const int32_t*>(tile_seq),
+                     static_cast<const int32_t*>(tile_token), static_cast<const int32_t*>(tile_count),
+                     static_cast<bf16*>(out), num_tiles, paired, num_q_heads, num_kv_heads, block_size, max_blocks,
+                     scale, window);
 }
 
 template <int D>
 void launch_prefill_heads(int hb, const void* q, const void* key_pool, const void* value_pool,
                           const void* block_table, const void* positions, const void* tile_seq,
-                          const void* tile_token, const void* tile_count, void* out, int num_tiles, int num_q_heads,
-                          int num_kv_heads, int block_size, int max_blocks, float scale, int window,
+                          const void* tile_token, const void* tile_count, void* out, int num_tiles, int paired,
+                          int num_q_heads, int num_kv_heads, int block_size, int max_blocks, float scale, int window,
                           hipStream_t stream) {
   if (hb == 1) {
-    launch_prefill<D, 1>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
-                         num_tiles, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, stream);
+    launch_prefill<D, 1, 4>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
+                            num_tiles, paired, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, stream);
   } else {
-    launch_prefill<D, 2>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
-                         num_tiles, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, stream);
+    launch_prefill<D, 2, 2>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
+                            num_tiles, paired, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, stream);
   }
 }
 
@@ -456,11 +485,14 @@ extern "C" int ms_attention_prefill_supported(int head_dim, int block_size) {
 // positions: int32 [num_tokens].  The query tokens are cut into num_tiles tiles of
 // at most 64 consecutive tokens of one sequence: tile_seq (row of block_table),
 // tile_token (index of its first token), tile_count (1..64), all int32 [num_tiles].
+// tiles_sorted: the tiles come in the order of the keys they walk, fewest first (then
+// a workgroup may take a long and a short one; in any other order every workgroup
+// takes one tile).
 extern "C" int ms_attention_prefill(const void* q, const void* key_pool, const void* value_pool,
                                     const void* block_table, const void* positions, const void* tile_seq,
                                     const void* tile_token, const void* tile_count, void* out, int num_tiles,
-                                    int num_q_heads, int num_kv_heads, int head_dim, int block_size, int max_blocks,
-                                    float scale, int window, hipStream_t stream) {
+                                    int tiles_sorted, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+                                    int max_blocks, float scale, int window, hipStream_t stream) {
   MS_REQUIRE(num_tiles > 0, "attention_prefill: no tiles");
   MS_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0,
              "attention_prefill: %d query heads are not a multiple of %d kv heads", num_q_heads, num_kv_heads);
@@ -472,13 +504,27 @@ extern "C" int ms_attention_prefill(const void* q, const void* key_pool, const v
   MS_REQUIRE(static_cast<int64_t>(num_kv_heads) * block_size * head_dim < (int64_t{1} << 31),
              "attention_prefill: a page of %d kv heads x %d keys x %d is too large", num_kv_heads, block_size, head_dim);
   const int group = num_q_heads / num_kv_heads;
-  const int hb = group >= 2 ? 2 : 1;   // query heads of one workgroup
+  // Two query heads of a kv head to a workgroup (every key and value loaded serves both,
+  // the keys dealt out to two parts) where that gives the chip workgroups enough to be
+  // handed out in pairs; a smaller launch, and one whose kv heads have one query head
+  // each, takes one head a workgroup and deals the keys out to four parts: twice the
+  // workgroups, and half the steps for the longest tile (1,024 tokens of 16 heads:
+  // 25.6 -> 21.0 us; 2,048: 42.3 -> 40.8 us).
+  const int64_t with_two = static_cast<int64_t>(num_tiles) * num_kv_heads * ((group + 1) / 2);
+  const int hb = (group >= 2 && with_two >= kPairedFrom) ? 2 : 1;
+  const int64_t workgroups = static_cast<int64_t>(num_tiles) * num_kv_heads * ((group + hb - 1) / hb);
+  // A long and a short tile to a workgroup where the pairs still fill the chip (256
+  // compute units hold one workgroup each): then every workgroup walks about the same
+  // number of keys (8,192 tokens of 16 heads: 396 -> 294 us).  A small launch keeps a tile
+  // a workgroup: the longest tile sets its time either way, and a second tile costs a
+  // workgroup a second start.
+  const int paired = tiles_sorted && workgroups >= kPairedFrom;
   MS_REQUIRE(num_kv_heads * ((group + hb - 1) / hb) <= 65535, "attention_prefill: too many heads");
 #define MS_PREFILL_CASE(DIM)                                                                                       \
   case DIM:                                                                                                        \
     launch_prefill_heads<DIM>(hb, q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, \
-                              out, num_tiles, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window,     \
-                              stream);                                                                             \
+                              out, num_tiles, paired, num_q_heads, num_kv_heads, block_size, max_blocks, scale,     \
+                              window, stream);                                                                     \
     break;
   switch (head_dim) {
     MS_PREFILL_CASE(16) MS_PREFILL_CASE(32) MS_PREFILL_CASE(48) MS_PREFILL_CASE(64) MS_PREFILL_CASE(80)

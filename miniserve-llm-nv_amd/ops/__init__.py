@@ -236,23 +236,27 @@ class QueryTiles:
     seq: torch.Tensor       # int32 [count]: the tile's sequence (row of the block tables)
     token: torch.Tensor     # int32 [count]: index of the tile's first token in the batch
     length: torch.Tensor    # int32 [count]: 1..PREFILL_TILE_TOKENS
+    by_keys: bool = False   # the tiles stand in the order of the keys they walk, fewest first
 
 
-def query_tiles_host(query_lens, query_start, decode_prefix: int) -> tuple[list[int], list[int], list[int]]:
+def query_tiles_host(query_lens, query_start, decode_prefix: int, first_positions=None) -> tuple[list[int], list[int], list[int]]:
     """The tiles of a batch as three lists (sequence, first token, length): every
     sequence after the first ``decode_prefix`` is cut into runs of at most
-    ``PREFILL_TILE_TOKENS`` tokens."""
+    ``PREFILL_TILE_TOKENS`` tokens.  With ``first_positions`` (the position of every
+    sequence's first token of the step) the tiles are put in the order of the keys they
+    walk, fewest first (``QueryTiles.by_keys``): the kernel then hands the long ones out
+    first and may give a workgroup a long and a short one."""
 
-    seqs: list[int] = []
-    tokens: list[int] = []
-    lengths: list[int] = []
+    tiles: list[tuple[int, int, int, int]] = []
     for index in range(decode_prefix, len(query_lens)):
         base, length = query_start[index], query_lens[index]
+        first = first_positions[index] if first_positions is not None else 0
         for start in range(0, length, PREFILL_TILE_TOKENS):
-            seqs.append(index)
-            tokens.append(base + start)
-            lengths.append(min(PREFILL_TILE_TOKENS, length - start))
-    return seqs, tokens, lengths
+            count = min(PREFILL_TILE_TOKENS, length - start)
+            tiles.append((first + start + count, index, base + start, count))
+    if first_positions is not None:
+        tiles.sort()
+    return [t[1] for t in tiles], [t[2] for t in tiles], [t[3] for t in tiles]
 
 
 # calls of attention() served by each kernel since the import; a bfloat16 call that no
@@ -372,8 +376,8 @@ def attention(
             for name in ("seq", "token", "length"):
                 _check(getattr(tiles, name), f"tiles.{name}", dtype=torch.int32, shape=(tiles.count,))
             call("ms_attention_prefill", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(positions),
-                 _ptr(tiles.seq), _ptr(tiles.token), _ptr(tiles.length), _ptr(out), tiles.count, heads, kv_heads,
-                 head_dim, block_size, max_blocks, float(scale), window, _stream())
+                 _ptr(tiles.seq), _ptr(tiles.token), _ptr(tiles.length), _ptr(out), tiles.count, int(tiles.by_keys),
+                 heads, kv_heads, head_dim, block_size, max_blocks, float(scale), window, _stream())
         return out
     attention_calls["generic"] += 1
     if q.dtype == torch.bfloat16 and not lib.ms_attention_decode_supported(head_dim, block_size):

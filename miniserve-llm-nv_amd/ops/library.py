@@ -30,7 +30,7 @@ _SIGNATURES: dict[str, list] = {
     "ms_attention_generic": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ms_attention_decode": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ms_attention_decode_supported": [_I, _I],
-    "ms_attention_prefill": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "ms_attention_prefill": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "ms_attention_prefill_supported": [_I, _I],
     "ms_gemm_f32": [_P, _P, _P, _I, _I, _I, _I, _P],
     "ms_gemm_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _P],

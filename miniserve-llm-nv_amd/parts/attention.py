@@ -95,7 +95,8 @@ class Attention(Part):
 
     @staticmethod
     def step_tables(batch: HostBatch) -> dict[str, list[int]]:
-        seqs, tokens, lengths = ops.query_tiles_host(batch.query_lens, batch.query_start, batch.decode_prefix)
+        seqs, tokens, lengths = ops.query_tiles_host(batch.query_lens, batch.query_start, batch.decode_prefix,
+                                                     batch.first_positions)
         return {"attention.tile_seq": seqs, "attention.tile_token": tokens, "attention.tile_length": lengths}
 
     @staticmethod
@@ -104,7 +105,8 @@ class Attention(Part):
             seq = ctx.tables.get("attention.tile_seq")
             tiles = None
             if seq is not None and seq.numel() > 0:
-                tiles = ops.QueryTiles(seq.numel(), seq, ctx.tables["attention.tile_token"], ctx.tables["attention.tile_length"])
+                tiles = ops.QueryTiles(seq.numel(), seq, ctx.tables["attention.tile_token"],
+                                       ctx.tables["attention.tile_length"], by_keys=True)
             ctx.scratch["attention.tiles"] = tiles
         return ctx.scratch["attention.tiles"]
 

@@ -294,10 +294,12 @@ def attention_reference(case, scale, window=None):
     return torch.cat(outs)
 
 
-def query_tiles(case, first_sequence):
-    """Tiles of at most 64 consecutive tokens for the sequences from ``first_sequence`` on."""
+def query_tiles(case, first_sequence, by_keys=False):
+    """Tiles of at most 64 consecutive tokens for the sequences from ``first_sequence`` on,
+    in the order of the batch, or (``by_keys``) as the attention part makes them: in the
+    order of the keys they walk."""
 
-    from miniserve_amd.ops import QueryTiles
+    from miniserve_amd.ops import QueryTiles, query_tiles_host
 
     seqs, tokens, lengths, base = [], [], [], 0
     for index, qlen in enumerate(case["query_lens"]):
@@ -309,12 +311,18 @@ def query_tiles(case, first_sequence):
         base += qlen
     if not seqs:
         return None
+    if by_keys:
+        starts = [0]
+        for qlen in case["query_lens"]:
+            starts.append(starts[-1] + qlen)
+        firsts = [int(case["positions"][start]) for start in starts[:-1]]
+        seqs, tokens, lengths = query_tiles_host(case["query_lens"], starts[:-1], first_sequence, firsts)
     device = case["q"].device
     as_tensor = lambda values: torch.tensor(values, dtype=torch.int32, device=device)
-    return QueryTiles(len(seqs), as_tensor(seqs), as_tensor(tokens), as_tensor(lengths))
+    return QueryTiles(len(seqs), as_tensor(seqs), as_tensor(tokens), as_tensor(lengths), by_keys=by_keys)
 
 
-def run_attention(ops, case, scale, window=None, splits=None):
+def run_attention(ops, case, scale, window=None, splits=None, by_keys=False):
     """As the engine calls it: sequences that bring one token stand first and are
     served as single tokens, the others in tiles."""
 
@@ -324,7 +332,7 @@ def run_attention(ops, case, scale, window=None, splits=None):
         prefix += 1
     return ops.attention(case["q"], case["key_pool"], case["value_pool"], block_table=case["block_table"],
                          seq_of_token=case["seq_of_token"], positions=case["positions"], scale=scale, window=window,
-                         decode_prefix=prefix, tiles=query_tiles(case, prefix),
+                         decode_prefix=prefix, tiles=query_tiles(case, prefix, by_keys),
                          max_context=int(case["positions"].max()) + 1, splits=splits)
 
 
@@ -438,19 +446,25 @@ def test_tiled_kernel_sizes_portions_and_windows(ops, heads, kv_heads, dim, bloc
         torch.testing.assert_close(out.cpu().double(), expected, atol=ATTENTION_BF16, rtol=ATTENTION_BF16, msg=lambda m: f"window {window}: {m}")
 
 
+@pytest.mark.parametrize("by_keys", [False, True])
 @pytest.mark.parametrize("contexts,query_lens,heads,kv_heads,dim", [
-    ([2048], [2048], 16, 8, 128),                 # a prompt of the served sizes: 32 tiles, the last walks 2,048 keys
+    ([2048], [2048], 16, 8, 128),                 # a prompt of the served sizes: 32 tiles, the last walks 2,048 keys;
+                                                  # one head and four parts a workgroup, a long and a short tile each
     ([1100, 1200], [1100, 1200], 32, 8, 64),      # two prompts, two workgroups of heads to a kv head
     ([700, 300, 40], [500, 33, 40], 4, 1, 32),    # portions with history, an odd tail
     ([1500] * 3, [1000] * 3, 4, 4, 48),           # one head a workgroup
+    ([1990, 130], [1990 - 64, 130], 16, 8, 128),  # an odd number of tiles: the middle one has a workgroup to itself
+    ([3000], [3000], 40, 8, 128),                 # two heads a workgroup, tiles in pairs
 ])
-def test_tiled_kernel_over_long_prompts(ops, contexts, query_lens, heads, kv_heads, dim):
+def test_tiled_kernel_over_long_prompts(ops, contexts, query_lens, heads, kv_heads, dim, by_keys):
     """Prompts of a thousand tokens and more (dozens of tiles, walks of thousands of
-    keys), against the plain attention, with a window as well."""
+    keys), against the plain attention, with a window as well; the tiles in the order of
+    the batch (a tile a workgroup) and in the order of their keys (where the launch is
+    small, a long and a short tile a workgroup)."""
 
     case = paged_case(contexts, heads, kv_heads, dim, 16, torch.bfloat16, query_lens=query_lens, seed=dim)
     for window in (None, 300):
-        out = run_attention(ops, case, dim**-0.5, window=window)
+        out = run_attention(ops, case, dim**-0.5, window=window, by_keys=by_keys)
         expected = attention_reference(case, dim**-0.5, window=window)
         torch.testing.assert_close(out.cpu().double(), expected, atol=ATTENTION_BF16, rtol=ATTENTION_BF16,
                                    msg=lambda m: f"window {window}: {m}")
