@@ -33,7 +33,9 @@ class StepEntry:
             return          # a decoded token: the common case, checked without loops
         if not self.token_ids:
             raise ValueError(f"entry {self.request_id!r} brings no tokens.")
-        if any(not isinstance(t, int) or isinstance(t, bool) or t < 0 for t in self.token_ids):
+        # a portion of a prompt has hundreds of tokens: their types and their least are taken
+        # without a Python-level loop (a bool is an int to isinstance, not to type)
+        if set(map(type, self.token_ids)) != {int} or min(self.token_ids) < 0:
             raise ValueError(f"entry {self.request_id!r}: token ids must be non-negative integers.")
         if any(not isinstance(w, int) or isinstance(w, bool) or not 0 <= w < len(self.token_ids) for w in self.want):
             raise ValueError(f"entry {self.request_id!r}: wanted places must index its tokens.")

@@ -38,6 +38,16 @@ class GenerationResult:
     num_preemptions: int = 0
 
 
+def _longest_first(decode_items):
+    """The rows of single tokens in the order in which the step runs them: the longest
+    context first (equal ones stay in the scheduler's order).  The attention kernel's
+    workgroups start in row order, and a step takes as long as its last workgroup: a long
+    row that starts late would run on after the others (64 rows of 128 to 2,200 keys:
+    75 us a layer in random order, 69 us longest first)."""
+
+    return sorted(decode_items, key=lambda item: -item.position)
+
+
 @dataclass(frozen=True)
 class _StepAhead:
     version: int            # of the engine's request set when the step was planned
@@ -158,7 +168,7 @@ class Engine:
 
         entries: list[StepEntry] = []
         sampled: list[SequenceState] = []
-        for item in plan.decode_items:
+        for item in _longest_first(plan.decode_items):
             state = self._sequences[item.request_id]
             # (a step planned ahead did not know the token yet)
             entries.append(StepEntry(item.request_id, (state.token_at(state.computed_tokens),), (0,)))
@@ -279,10 +289,10 @@ class Engine:
             return None
         try:
             if not next_plan.prefill_items:
-                prepared = prepare_decode([item.request_id for item in next_plan.decode_items])
+                prepared = prepare_decode([item.request_id for item in _longest_first(next_plan.decode_items)])
             elif prepare_step is not None:
                 entries, admit = [], []
-                for item in next_plan.decode_items:
+                for item in _longest_first(next_plan.decode_items):
                     state = self._sequences[item.request_id]
                     token = 0 if item.request_id in sampled_ids else state.token_at(state.computed_tokens)
                     entries.append(StepEntry(item.request_id, (token,), (0,)))

@@ -316,6 +316,35 @@ def test_generate_is_the_same_whatever_the_scheduling():
     runner.cache.assert_invariants()
 
 
+def test_decoded_tokens_run_longest_context_first():
+    """The rows of single decoded tokens of a step stand first, in the order of their
+    contexts, the longest first, with and without steps planned ahead; the portions of
+    prompts follow in the plan's order."""
+
+    for ahead in (False, True):
+        engine, runner = make_engine(enable_chunked_prefill=True, prefill_chunk_size=8, max_num_batched_tokens=16)
+        runner.prepare_ahead = ahead
+        for index, prompt in enumerate(PROMPTS):
+            engine.add_request(f"r{index}", prompt, SamplingParams(max_new_tokens=12), arrival_ns=index)
+        decided = 0
+        while engine.has_unfinished():
+            before = len(runner.steps)
+            engine.step()
+            plan = engine.last_plan
+            if plan.empty:
+                continue
+            assert len(runner.steps) == before + 1
+            rows = runner.steps[-1]
+            decoded = {item.request_id: item.position for item in plan.decode_items}
+            first = rows[: len(decoded)]
+            assert {request for request, _, _ in first} == set(decoded)
+            starts = [start for _, start, _ in first]
+            assert starts == sorted(starts, reverse=True) and all(decoded[r] == start for r, start, _ in first)
+            assert [request for request, _, _ in rows[len(decoded):]] == [item.request_id for item in plan.prefill_items]
+            decided += len(set(starts)) > 1 and starts != sorted(decoded.values())
+        assert decided >= 5                                             # steps in which the order had something to decide
+
+
 def test_steps_planned_ahead_change_no_token():
     """While a step of decoding requests runs, the next one is scheduled and its cache
     transaction opened; what the requests generate is what they generate without that,
