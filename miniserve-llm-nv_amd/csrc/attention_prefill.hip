@@ -255,38 +255,49 @@ __device__ __forceinline__ void consume_pair(PrefillState<D>& st, const PairBuff
     for (int j = 0; j < 2; ++j) st.o[c] = ms::mfma_32x32x16(values[c][j], p[j], st.o[c]);
 }
 
-// What a part of a workgroup hands to the first part at the end: every register of the
-// state, lane by lane.
-template <int D>
+// At the end the parts of a workgroup share the finishing: of the blocks of 32 rows of
+// O^T, block c is finished (joined over the parts, divided by the sum, stored) by part
+// c % PARTS.  What a wave publishes for that: its maximum, its sum, and the blocks that
+// another part finishes, lane by lane.
+template <int D, int PARTS>
 struct MergeSlot {
-  float value[PrefillState<D>::CS * 16 + 2][ms::kWave];
+  static constexpr int CS = PrefillState<D>::CS;
+  static constexpr int kBlocks = CS - CS / PARTS;      // most blocks that a part does not finish itself
+  float value[kBlocks * 16 + 2][ms::kWave];
+  // where part `part` keeps block c (which it does not finish): behind its other such blocks
+  __device__ static __forceinline__ int place(int part, int c) {
+    const int own_below = c > part ? (c - part - 1) / PARTS + 1 : 0;
+    return c - own_below;
+  }
 };
 
 template <int D, int HB, int PARTS>
 constexpr size_t prefill_lds_bytes() {
   constexpr size_t buffers = 2 * PARTS * sizeof(PairBuffer<D>);
-  constexpr size_t slots = (PARTS - 1) * 2 * HB * sizeof(MergeSlot<D>);
+  constexpr size_t slots = PARTS * 2 * HB * sizeof(MergeSlot<D, PARTS>);
   return buffers > slots ? buffers : slots;
 }
 
 template <int D, int HB, int PARTS>
 __global__ __launch_bounds__(128 * HB * PARTS) MS_WAVES_PER_EU(2, 2) void attention_prefill_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ key_pool, const bf16* __restrict__ value_pool,
-    const int32_t* __restrict__ block_table, const int32_t* __restrict__ positions,
-    const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_token, const int32_t* __restrict__ tile_count,
-    bf16* __restrict__ out, int num_tiles, int paired, int num_q_heads, int num_kv_heads, int block_size,
+    const int32_t* __restrict__ block_table, const int32_t* __restrict__ tile_seq,
+    const int32_t* __restrict__ tile_token, const int32_t* __restrict__ tile_count,
+    const int32_t* __restrict__ tile_first, bf16* __restrict__ out, int num_tiles, int paired, int num_q_heads, int num_kv_heads, int block_size,
     int max_blocks, float scale, int window) {
   // The workgroup is PARTS parts of 2 HB waves.  All hold the same 64 HB columns; part p
   // takes the pairs of key tiles p, p + PARTS, p + 2 PARTS, ... of the tile's range: two
   // waves on every SIMD, one in the matrix cores while the other is in its softmax, and
   // 1 / PARTS of the steps for the longest tile.  Each part loads its own pairs into its
-  // own LDS buffers; at the end the others hand their states to the first through LDS.
+  // own LDS buffers; at the end they exchange their states through LDS and each finishes
+  // a share of the outputs.
   constexpr int PART_THREADS = 128 * HB;
   constexpr int PART_WAVES = 2 * HB;
   constexpr int KS = D / 16, CS = PrefillState<D>::CS;
   __shared__ __align__(16) unsigned char lds[prefill_lds_bytes<D, HB, PARTS>()];
   PairBuffer<D>* buffers = reinterpret_cast<PairBuffer<D>*>(lds);        // [parity][part]
-  MergeSlot<D>* slots = reinterpret_cast<MergeSlot<D>*>(lds);            // [part - 1][wave]
+  using Slot = MergeSlot<D, PARTS>;
+  Slot* slots = reinterpret_cast<Slot*>(lds);                            // [part][wave]
 
   const int lane = threadIdx.x & 63;
   const int wave_of_group = ms::uniform(threadIdx.x >> 6);   // the same in all lanes: kept in a scalar register
@@ -313,11 +324,12 @@ __global__ __launch_bounds__(128 * HB * PARTS) MS_WAVES_PER_EU(2, 2) void attent
     const int tile_index = pass == 0 ? num_tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x);
     if (pass > 0) __syncthreads();      // the hand-over of the tile before is read
 
-    // The workgroup's tile: up to 64 consecutive tokens of one sequence.
+    // The workgroup's tile: up to 64 consecutive tokens of one sequence, at consecutive
+    // positions from the tile's first (all four numbers come with one trip to memory).
     const int token0 = tile_token[tile_index];
     const int count = tile_count[tile_index];
     const int32_t* table = block_table + static_cast<int64_t>(tile_seq[tile_index]) * max_blocks;
-    const int first_pos = positions[token0];
+    const int first_pos = tile_first[tile_index];
     const int last_key = first_pos + count - 1;          // all keys up to it are written
     const int first_lo = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
     const int t0 = first_lo / kTileKeys;
@@ -330,9 +342,10 @@ __global__ __launch_bounds__(128 * HB * PARTS) MS_WAVES_PER_EU(2, 2) void attent
     const int my_local = HB == 1 ? column : (column & 15);
     const int my_count = max(0, min(wave_span, count - wave_token));
     // a column past the wave's tokens repeats the last one and is not stored
-    const int64_t my_token = token0 + (my_count > 0 ? wave_token + min(my_local, my_count - 1) : 0);
+    const int my_offset = my_count > 0 ? wave_token + min(my_local, my_count - 1) : 0;
+    const int64_t my_token = token0 + my_offset;
     const bool head_live = my_head < heads_here;
-    const int pos = positions[my_token];
+    const int pos = first_pos + my_offset;
     const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
     const int wave_first_pos = first_pos + wave_token;
     const int wave_last_key = my_count > 0 ? wave_first_pos + my_count - 1 : -1;
@@ -391,59 +404,79 @@ __global__ __launch_bounds__(128 * HB * PARTS) MS_WAVES_PER_EU(2, 2) void attent
       }
     }
 
-    // The other parts hand over; the states of a column are joined as steps of the
-    // online softmax are.
+    // The parts exchange their states; the states of a column are joined as steps of the
+    // online softmax are, the parts in their order whichever part does the sum.
     __syncthreads();    // everybody is done with what the memory held before
-    if (part_id > 0) {
-      MergeSlot<D>& slot = slots[(part_id - 1) * PART_WAVES + wave];
+    {
+      Slot& mine = slots[part_id * PART_WAVES + wave];
 #pragma unroll
-      for (int c = 0; c < CS; ++c)
+      for (int c = 0; c < CS; ++c) {
+        if (c % PARTS == part_id) continue;
+        const int at = 16 * Slot::place(part_id, c);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) slot.value[16 * c + v][lane] = st.o[c][v];
-      slot.value[16 * CS][lane] = st.run_max;
-      slot.value[16 * CS + 1][lane] = st.run_sum;
+        for (int v = 0; v < 16; ++v) mine.value[at + v][lane] = st.o[c][v];
+      }
+      mine.value[16 * Slot::kBlocks][lane] = st.run_max;
+      mine.value[16 * Slot::kBlocks + 1][lane] = st.run_sum;
     }
     __syncthreads();
-    if (part_id > 0) continue;
-#pragma unroll 1
-    for (int other = 1; other < PARTS; ++other) {
-      const MergeSlot<D>& slot = slots[(other - 1) * PART_WAVES + wave];
-      const float other_max = slot.value[16 * CS][lane];
-      const float joint = fmaxf(st.run_max, other_max);
-      // a part may have seen no key of a column: its share is zero
-      const float mine = st.run_max == -INFINITY ? 0.f : ms::fast_exp2(st.run_max - joint);
-      const float theirs = other_max == -INFINITY ? 0.f : ms::fast_exp2(other_max - joint);
-      st.run_sum = st.run_sum * mine + slot.value[16 * CS + 1][lane] * theirs;
-      st.run_max = joint;
+    if (part_id >= CS) continue;      // no block of rows is this part's to finish
+    float joint = st.run_max;
 #pragma unroll
-      for (int c = 0; c < CS; ++c)
+    for (int q = 0; q < PARTS; ++q)
+      if (q != part_id) joint = fmaxf(joint, slots[q * PART_WAVES + wave].value[16 * Slot::kBlocks][lane]);
+    // a part may have seen no key of a column: its share is zero
+    float factor[PARTS];
+    float total = 0.f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) st.o[c][v] = st.o[c][v] * mine + slot.value[16 * c + v][lane] * theirs;
+    for (int q = 0; q < PARTS; ++q) {
+      const Slot& theirs = slots[q * PART_WAVES + wave];
+      const float part_max = q == part_id ? st.run_max : theirs.value[16 * Slot::kBlocks][lane];
+      const float part_sum = q == part_id ? st.run_sum : theirs.value[16 * Slot::kBlocks + 1][lane];
+      factor[q] = part_max == -INFINITY ? 0.f : ms::fast_exp2(part_max - joint);
+      total += part_sum * factor[q];
     }
-
     // this lane: column's rows d = 32 c + 8 (v / 4) + 4 h + v % 4; its sum is shared with lane + 32
-    const float total = st.run_sum + __shfl_xor(st.run_sum, 32, ms::kWave);
+    total += __shfl_xor(total, 32, ms::kWave);
     const float inv = 1.0f / total;
-    if (!head_live || my_local >= my_count) continue;
+    const bool stores = head_live && my_local < my_count;
     bf16* dst = out + (my_token * num_q_heads + head0 + my_head) * D;
 #pragma unroll
-    for (int c = 0; c < CS; ++c)
+    for (int c = 0; c < CS; ++c) {
+      if (c % PARTS != part_id) continue;
+      float row[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) row[v] = 0.f;
+#pragma unroll
+      for (int q = 0; q < PARTS; ++q) {
+        if (q == part_id) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) row[v] = fmaf(st.o[c][v], factor[q], row[v]);
+        } else {
+          const Slot& theirs = slots[q * PART_WAVES + wave];
+          const int at = 16 * Slot::place(q, c);
+#pragma unroll
+          for (int v = 0; v < 16; ++v) row[v] = fmaf(theirs.value[at + v][lane], factor[q], row[v]);
+        }
+      }
+      if (!stores) continue;
 #pragma unroll
       for (int quad = 0; quad < 4; ++quad) {
         const int d = 32 * c + 8 * quad + 4 * h;
         if (D % 32 != 0 && d >= D) continue;
-        const uint32_t low = static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad] * inv)) |
-                             (static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 1] * inv)) << 16);
-        const uint32_t high = static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 2] * inv)) |
-                              (static_cast<uint32_t>(ms::float_to_bf16_bits(st.o[c][4 * quad + 3] * inv)) << 16);
+        const uint32_t low = static_cast<uint32_t>(ms::float_to_bf16_bits(row[4 * quad] * inv)) |
+                             (static_cast<uint32_t>(ms::float_to_bf16_bits(row[4 * quad + 1] * inv)) << 16);
+        const uint32_t high = static_cast<uint32_t>(ms::float_to_bf16_bits(row[4 * quad + 2] * inv)) |
+                              (static_cast<uint32_t>(ms::float_to_bf16_bits(row[4 * quad + 3] * inv)) << 16);
         *reinterpret_cast<uint2*>(dst + d) = make_uint2(low, high);
       }
+    }
   }
 }
 
 template <int D, int HB, int PARTS>
 void launch_prefill(const void* q, const void* key_pool, const void* value_pool, const void* block_table,
-                    const void* positions, const void* tile_seq, const void* tile_token, const void* tile_count,
+                    const void* tile_seq, const void* tile_token, const void* tile_count, const void* tile_first,
                     void* out, int num_tiles, int paired, int num_q_heads, int num_kv_heads, int block_size,
                     int max_blocks, float scale, int window, hipStream_t stream) {
   const int head_blocks = (num_q_heads / num_kv_heads + HB - 1) / HB;
@@ -451,23 +484,23 @@ void launch_prefill(const void* q, const void* key_pool, const void* value_pool,
   hipLaunchKernelGGL((attention_prefill_kernel<D, HB, PARTS>), grid, dim3(128 * HB * PARTS), 0, stream,
                      static_cast<const bf16*>(q), static_cast<const bf16*>(key_pool),
                      static_cast<const bf16*>(value_pool), static_cast<const int32_t*>(block_table),
-                     static_cast<const int32_t*>(positions), static_cast<const int32_t*>(tile_seq),
-                     static_cast<const int32_t*>(tile_token), static_cast<const int32_t*>(tile_count),
+                     static_cast<const int32_t*>(tile_seq), static_cast<const int32_t*>(tile_token),
+                     static_cast<const int32_t*>(tile_count), static_cast<const int32_t*>(tile_first),
                      static_cast<bf16*>(out), num_tiles, paired, num_q_heads, num_kv_heads, block_size, max_blocks,
                      scale, window);
 }
 
 template <int D>
 void launch_prefill_heads(int hb, const void* q, const void* key_pool, const void* value_pool,
-                          const void* block_table, const void* positions, const void* tile_seq,
-                          const void* tile_token, const void* tile_count, void* out, int num_tiles, int paired,
+                          const void* block_table, const void* tile_seq, const void* tile_token,
+                          const void* tile_count, const void* tile_first, void* out, int num_tiles, int paired,
                           int num_q_heads, int num_kv_heads, int block_size, int max_blocks, float scale, int window,
                           hipStream_t stream) {
   if (hb == 1) {
-    launch_prefill<D, 1, 4>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
+    launch_prefill<D, 1, 4>(q, key_pool, value_pool, block_table, tile_seq, tile_token, tile_count, tile_first, out,
                             num_tiles, paired, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, stream);
   } else {
-    launch_prefill<D, 2, 2>(q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, out,
+    launch_prefill<D, 2, 2>(q, key_pool, value_pool, block_table, tile_seq, tile_token, tile_count, tile_first, out,
                             num_tiles, paired, num_q_heads, num_kv_heads, block_size, max_blocks, scale, window, stream);
   }
 }
@@ -481,16 +514,17 @@ extern "C" int ms_attention_prefill_supported(int head_dim, int block_size) {
 }
 
 // q, out: bfloat16 [num_tokens, num_q_heads, head_dim]; key_pool: [pages, kv_heads,
-// block_size, head_dim]; value_pool: [pages, kv_heads, head_dim, block_size];
-// positions: int32 [num_tokens].  The query tokens are cut into num_tiles tiles of
-// at most 64 consecutive tokens of one sequence: tile_seq (row of block_table),
-// tile_token (index of its first token), tile_count (1..64), all int32 [num_tiles].
+// block_size, head_dim]; value_pool: [pages, kv_heads, head_dim, block_size].  The
+// query tokens are cut into num_tiles tiles of at most 64 consecutive tokens of one
+// sequence, at consecutive positions: tile_seq (row of block_table), tile_token (index
+// of its first token), tile_count (1..64), tile_first (position of its first token),
+// all int32 [num_tiles].
 // tiles_sorted: the tiles come in the order of the keys they walk, fewest first (then
 // a workgroup may take a long and a short one; in any other order every workgroup
 // takes one tile).
 extern "C" int ms_attention_prefill(const void* q, const void* key_pool, const void* value_pool,
-                                    const void* block_table, const void* positions, const void* tile_seq,
-                                    const void* tile_token, const void* tile_count, void* out, int num_tiles,
+                                    const void* block_table, const void* tile_seq, const void* tile_token,
+                                    const void* tile_count, const void* tile_first, void* out, int num_tiles,
                                     int tiles_sorted, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
                                     int max_blocks, float scale, int window, hipStream_t stream) {
   MS_REQUIRE(num_tiles > 0, "attention_prefill: no tiles");
@@ -522,7 +556,7 @@ extern "C" int ms_attention_prefill(const void* q, const void* key_pool, const v
   MS_REQUIRE(num_kv_heads * ((group + hb - 1) / hb) <= 65535, "attention_prefill: too many heads");
 #define MS_PREFILL_CASE(DIM)                                                                                       \
   case DIM:                                                                                                        \
-    launch_prefill_heads<DIM>(hb, q, key_pool, value_pool, block_table, positions, tile_seq, tile_token, tile_count, \
+    launch_prefill_heads<DIM>(hb, q, key_pool, value_pool, block_table, tile_seq, tile_token, tile_count, tile_first, \
                               out, num_tiles, paired, num_q_heads, num_kv_heads, block_size, max_blocks, scale,     \
                               window, stream);                                                                     \
     break;

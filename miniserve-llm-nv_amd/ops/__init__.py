@@ -236,27 +236,27 @@ class QueryTiles:
     seq: torch.Tensor       # int32 [count]: the tile's sequence (row of the block tables)
     token: torch.Tensor     # int32 [count]: index of the tile's first token in the batch
     length: torch.Tensor    # int32 [count]: 1..PREFILL_TILE_TOKENS
+    first: torch.Tensor     # int32 [count]: position of the tile's first token; the others follow one by one
     by_keys: bool = False   # the tiles stand in the order of the keys they walk, fewest first
 
 
-def query_tiles_host(query_lens, query_start, decode_prefix: int, first_positions=None) -> tuple[list[int], list[int], list[int]]:
-    """The tiles of a batch as three lists (sequence, first token, length): every
-    sequence after the first ``decode_prefix`` is cut into runs of at most
-    ``PREFILL_TILE_TOKENS`` tokens.  With ``first_positions`` (the position of every
-    sequence's first token of the step) the tiles are put in the order of the keys they
-    walk, fewest first (``QueryTiles.by_keys``): the kernel then hands the long ones out
-    first and may give a workgroup a long and a short one."""
+def query_tiles_host(query_lens, query_start, decode_prefix: int, first_positions, *, by_keys: bool = True):
+    """The tiles of a batch as four lists (sequence, first token, length, position of the
+    first token): every sequence after the first ``decode_prefix`` is cut into runs of at
+    most ``PREFILL_TILE_TOKENS`` tokens.  ``first_positions``: the position of every
+    sequence's first token of the step.  ``by_keys``: the tiles are put in the order of
+    the keys they walk, fewest first (``QueryTiles.by_keys``): the kernel then hands the
+    long ones out first and may give a workgroup a long and a short one."""
 
     tiles: list[tuple[int, int, int, int]] = []
     for index in range(decode_prefix, len(query_lens)):
-        base, length = query_start[index], query_lens[index]
-        first = first_positions[index] if first_positions is not None else 0
+        base, length, first = query_start[index], query_lens[index], first_positions[index]
         for start in range(0, length, PREFILL_TILE_TOKENS):
             count = min(PREFILL_TILE_TOKENS, length - start)
             tiles.append((first + start + count, index, base + start, count))
-    if first_positions is not None:
+    if by_keys:
         tiles.sort()
-    return [t[1] for t in tiles], [t[2] for t in tiles], [t[3] for t in tiles]
+    return [t[1] for t in tiles], [t[2] for t in tiles], [t[3] for t in tiles], [t[0] - t[3] for t in tiles]
 
 
 # calls of attention() served by each kernel since the import; a bfloat16 call that no
@@ -373,10 +373,10 @@ def attention(
                  kv_heads, head_dim, block_size, max_blocks, float(scale), window, int(splits), _stream())
         if tiled and decode_prefix < n:
             attention_calls["prefill"] += 1
-            for name in ("seq", "token", "length"):
+            for name in ("seq", "token", "length", "first"):
                 _check(getattr(tiles, name), f"tiles.{name}", dtype=torch.int32, shape=(tiles.count,))
-            call("ms_attention_prefill", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table), _ptr(positions),
-                 _ptr(tiles.seq), _ptr(tiles.token), _ptr(tiles.length), _ptr(out), tiles.count, int(tiles.by_keys),
+            call("ms_attention_prefill", _ptr(q), _ptr(key_pool), _ptr(value_pool), _ptr(block_table),
+                 _ptr(tiles.seq), _ptr(tiles.token), _ptr(tiles.length), _ptr(tiles.first), _ptr(out), tiles.count, int(tiles.by_keys),
                  heads, kv_heads, head_dim, block_size, max_blocks, float(scale), window, _stream())
         return out
     attention_calls["generic"] += 1

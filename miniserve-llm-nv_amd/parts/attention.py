@@ -95,9 +95,10 @@ class Attention(Part):
 
     @staticmethod
     def step_tables(batch: HostBatch) -> dict[str, list[int]]:
-        seqs, tokens, lengths = ops.query_tiles_host(batch.query_lens, batch.query_start, batch.decode_prefix,
-                                                     batch.first_positions)
-        return {"attention.tile_seq": seqs, "attention.tile_token": tokens, "attention.tile_length": lengths}
+        seqs, tokens, lengths, firsts = ops.query_tiles_host(batch.query_lens, batch.query_start, batch.decode_prefix,
+                                                             batch.first_positions)
+        return {"attention.tile_seq": seqs, "attention.tile_token": tokens, "attention.tile_length": lengths,
+                "attention.tile_first": firsts}
 
     @staticmethod
     def _tiles(ctx: StepContext):
@@ -106,7 +107,7 @@ class Attention(Part):
             tiles = None
             if seq is not None and seq.numel() > 0:
                 tiles = ops.QueryTiles(seq.numel(), seq, ctx.tables["attention.tile_token"],
-                                       ctx.tables["attention.tile_length"], by_keys=True)
+                                       ctx.tables["attention.tile_length"], ctx.tables["attention.tile_first"], by_keys=True)
             ctx.scratch["attention.tiles"] = tiles
         return ctx.scratch["attention.tiles"]
 

@@ -301,25 +301,16 @@ def query_tiles(case, first_sequence, by_keys=False):
 
     from miniserve_amd.ops import QueryTiles, query_tiles_host
 
-    seqs, tokens, lengths, base = [], [], [], 0
-    for index, qlen in enumerate(case["query_lens"]):
-        if index >= first_sequence:
-            for start in range(0, qlen, 64):
-                seqs.append(index)
-                tokens.append(base + start)
-                lengths.append(min(64, qlen - start))
-        base += qlen
-    if not seqs:
+    starts = [0]
+    for qlen in case["query_lens"]:
+        starts.append(starts[-1] + qlen)
+    if starts[first_sequence] == starts[-1]:
         return None
-    if by_keys:
-        starts = [0]
-        for qlen in case["query_lens"]:
-            starts.append(starts[-1] + qlen)
-        firsts = [int(case["positions"][start]) for start in starts[:-1]]
-        seqs, tokens, lengths = query_tiles_host(case["query_lens"], starts[:-1], first_sequence, firsts)
+    firsts = [int(case["positions"][start]) for start in starts[:-1]]
+    lists = query_tiles_host(case["query_lens"], starts[:-1], first_sequence, firsts, by_keys=by_keys)
     device = case["q"].device
-    as_tensor = lambda values: torch.tensor(values, dtype=torch.int32, device=device)
-    return QueryTiles(len(seqs), as_tensor(seqs), as_tensor(tokens), as_tensor(lengths), by_keys=by_keys)
+    return QueryTiles(len(lists[0]), *(torch.tensor(values, dtype=torch.int32, device=device) for values in lists),
+                      by_keys=by_keys)
 
 
 def run_attention(ops, case, scale, window=None, splits=None, by_keys=False):
@@ -511,6 +502,7 @@ def test_attention_is_bit_identical_across_batches_in_float32(ops):
     alone["q"] = torch.stack([case["q"][199], case["q"][200]])
     alone["seq_of_token"] = torch.tensor([0, 1], dtype=torch.int32, device=DEVICE)
     alone["positions"] = torch.tensor([199, 76], dtype=torch.int32, device=DEVICE)
+    alone["query_lens"] = [1, 1]
     separate = run_attention(ops, alone, 0.2)
     assert torch.equal(separate[0], together[199]) and torch.equal(separate[1], together[200])
 

@@ -56,13 +56,15 @@ def step_context(query_lens, starts, block_size, *, tables=None):
     prefix = 0
     while prefix < len(query_lens) and query_lens[prefix] == 1:
         prefix += 1
-    tile_seq, tile_token, tile_length = [], [], []
+    tile_seq, tile_token, tile_length, tile_first = [], [], [], []
     for index in range(prefix, len(query_lens)):
         for start in range(0, query_lens[index], 64):
             tile_seq.append(index)
             tile_token.append(starts_q[index] + start)
             tile_length.append(min(64, query_lens[index] - start))
-    tile_tables = {"attention.tile_seq": i32(tile_seq), "attention.tile_token": i32(tile_token), "attention.tile_length": i32(tile_length)}
+            tile_first.append(starts[index] + start)
+    tile_tables = {"attention.tile_seq": i32(tile_seq), "attention.tile_token": i32(tile_token),
+                   "attention.tile_length": i32(tile_length), "attention.tile_first": i32(tile_first)}
     return StepContext(
         num_tokens=len(token_pos), num_seqs=len(query_lens), token_ids=i32([0] * len(token_pos)), positions=i32(token_pos),
         seq_of_token=i32(seq_of), query_start=i32(starts_q), context_lens=i32([s + q for s, q in zip(starts, query_lens)]),
