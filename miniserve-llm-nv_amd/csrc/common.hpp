@@ -20,12 +20,10 @@ __device__ __forceinline__ float bf16_bits_to_float(uint16_t bits) {
   return __uint_as_float(static_cast<uint32_t>(bits) << 16);
 }
 
-// Round to nearest even; NaN stays NaN.
+// Round to nearest even; NaN stays NaN.  The conversion is one instruction of gfx950
+// (two values at a time where the compiler finds two).
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float value) {
-  uint32_t u = __float_as_uint(value);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(value));
 }
 
 __device__ __forceinline__ float to_float(float v) { return v; }

@@ -156,14 +156,17 @@ constexpr int kTiledThreads = 256;
 constexpr int kTiledMaxElements = kTiledThreads * 16;   // elements of one head of a tile
 constexpr int kTiledHeads = 4;                          // query and key heads that one workgroup rotates
 
-__device__ __forceinline__ void load8(const ms::bf16* src, float out[8]) {
-  const uint4 raw = *reinterpret_cast<const uint4*>(src);
+__device__ __forceinline__ void unpack8(const uint4& raw, float out[8]) {
   const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     out[2 * i] = ms::bf16_bits_to_float(static_cast<uint16_t>(words[i]));
     out[2 * i + 1] = ms::bf16_bits_to_float(static_cast<uint16_t>(words[i] >> 16));
   }
+}
+
+__device__ __forceinline__ void load8(const ms::bf16* src, float out[8]) {
+  unpack8(*reinterpret_cast<const uint4*>(src), out);
 }
 
 __device__ __forceinline__ void load8(const float* src, float out[8]) {
@@ -192,6 +195,7 @@ __global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kerne
   constexpr int kGroup = 16 / static_cast<int>(sizeof(T));   // values of one 16-byte store
   __shared__ float square_s[kTiledHeads][kTiledThreads];
   __shared__ int32_t slot_s[kTiledThreads];
+  __shared__ bool whole_s[kTiledThreads];
   __shared__ __align__(16) T tile_s[kTiledMaxElements];
 
   // blockIdx.y: first the groups of kTiledHeads query and key heads (one workgroup reads
@@ -213,40 +217,46 @@ __global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kerne
     // values: through LDS, written along the page's offset axis
     const int kv_head = static_cast<int>(blockIdx.y) - rotated_groups;
     const T* row = packed + (token * packed_heads + rotated_heads + kv_head) * head_dim;
-    if (live) {
-      float lo[8], hi[8];
-      load8(row + 8 * part, lo);
-      load8(row + half + 8 * part, hi);
-      store8(tile_s + item * head_dim + 8 * part, lo);
-      store8(tile_s + item * head_dim + half + 8 * part, hi);
+    if (live) {      // 16 bytes as they are
+      const uint4 lo = *reinterpret_cast<const uint4*>(row + 8 * part);
+      const uint4 hi = *reinterpret_cast<const uint4*>(row + half + 8 * part);
+      *reinterpret_cast<uint4*>(tile_s + item * head_dim + 8 * part) = lo;
+      *reinterpret_cast<uint4*>(tile_s + item * head_dim + half + 8 * part) = hi;
     }
     if (threadIdx.x < live_tokens) slot_s[threadIdx.x] = slot_mapping[first_token + threadIdx.x];
     __syncthreads();
-    const bool vector_ok = block_size % kGroup == 0;
-    for (int task = threadIdx.x; task < live_tokens * head_dim; task += kTiledThreads) {
-      const int j = task / head_dim;
-      const int d = task - j * head_dim;
-      const int32_t slot = slot_s[j];
-      // a run starts where the slots stop being consecutive or a 16-byte group begins
-      if (j > 0 && slot == slot_s[j - 1] + 1 && slot % kGroup != 0) continue;
-      int run = 1;
-      while (run < kGroup && j + run < live_tokens && slot_s[j + run] == slot + run && (slot + run) % kGroup != 0)
-        ++run;
-      const int64_t page = slot / block_size;
-      const int offset = slot - static_cast<int32_t>(page) * block_size;
-      T* dst = value_pool + ((page * num_kv_heads + kv_head) * head_dim + d) * block_size + offset;
-      if (vector_ok && run == kGroup && offset % kGroup == 0) {
+    // A group of kGroup consecutive tokens whose slots are consecutive and begin a
+    // 16-byte group of a page's row is written with one store for every d (a prompt's
+    // tokens are, but for the first and the last group of a portion); the tokens of any
+    // other group go one by one.
+    const int groups = (live_tokens + kGroup - 1) / kGroup;
+    if (threadIdx.x < groups) {
+      const int j0 = threadIdx.x * kGroup;
+      bool whole = block_size % kGroup == 0 && j0 + kGroup <= live_tokens && slot_s[j0] % kGroup == 0;
+      for (int i = 1; whole && i < kGroup; ++i) whole = slot_s[j0 + i] == slot_s[j0] + i;
+      whole_s[threadIdx.x] = whole;
+    }
+    __syncthreads();
+    for (int task = threadIdx.x; task < groups * head_dim; task += kTiledThreads) {
+      const int group = task / head_dim;
+      const int d = task - group * head_dim;
+      const int j0 = group * kGroup;
+      if (whole_s[group]) {
+        const int32_t slot = slot_s[j0];
+        const int page = slot / block_size;
+        const int offset = slot - page * block_size;
         __align__(16) T gathered[kGroup];
 #pragma unroll
-        for (int i = 0; i < kGroup; ++i) gathered[i] = tile_s[(j + i) * head_dim + d];
+        for (int i = 0; i < kGroup; ++i) gathered[i] = tile_s[(j0 + i) * head_dim + d];
+        T* dst = value_pool + ((static_cast<int64_t>(page) * num_kv_heads + kv_head) * head_dim + d) * block_size + offset;
         *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(gathered);
       } else {
-        // the run stays inside one page only if the offsets do
-        for (int i = 0; i < run; ++i) {
-          const int32_t s = slot + i;
-          const int64_t pg = s / block_size;
-          const int off = s - static_cast<int32_t>(pg) * block_size;
-          value_pool[((pg * num_kv_heads + kv_head) * head_dim + d) * block_size + off] = tile_s[(j + i) * head_dim + d];
+        for (int i = 0; i < kGroup && j0 + i < live_tokens; ++i) {
+          const int32_t slot = slot_s[j0 + i];
+          const int page = slot / block_size;
+          const int offset = slot - page * block_size;
+          value_pool[((static_cast<int64_t>(page) * num_kv_heads + kv_head) * head_dim + d) * block_size + offset] =
+              tile_s[(j0 + i) * head_dim + d];
         }
       }
     }
@@ -257,22 +267,45 @@ __global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kerne
   // out together, with the tile's cos and sin
   const int first_head = static_cast<int>(blockIdx.y) * kTiledHeads;
   const int heads_here = min(kTiledHeads, rotated_heads - first_head);
-  float lo[kTiledHeads][8], hi[kTiledHeads][8];
+  // No branch that differs between lanes stands around a load (a dead lane reads the
+  // tile's first token, a missing head the last one, and stores nothing): a value that is
+  // used behind such a branch is waited for behind it, head after head, and the kernel
+  // would take as many trips to memory as it has heads.  The values are turned into
+  // floats when all loads are on their way.
+  static_assert(sizeof(T) == 2, "16 bytes are 8 elements");
+  uint4 raw_lo[kTiledHeads], raw_hi[kTiledHeads];
 #pragma unroll
   for (int i = 0; i < kTiledHeads; ++i) {
-    if (live && i < heads_here) {
-      const T* row = packed + (token * packed_heads + first_head + i) * head_dim;
-      load8(row + 8 * part, lo[i]);
-      load8(row + half + 8 * part, hi[i]);
-    }
+    const T* row = packed + (token * packed_heads + first_head + min(i, heads_here - 1)) * head_dim;
+    raw_lo[i] = *reinterpret_cast<const uint4*>(row + 8 * part);
+    raw_hi[i] = *reinterpret_cast<const uint4*>(row + half + 8 * part);
   }
   float cs[8], sn[8];
-  if (live && cos_table != nullptr) {
+  if (cos_table != nullptr) {
     load8(cos_table + token * half + 8 * part, cs);
     load8(sin_table + token * half + 8 * part, sn);
   }
-  int64_t slot = 0;
-  if (live && first_head + heads_here > num_q_heads) slot = slot_mapping[token];
+  int slot = 0;      // a slot number is below 2^31
+  if (first_head + heads_here > num_q_heads) slot = slot_mapping[token];
+  // the norms' weights go out with the rows: asked for where they are used, behind the
+  // barrier, each head would wait for memory once more
+  uint4 raw_wq[2], raw_wk[2];
+  const bool has_q = q_weight != nullptr && first_head < num_q_heads;
+  const bool has_k = k_weight != nullptr && first_head + heads_here > num_q_heads;
+  if (has_q) {
+    raw_wq[0] = *reinterpret_cast<const uint4*>(q_weight + 8 * part);
+    raw_wq[1] = *reinterpret_cast<const uint4*>(q_weight + half + 8 * part);
+  }
+  if (has_k) {
+    raw_wk[0] = *reinterpret_cast<const uint4*>(k_weight + 8 * part);
+    raw_wk[1] = *reinterpret_cast<const uint4*>(k_weight + half + 8 * part);
+  }
+  float lo[kTiledHeads][8], hi[kTiledHeads][8];
+#pragma unroll
+  for (int i = 0; i < kTiledHeads; ++i) {
+    unpack8(raw_lo[i], lo[i]);
+    unpack8(raw_hi[i], hi[i]);
+  }
 
   if (q_weight != nullptr || k_weight != nullptr) {
 #pragma unroll
@@ -302,8 +335,8 @@ __global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kerne
       for (int p = 0; p < lanes_per_row; ++p) total += square_s[i][item * lanes_per_row + p];
       const float inv = 1.0f / sqrtf(total / static_cast<float>(head_dim) + eps);
       float w_lo[8], w_hi[8];
-      load8(weight + 8 * part, w_lo);
-      load8(weight + half + 8 * part, w_hi);
+      unpack8(is_q ? raw_wq[0] : raw_wk[0], w_lo);
+      unpack8(is_q ? raw_wq[1] : raw_wk[1], w_hi);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         lo[i][e] = ms::round_to<T>(w_lo[e] * ms::round_to<T>(lo[i][e] * inv));
@@ -323,9 +356,9 @@ __global__ __launch_bounds__(kTiledThreads) void qk_norm_rope_append_tiled_kerne
       dst = q_out + (token * num_q_heads + head) * head_dim;
     } else {
       const int kv_head = head - num_q_heads;
-      const int64_t page = slot / block_size;
-      const int64_t offset = slot - page * block_size;
-      dst = key_pool + ((page * num_kv_heads + kv_head) * block_size + offset) * head_dim;
+      const int page = slot / block_size;
+      const int offset = slot - page * block_size;
+      dst = key_pool + ((static_cast<int64_t>(page) * num_kv_heads + kv_head) * block_size + offset) * head_dim;
     }
     store8(dst + 8 * part, lo[i]);
     store8(dst + half + 8 * part, hi[i]);
@@ -401,12 +434,12 @@ extern "C" int ms_qk_norm_rope_append(const void* packed, const void* q_weight, 
   MS_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "qk_norm_rope_append: rotation needs both tables");
   MS_REQUIRE(num_q_heads + 2 * num_kv_heads <= 65535, "qk_norm_rope_append: too many heads");
   // bfloat16, 16 bytes a lane, where the head size is a multiple of 16 and every operand
-  // is aligned to 16 bytes (null operands are), for more tokens than two tiles; few
+  // is aligned to 16 bytes (null operands are), for more tokens than four tiles; few
   // tokens are quicker with a wave to each row.  32-bit storage always takes the wave
   // to each row: the order of its sums never depends on the number of tokens, so a
   // position's result is the same to the bit however the tokens are cut into steps.
   const bool tiled = dtype == MS_BF16 && head_dim % 16 == 0 && head_dim <= 16 * kTiledThreads &&
-                     num_tokens > 2 * (kTiledThreads / (head_dim / 16)) && aligned16(packed) &&
+                     num_tokens > 4 * (kTiledThreads / (head_dim / 16)) && aligned16(packed) &&
                      aligned16(q_weight) && aligned16(k_weight) && aligned16(cos_table) && aligned16(sin_table) &&
                      aligned16(q_out) && aligned16(key_pool) && aligned16(value_pool);
   if (tiled) {

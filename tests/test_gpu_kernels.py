@@ -180,7 +180,7 @@ def test_append_of_a_run_of_tokens_beside_single_ones(ops, dtype, heads, kv_head
 
     from miniserve_amd.parts.rotary import inverse_frequencies
 
-    run, theta, eps = max(150, 2 * 256 * 16 // dim + 40), 1e4, 1e-6     # enough for the many-token kernel
+    run, theta, eps = max(150, 4 * 256 * 16 // dim + 40), 1e4, 1e-6     # enough for the many-token kernel
     run_pages = (start + run + block - 1) // block
     pages = run_pages + 3
     table = list(range(run_pages - 1, -1, -1))                                  # logical -> physical page
