@@ -171,20 +171,30 @@ __global__ __launch_bounds__(kThreads) MS_WAVES_PER_EU(D <= 128 ? 2 : 1, 2) void
   if (!kPrefetch) {
     for (; t < t1; t += kStep) {
       TilePair<D> pair;
-      load_pair<D>(pair, t, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+      load_pair<D>(pair, ms::find_pair(t, t1, table, block_size), key_pool, value_pool, num_kv_heads, kv_head,
+                   block_size, g, r);
       consume_pair<D>(st, pair, q_reg, t, lo, pos, scale, g);
     }
   } else if (t < t1) {
+    // the pages of a pair are looked up while the pair before it is on its way
     TilePair<D> ping, pong;
-    load_pair<D>(ping, t, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+    load_pair<D>(ping, ms::find_pair(t, t1, table, block_size), key_pool, value_pool, num_kv_heads, kv_head, block_size,
+                 g, r);
+    ms::PairPlace ahead = ms::find_pair(t + kStep, t1, table, block_size);
     while (true) {
       int next = t + kStep;
-      if (next < t1) load_pair<D>(pong, next, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+      if (next < t1) {
+        load_pair<D>(pong, ahead, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+        ahead = ms::find_pair(next + kStep, t1, table, block_size);
+      }
       consume_pair<D>(st, ping, q_reg, t, lo, pos, scale, g);
       t = next;
       if (t >= t1) break;
       next = t + kStep;
-      if (next < t1) load_pair<D>(ping, next, t1, table, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+      if (next < t1) {
+        load_pair<D>(ping, ahead, key_pool, value_pool, num_kv_heads, kv_head, block_size, g, r);
+        ahead = ms::find_pair(next + kStep, t1, table, block_size);
+      }
       consume_pair<D>(st, pong, q_reg, t, lo, pos, scale, g);
       t = next;
       if (t >= t1) break;

@@ -19,22 +19,49 @@ struct TilePair {
   bool has_b;
 };
 
-template <int D>
-__device__ __forceinline__ void load_pair(TilePair<D>& pair, int tile, int end_tile, const int32_t* __restrict__ table,
-                                          const bf16* __restrict__ key_pool, const bf16* __restrict__ value_pool,
-                                          int num_kv_heads, int kv_head, int block_size, int g, int r) {
-  const bool has_b = tile + 1 < end_tile;
-  pair.has_b = has_b;
+// Where the two tiles of a pair lie: the page of each and the offset of its first key
+// in the page (the same in all lanes of a wave).  Looked up one step before the pair's
+// loads go out, so that those do not wait for the block table.
+struct PairPlace {
+  int32_t page_a, page_b;
+  int off_a, off_b;
+  bool has_b;
+};
+
+__device__ __forceinline__ PairPlace find_pair(int tile, int end_tile, const int32_t* __restrict__ table,
+                                               int block_size) {
+  // a pair past the end is never loaded; it is looked up as the last tile so that the
+  // table is not read beyond its row
+  tile = min(tile, end_tile - 1);
+  PairPlace place;
+  place.has_b = tile + 1 < end_tile;
   const int key_a = tile * kTileKeys;
-  const int key_b = key_a + kTileKeys;
-  const int64_t page_a = table[key_a / block_size];
-  const int off_a = key_a % block_size;
-  const int64_t page_b = has_b ? table[key_b / block_size] : page_a;
-  const int off_b = has_b ? key_b % block_size : off_a;
-  const bf16* k_row_a = key_pool + ((page_a * num_kv_heads + kv_head) * block_size + off_a + r) * D;
-  const bf16* k_row_b = key_pool + ((page_b * num_kv_heads + kv_head) * block_size + off_b + r) * D;
-  const bf16* v_a = value_pool + (page_a * num_kv_heads + kv_head) * D * block_size + off_a + 4 * g;
-  const bf16* v_b = value_pool + (page_b * num_kv_heads + kv_head) * D * block_size + off_b + 4 * g;
+  const int key_b = place.has_b ? key_a + kTileKeys : key_a;
+  if (block_size == kTileKeys) {      // a page is a tile: no division
+    place.page_a = table[tile];
+    place.page_b = table[place.has_b ? tile + 1 : tile];
+    place.off_a = place.off_b = 0;
+  } else {
+    place.page_a = table[key_a / block_size];
+    place.off_a = key_a % block_size;
+    place.page_b = table[key_b / block_size];
+    place.off_b = key_b % block_size;
+  }
+  return place;
+}
+
+template <int D>
+__device__ __forceinline__ void load_pair(TilePair<D>& pair, const PairPlace& place, const bf16* __restrict__ key_pool,
+                                          const bf16* __restrict__ value_pool, int num_kv_heads, int kv_head,
+                                          int block_size, int g, int r) {
+  const bool has_b = place.has_b;
+  pair.has_b = has_b;
+  const int64_t slab_a = static_cast<int64_t>(place.page_a) * num_kv_heads + kv_head;
+  const int64_t slab_b = static_cast<int64_t>(place.page_b) * num_kv_heads + kv_head;
+  const bf16* k_row_a = key_pool + (slab_a * block_size + place.off_a + r) * D;
+  const bf16* k_row_b = key_pool + (slab_b * block_size + place.off_b + r) * D;
+  const bf16* v_a = value_pool + slab_a * D * block_size + place.off_a + 4 * g;
+  const bf16* v_b = value_pool + slab_b * D * block_size + place.off_b + 4 * g;
 #pragma unroll
   for (int s = 0; s < TilePair<D>::KS; ++s) {
     const int d0 = 32 * s + 8 * g;
