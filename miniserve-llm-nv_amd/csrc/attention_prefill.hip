@@ -519,13 +519,13 @@ extern "C" int ms_attention_prefill_supported(int head_dim, int block_size) {
 // sequence, at consecutive positions: tile_seq (row of block_table), tile_token (index
 // of its first token), tile_count (1..64), tile_first (position of its first token),
 // all int32 [num_tiles].
-// tiles_sorted: the tiles come in the order of the keys they walk, fewest first (then
-// a workgroup may take a long and a short one; in any other order every workgroup
+// tile_order: not 0 if the tiles come in the order of the keys they walk, fewest first
+// (then a workgroup may take a long and a short one; in any other order every workgroup
 // takes one tile).
 extern "C" int ms_attention_prefill(const void* q, const void* key_pool, const void* value_pool,
                                     const void* block_table, const void* tile_seq, const void* tile_token,
                                     const void* tile_count, const void* tile_first, void* out, int num_tiles,
-                                    int tiles_sorted, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+                                    int tile_order, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
                                     int max_blocks, float scale, int window, hipStream_t stream) {
   MS_REQUIRE(num_tiles > 0, "attention_prefill: no tiles");
   MS_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0,
@@ -539,20 +539,24 @@ extern "C" int ms_attention_prefill(const void* q, const void* key_pool, const v
              "attention_prefill: a page of %d kv heads x %d keys x %d is too large", num_kv_heads, block_size, head_dim);
   const int group = num_q_heads / num_kv_heads;
   // Two query heads of a kv head to a workgroup (every key and value loaded serves both,
-  // the keys dealt out to two parts) where that gives the chip workgroups enough to be
-  // handed out in pairs; a smaller launch, and one whose kv heads have one query head
-  // each, takes one head a workgroup and deals the keys out to four parts: twice the
-  // workgroups, and half the steps for the longest tile (1,024 tokens of 16 heads:
-  // 25.6 -> 21.0 us; 2,048: 42.3 -> 40.8 us).
+  // the keys dealt out to two parts) is the rule.  One head a workgroup, the keys dealt
+  // out to four parts, gives twice the workgroups and half the steps for the longest
+  // tile, at the price of loading every key and value for 64 columns instead of 128.  It
+  // is taken for kv heads with one query head and for launches that would leave a quarter
+  // of the chip without a workgroup (1,024 tokens of 16 heads: 25.6 -> 19.0 us).  (For
+  // 256 workgroups of two heads it was measured both ways: one prompt of 2,048 tokens
+  // gains by it when its tiles go out in pairs, 42 -> 37 us, steps of four portions of
+  // 512 tokens with histories lose, 37 -> 46 us: left as the rule has it.)
+  const bool sorted = tile_order != 0;
   const int64_t with_two = static_cast<int64_t>(num_tiles) * num_kv_heads * ((group + 1) / 2);
-  const int hb = (group >= 2 && with_two >= kPairedFrom) ? 2 : 1;
+  const int hb = (group >= 2 && with_two >= kComputeUnits - kComputeUnits / 4) ? 2 : 1;
   const int64_t workgroups = static_cast<int64_t>(num_tiles) * num_kv_heads * ((group + hb - 1) / hb);
   // A long and a short tile to a workgroup where the pairs still fill the chip (256
   // compute units hold one workgroup each): then every workgroup walks about the same
   // number of keys (8,192 tokens of 16 heads: 396 -> 294 us).  A small launch keeps a tile
   // a workgroup: the longest tile sets its time either way, and a second tile costs a
   // workgroup a second start.
-  const int paired = tiles_sorted && workgroups >= kPairedFrom;
+  const int paired = sorted && workgroups >= kPairedFrom;
   MS_REQUIRE(num_kv_heads * ((group + hb - 1) / hb) <= 65535, "attention_prefill: too many heads");
 #define MS_PREFILL_CASE(DIM)                                                                                       \
   case DIM:                                                                                                        \
