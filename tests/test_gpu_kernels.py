@@ -480,6 +480,61 @@ def test_decode_kernel_ignores_stale_values(ops):
     torch.testing.assert_close(out.cpu().double(), attention_reference(case, 0.125), atol=ATTENTION_BF16, rtol=ATTENTION_BF16)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_pages_whose_offsets_pass_32_bits(ops, dtype):
+    """A pool sized for the card's memory has pages that lie more than 2^31 elements into
+    it.  The same keys and values at such pages give the results they give at pages 0, 1,
+    2, ... to the bit, from the single-token kernel, the tiled kernel, the generic one (32-bit)
+    and the kernel that writes the cache: an offset computed in 32 bits would read or write
+    elsewhere.  (The pools are not initialised; 9 and 17 GB of the card's 288.)"""
+
+    from miniserve_amd.parts.rotary import inverse_frequencies
+
+    heads, kv_heads, dim, block = 16, 8, 128, 16
+    scale = dim**-0.5
+    case = paged_case([300, 77, 150], heads, kv_heads, dim, block, dtype, query_lens=[1, 1, 40], seed=5)
+    low = run_attention(ops, case, scale)
+    small_pages = case["key_pool"].shape[0]
+    pages = (1 << 31) // (kv_heads * block * dim) + 600
+    key_pool = torch.empty(pages, kv_heads, block, dim, dtype=dtype, device=DEVICE)
+    value_pool = torch.empty(pages, kv_heads, dim, block, dtype=dtype, device=DEVICE)
+    moved = torch.arange(pages - 1, pages - 1 - small_pages, -1, device=DEVICE)          # page i lies at pages - 1 - i
+    assert int(moved.min()) * kv_heads * block * dim > 1 << 31
+    key_pool[moved] = case["key_pool"]
+    value_pool[moved] = case["value_pool"]
+    high_case = dict(case, key_pool=key_pool, value_pool=value_pool,
+                     block_table=(pages - 1 - case["block_table"]).to(torch.int32))
+    high = run_attention(ops, high_case, scale)
+    assert torch.equal(low, high)
+
+    # the write: the same tokens to slots of low pages and to the same places of high ones
+    n, region = 150, 12                      # enough tokens for the tiled form; the pages they and two more are written to
+    packed = rand(n, (heads + 2 * kv_heads) * dim, seed=3, dtype=dtype)
+    weight = (1 + 0.1 * rand(dim, seed=1)).to(dtype)
+    positions = torch.arange(5, 5 + n, dtype=torch.int32, device=DEVICE)
+    rope = ops.rope_table(positions, inverse_frequencies(dim, 1e6).to(DEVICE))
+    slots = torch.arange(3, 3 + n, dtype=torch.int32, device=DEVICE)
+    pools = {}
+    for name, shift in (("low", 0), ("high", (pages - region) * block)):
+        if shift == 0:
+            keys = torch.zeros(region, kv_heads, block, dim, dtype=dtype, device=DEVICE)
+            values = torch.zeros(region, kv_heads, dim, block, dtype=dtype, device=DEVICE)
+        else:
+            keys, values = key_pool, value_pool
+            keys[pages - region :] = 0
+            values[pages - region :] = 0
+        for count in (n, 2):                         # many tokens: the tiled form; two: a token a workgroup
+            ops.qk_norm_rope_append(packed[:count], num_q_heads=heads, num_kv_heads=kv_heads, head_dim=dim, q_weight=weight,
+                                    k_weight=weight, eps=1e-6, rope=(rope[0][:count].contiguous(), rope[1][:count].contiguous()),
+                                    slot_mapping=(slots[:count] + shift + (0 if count == n else n)).contiguous(),
+                                    key_pool=keys, value_pool=values)
+        pools[name] = (keys[-region:].clone(), values[-region:].clone())
+    assert torch.equal(pools["low"][0], pools["high"][0]) and torch.equal(pools["low"][1], pools["high"][1])
+    assert bool(pools["low"][0].any()) and bool(pools["low"][1].any())
+    del key_pool, value_pool, high_case, keys, values
+    torch.cuda.empty_cache()
+
+
 def test_decode_kernel_is_refused_for_other_geometries(ops):
     lib = ops.load()
     assert not lib.ms_attention_decode_supported(128, 8)          # pages of 8 keys
