@@ -1,9 +1,9 @@
 """(c)'s generality: a toy mixer with state of its own, a toy feed-forward with
-routing, a toy position encoding and a toy architecture that uses them beside
-attention layers - one of them with a window, one named twice, one reading another
-call's cache - are defined HERE, registered, built from a model folder with random
-weights and stepped, without a change to the framework's files.  They are no model
-of anyone's."""
+routing, a toy position encoding, a toy norm, a toy arrangement of a layer's parts and
+a toy architecture that uses them beside attention layers - one of them with a window,
+one named twice, one reading another call's cache - are defined HERE, registered, built
+from a model folder with random weights and stepped, without a change to the
+framework's files.  They are no model of anyone's."""
 
 from __future__ import annotations
 
@@ -22,15 +22,16 @@ pytestmark = pytest.mark.gpu
 WINDOW = 6
 WINDOW_PAGE = 32        # the window layers keep pages of their own size (the engine's are 16 or 4 below)
 EXPERTS, EXPERT_WIDTH = 3, 40
-KINDS = ("attention", "running_mean", "window_attention")      # the mixers; layer 1 also has the routed feed-forward,
-                                                                # layer 2 the rotation of neighbouring pairs
-ORDER = ((0, None), (1, None), (2, None), (0, 0), (2, None), (1, None))    # (layer, cache_from)
+# the mixers; layer 1 also has the routed feed-forward, layer 2 the rotation of neighbouring pairs, layer 3 its
+# norms after the sums (the first of them a norm that subtracts the mean)
+KINDS = ("attention", "running_mean", "window_attention", "post_norm_attention")
+ORDER = ((0, None), (1, None), (2, None), (0, 0), (3, None), (2, None), (1, None))    # (layer, cache_from)
 
 
 def define_toy():
     from miniserve_amd import ops
     from miniserve_amd.config import LayerCall, LayerSpec, ModelSpec, PartSpec, Qwen3Config, register_architecture
-    from miniserve_amd.parts import Part, StateNeed, StateView, WeightSpec, register_part
+    from miniserve_amd.parts import Part, StateNeed, StateView, WeightSpec, build_part, register_part
 
     class RunningMean(Part):
         """out_t = W * mean(x_0 .. x_t).  Its state per request: the running sum and
@@ -114,6 +115,53 @@ def define_toy():
             even, odd = x[..., 0::2].float(), x[..., 1::2].float()
             return torch.stack([even * cos - odd * sin, odd * cos + even * sin], dim=-1).reshape(x.shape).to(x.dtype)
 
+    class CenterNorm(Part):
+        """Another norm: ``y = w * (x - mean(x)) * rsqrt(var(x) + eps)``, statistics in 32-bit."""
+
+        def __init__(self, spec, dtype):
+            self.dim, self.eps, self.dtype = spec.params["dim"], spec.params["eps"], dtype
+            self.name = spec.prefix + "weight"
+
+        def weight_specs(self):
+            return [WeightSpec(self.name, (self.dim,), init="norm")]
+
+        def load_weights(self, tensors):
+            self.weight = tensors[self.name]
+
+        def forward(self, x):
+            centred = x.float() - x.float().mean(dim=-1, keepdim=True)
+            scaled = centred * torch.rsqrt(centred.pow(2).mean(dim=-1, keepdim=True) + self.eps)
+            return (scaled * self.weight.float()).to(self.dtype)
+
+        def add_forward(self, residual, delta, *, rows=None, write_back=True):
+            total = residual if delta is None else residual + delta.float()
+            if delta is not None and write_back and rows is None:
+                residual.copy_(total)
+            return self.forward(total if rows is None else total[rows.long()])
+
+    class PostNormBlock(Part):
+        """Another arrangement: ``h <- norm(h + mixer(h)); h <- norm(h + feed_forward(h))``.
+        The stream it hands on is the second norm's output; nothing is left to be added."""
+
+        def __init__(self, layer, dtype):
+            self.mixer = build_part("mixer", layer.mixer, dtype)
+            self.post_mixer = build_part("norm", layer.norms["post_mixer"], dtype)
+            self.feed_forward = build_part("feed_forward", layer.feed_forward, dtype)
+            self.post_feed_forward = build_part("norm", layer.norms["post_feed_forward"], dtype)
+            self.dtype = dtype
+
+        def sub_parts(self):
+            return [self.mixer, self.post_mixer, self.feed_forward, self.post_feed_forward]
+
+        def forward(self, residual, delta, ctx, cache):
+            if delta is not None:
+                ops.residual_add(residual, delta)
+            mixed = self.mixer.forward(residual.to(self.dtype), ctx, cache)
+            stream = self.post_mixer.add_forward(residual, mixed)
+            out = self.feed_forward.forward(stream, ctx)
+            stream = self.post_feed_forward.add_forward(stream.float(), out)
+            return stream.float(), None
+
     @dataclass(frozen=True)
     class ToyConfig:
         base: Qwen3Config
@@ -149,7 +197,13 @@ def define_toy():
                 if kind == "running_mean":
                     feed_forward = PartSpec("test_routed_experts", {"hidden_size": spec.hidden_size, "width": EXPERT_WIDTH,
                                                                     "experts": EXPERTS}, f"model.layers.{index}.moe.")
-                layers.append(LayerSpec(layer.block, mixer, feed_forward, layer.norms))
+                block, norms = layer.block, layer.norms
+                if kind == "post_norm_attention":
+                    first = layer.norms["pre_mixer"]
+                    block = "test_post_norm"
+                    norms = {"post_mixer": PartSpec("test_center_norm", dict(first.params), first.prefix),
+                             "post_feed_forward": layer.norms["pre_feed_forward"]}
+                layers.append(LayerSpec(block, mixer, feed_forward, norms))
             return ModelSpec(
                 architecture=self.architecture, hidden_size=spec.hidden_size, vocab_size=spec.vocab_size,
                 max_positions=spec.max_positions, embedding=spec.embedding, layers=tuple(layers),
@@ -159,6 +213,8 @@ def define_toy():
     register_part("mixer", "test_running_mean", RunningMean)
     register_part("feed_forward", "test_routed_experts", RoutedExperts)
     register_part("position", "test_rotary_pairs", RotaryPairs)
+    register_part("norm", "test_center_norm", CenterNorm)
+    register_part("block", "test_post_norm", PostNormBlock)
     register_architecture(ToyConfig.architecture, ToyConfig)
     return ToyConfig
 
@@ -205,6 +261,12 @@ def toy_logits(weights, config, tokens):
     kept = {}
     for call, (layer, source) in enumerate(ORDER):
         base = f"model.layers.{layer}."
+        if KINDS[layer] == "post_norm_attention":
+            mixed, kept[call] = plain.attention_block(h, w, base + "self_attn.", config, positions, None, None)
+            centred = (h + mixed) - (h + mixed).mean(dim=-1, keepdim=True)
+            h = w[base + "input_layernorm.weight"] * centred * torch.rsqrt(centred.pow(2).mean(dim=-1, keepdim=True) + eps)
+            h = plain.rms_norm(h + plain.swiglu(h, w, base + "mlp."), w[base + "post_attention_layernorm.weight"], eps)
+            continue
         x = plain.rms_norm(h, w[base + "input_layernorm.weight"], eps)
         if KINDS[layer] == "running_mean":
             mean = torch.cumsum(x, dim=0) / torch.arange(1, length + 1, dtype=torch.float64)[:, None]
@@ -229,7 +291,7 @@ def toy(tmp_path_factory):
 
     toy_config = define_toy()
     data = tiny_a()
-    data["num_hidden_layers"] = 3
+    data["num_hidden_layers"] = len(KINDS)
     data["architectures"] = [toy_config.architecture]
     folder = write_random_model(toy_config.from_dict(data), tmp_path_factory.mktemp("toy") / "model", seed=8)
     assert type(load_config(folder)).__name__ == "ToyConfig"            # chosen by config.json through the registry
@@ -237,6 +299,8 @@ def toy(tmp_path_factory):
     unregister_part("mixer", "test_running_mean")
     unregister_part("feed_forward", "test_routed_experts")
     unregister_part("position", "test_rotary_pairs")
+    unregister_part("norm", "test_center_norm")
+    unregister_part("block", "test_post_norm")
 
 
 def test_the_toy_model_is_built_from_its_folder(toy):
@@ -250,11 +314,13 @@ def test_the_toy_model_is_built_from_its_folder(toy):
     assert float(weights["model.layers.1.moe.router.weight"].std()) > 0.5         # drawn by the part's own rule
     model = DecoderModel(load_config(toy).model_spec(), "float32")
     layout = CacheLayout.from_needs(model.cache_needs())
-    # full attention: one cache (call 0, read again by call 3); window: two caches (calls 2, 4); two states (calls 1, 5)
-    assert [(g.need.window, g.need.block_size, g.calls) for g in layout.groups] == [(None, None, [0]), (WINDOW, WINDOW_PAGE, [2, 4])]
+    # full attention: two caches (call 0, read again by call 3, and call 4); window: two caches (calls 2, 5); two
+    # states (calls 1, 6)
+    assert [(g.need.window, g.need.block_size, g.calls) for g in layout.groups] == [(None, None, [0, 4]), (WINDOW, WINDOW_PAGE, [2, 5])]
     assert len(layout.states) == 2
-    assert [p.kind for p in layout.placements] == ["kv", "state", "kv", "kv", "kv", "state"]
+    assert [p.kind for p in layout.placements] == ["kv", "state", "kv", "kv", "kv", "kv", "state"]
     assert layout.placements[3].write is False and layout.placements[3].index == 0
+    assert type(model.layers[3]).__name__ == "PostNormBlock" and type(model.layers[3].post_mixer).__name__ == "CenterNorm"
 
 
 @pytest.mark.parametrize("shape", ["whole", "portions", "mixed"])
