@@ -65,6 +65,7 @@ struct Keep {
 // What the choice is made from: the whole row, or the few tokens of it that can
 // still matter, gathered in LDS in token order.  value(i) is logit / temperature.
 struct RowView {
+  static constexpr bool kInDeviceMemory = true;
   const float* x;
   float temp;
   int size;
@@ -72,13 +73,17 @@ struct RowView {
   __device__ __forceinline__ int index(int i) const { return i; }
 };
 
-struct ListView {
+template <bool InDeviceMemory>
+struct ListViewAt {
+  static constexpr bool kInDeviceMemory = InDeviceMemory;
   const float* values;
   const int* indices;
   int size;
   __device__ __forceinline__ float value(int i) const { return values[i]; }
   __device__ __forceinline__ int index(int i) const { return indices[i]; }
 };
+using ListView = ListViewAt<false>;          // gathered in LDS
+using LongListView = ListViewAt<true>;       // too long for that: where the gathering kernel left it
 
 constexpr int kListCap = 4096;      // tokens that the short list holds at most
 // Distances below the row's maximum (in units of logit / temperature) at which the
@@ -161,6 +166,55 @@ __device__ int choose_among_few(const View& view, int limit_index, float scaled_
   return chosen;
 }
 
+// f(value, index) for the elements tid, tid + kThreads, ... of the view, in that order.
+// Of a view in device memory eight at a time with their loads issued together: a loop that
+// loads an element and then decides on it waits for memory once per element.
+constexpr int kLoadsAhead = 8;
+
+template <typename View, typename F>
+__device__ __forceinline__ void for_each_strided(const View& view, int n, int tid, F&& f) {
+  if constexpr (!View::kInDeviceMemory) {
+    for (int i = tid; i < n; i += kThreads) f(view.value(i), view.index(i));
+    return;
+  }
+  for (int base = tid; base < n; base += kLoadsAhead * kThreads) {
+    float value[kLoadsAhead];
+    int index[kLoadsAhead];
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u) {
+      const int i = min(base + u * kThreads, n - 1);      // past the end: loaded again, not used
+      value[u] = view.value(i);
+      index[u] = view.index(i);
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u)
+      if (base + u * kThreads < n) f(value[u], index[u]);
+  }
+}
+
+// The same for the consecutive elements begin .. end - 1 of one thread; f returns false to stop.
+template <typename View, typename F>
+__device__ __forceinline__ void for_each_in_order(const View& view, int begin, int end, F&& f) {
+  if constexpr (!View::kInDeviceMemory) {
+    for (int i = begin; i < end; ++i)
+      if (!f(view.value(i), view.index(i))) return;
+    return;
+  }
+  for (int base = begin; base < end; base += kLoadsAhead) {
+    float value[kLoadsAhead];
+    int index[kLoadsAhead];
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u) {
+      const int i = min(base + u, end - 1);
+      value[u] = view.value(i);
+      index[u] = view.index(i);
+    }
+#pragma unroll
+    for (int u = 0; u < kLoadsAhead; ++u)
+      if (base + u < end && !f(value[u], index[u])) return;
+  }
+}
+
 // temperature -> top-k -> top-p -> draw over `view`; `limit_index`: an index beyond
 // every token's; `whole_mass`: the mass of all tokens where the view holds only some
 // of them and top-k is off (top_p is a share of that), else negative; `mass_before`:
@@ -194,11 +248,28 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
       int count[kDigits];
 #pragma unroll
       for (int c = 0; c < kDigits; ++c) count[c] = 0;
-      for (int i = tid; i < n; i += kThreads) {
-        const uint32_t o = ordered(view.value(i));
+      // A value whose bits above this digit differ from the threshold's lies above every
+      // candidate or below every one: it is counted once, not fifteen times (over a long
+      // view, where whole waves meet such values; among the few of a short list the branch
+      // costs more than it saves).
+      int above = 0;
+      for_each_strided(view, n, tid, [&](float v, int) {
+        const uint32_t o = ordered(v);
+        if constexpr (View::kInDeviceMemory) {
+          if (shift < 28 && ((o ^ threshold) >> (shift + 4)) != 0u) {
+            above += o > threshold;
+          } else {
+            const int digit = static_cast<int>((o >> shift) & 15u);
 #pragma unroll
-        for (int c = 0; c < kDigits; ++c) count[c] += o >= (threshold | (static_cast<uint32_t>(c + 1) << shift));
-      }
+            for (int c = 0; c < kDigits; ++c) count[c] += c < digit;
+          }
+        } else {
+#pragma unroll
+          for (int c = 0; c < kDigits; ++c) count[c] += o >= (threshold | (static_cast<uint32_t>(c + 1) << shift));
+        }
+      });
+#pragma unroll
+      for (int c = 0; c < kDigits; ++c) count[c] += above;
       __syncthreads();                    // the tables' last readers are done
 #pragma unroll
       for (int c = 0; c < kDigits; ++c) {
@@ -218,11 +289,12 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
       threshold |= static_cast<uint32_t>(digit) << shift;
     }
     int greater = 0, equal = 0;
-    for (int i = seg_begin; i < seg_end; ++i) {
-      const uint32_t o = ordered(view.value(i));
+    for_each_in_order(view, seg_begin, seg_end, [&](float v, int) {
+      const uint32_t o = ordered(v);
       greater += o > threshold;
       equal += o == threshold;
-    }
+      return true;
+    });
     const int total_greater = block_sum_int(greater, sc.i_scratch);
     const int wanted = k - total_greater;  // >= 1 equal values to keep, lowest indices first
     sc.seg_count[tid] = equal;
@@ -238,12 +310,14 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
     }
     __syncthreads();
     int seen = sc.seg_count[tid];
-    for (int i = seg_begin; i < seg_end; ++i) {
-      if (ordered(view.value(i)) == threshold) {
+    int* const tie_index = sc.shared_index;
+    for_each_in_order(view, seg_begin, seg_end, [&, tie_index](float v, int index) {
+      if (ordered(v) == threshold) {
         ++seen;
-        if (seen == wanted) *sc.shared_index = view.index(i);  // exactly one thread reaches `wanted`
+        if (seen == wanted) *tie_index = index;  // exactly one thread reaches `wanted`
       }
-    }
+      return true;
+    });
     __syncthreads();
     keep.k_threshold = threshold;
     keep.tie_limit = *sc.shared_index;
@@ -253,10 +327,9 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
   // ---- top-p ----------------------------------------------------------------
   if (p < 1.f) {
     float mass = 0.f;
-    for (int i = tid; i < n; i += kThreads) {
-      const float v = view.value(i);
-      if (keep(ordered(v), view.index(i))) mass += expf(v - scaled_max);
-    }
+    for_each_strided(view, n, tid, [&](float v, int index) {
+      if (keep(ordered(v), index)) mass += expf(v - scaled_max);
+    });
     const float kept_mass = ms::block_sum(mass, sc.f_scratch);
     const float limit = p * (whole_mass >= 0.f ? whole_mass : kept_mass);
     // Largest t with mass{ordered >= t} > limit; tokens at or above it stay.  Four bits a
@@ -266,16 +339,28 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
       float part[kDigits];
 #pragma unroll
       for (int c = 0; c < kDigits; ++c) part[c] = 0.f;
-      for (int i = tid; i < n; i += kThreads) {
-        const float v = view.value(i);
+      float above = 0.f;      // of values above every candidate (see top-k)
+      for_each_strided(view, n, tid, [&](float v, int index) {
         const uint32_t o = ordered(v);
-        if (o >= threshold && keep(o, view.index(i))) {
+        if (o >= threshold && keep(o, index)) {
           const float weight = expf(v - scaled_max);
+          if constexpr (View::kInDeviceMemory) {
+            if (shift < 28 && ((o ^ threshold) >> (shift + 4)) != 0u) {
+              above += weight;
+            } else {
+              const int digit = static_cast<int>((o >> shift) & 15u);
 #pragma unroll
-          for (int c = 0; c < kDigits; ++c)
-            part[c] += o >= (threshold | (static_cast<uint32_t>(c + 1) << shift)) ? weight : 0.f;
+              for (int c = 0; c < kDigits; ++c) part[c] += c < digit ? weight : 0.f;
+            }
+          } else {
+#pragma unroll
+            for (int c = 0; c < kDigits; ++c)
+              part[c] += o >= (threshold | (static_cast<uint32_t>(c + 1) << shift)) ? weight : 0.f;
+          }
         }
-      }
+      });
+#pragma unroll
+      for (int c = 0; c < kDigits; ++c) part[c] += above;
       __syncthreads();
 #pragma unroll
       for (int c = 0; c < kDigits; ++c) {
@@ -300,13 +385,13 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
   // ---- draw -----------------------------------------------------------------
   float mine = 0.f;
   int last_kept = -1;
-  for (int i = seg_begin; i < seg_end; ++i) {
-    const float v = view.value(i);
-    if (keep(ordered(v), view.index(i))) {
+  for_each_in_order(view, seg_begin, seg_end, [&](float v, int index) {
+    if (keep(ordered(v), index)) {
       mine += expf(v - scaled_max);
-      last_kept = view.index(i);
+      last_kept = index;
     }
-  }
+    return true;
+  });
   __syncthreads();
   sc.seg_sum[tid] = mine;
   sc.seg_count[tid] = last_kept;
@@ -328,16 +413,17 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
                                                                      : uniform * *sc.shared_total;
   __syncthreads();
   float running = sc.seg_sum[tid];
-  for (int i = seg_begin; i < seg_end; ++i) {
-    const float v = view.value(i);
-    if (keep(ordered(v), view.index(i))) {
+  int* const first_past = sc.shared_index;
+  for_each_in_order(view, seg_begin, seg_end, [&, first_past](float v, int index) {
+    if (keep(ordered(v), index)) {
       running += expf(v - scaled_max);
       if (running > target) {
-        atomicMin(sc.shared_index, view.index(i));
-        break;
+        atomicMin(first_past, index);
+        return false;
       }
     }
-  }
+    return true;
+  });
   __syncthreads();
   return *sc.shared_index;
 }
@@ -370,7 +456,15 @@ __global__ __launch_bounds__(kThreads) void sample_rows_kernel(const float* __re
   const int wave = tid / ms::kWave;
   const float* x = logits + static_cast<int64_t>(row) * vocab;
   const float temp = temperature ? temperature[row] : 0.f;
-  Scratch sc{f_scratch, i_scratch, seg_sum, seg_count, &shared_index, &shared_total, digit_count, digit_mass};
+  Scratch sc;        // member by member: as one constant aggregate of LDS addresses the compiler cannot emit it
+  sc.f_scratch = f_scratch;
+  sc.i_scratch = i_scratch;
+  sc.seg_sum = seg_sum;
+  sc.seg_count = seg_count;
+  sc.shared_index = &shared_index;
+  sc.shared_total = &shared_total;
+  sc.digit_count = digit_count;
+  sc.digit_mass = digit_mass;
 
   // ---- finiteness, maximum and its lowest index ---------------------------
   float best = -INFINITY;
@@ -888,6 +982,7 @@ __global__ __launch_bounds__(kChunkThreads) void sample_gather_kernel(const floa
 
 // The view of one chunk of a row, for the draw without top-k and top-p.
 struct ChunkView {
+  static constexpr bool kInDeviceMemory = true;
   const float* x;
   float temp;
   int begin;
@@ -920,7 +1015,15 @@ __global__ __launch_bounds__(kThreads) void sample_choose_kernel(const float* __
   const RowTables t = row_tables(workspace, row, vocab);
   const float* x = logits + static_cast<int64_t>(row) * vocab;
   const float temp = temperature[row];
-  Scratch sc{f_scratch, i_scratch, seg_sum, seg_count, &shared_index, &shared_total, digit_count, digit_mass};
+  Scratch sc;        // member by member: as one constant aggregate of LDS addresses the compiler cannot emit it
+  sc.f_scratch = f_scratch;
+  sc.i_scratch = i_scratch;
+  sc.seg_sum = seg_sum;
+  sc.seg_count = seg_count;
+  sc.shared_index = &shared_index;
+  sc.shared_total = &shared_total;
+  sc.digit_count = digit_count;
+  sc.digit_mass = digit_mass;
   bool bad;
   const float row_max = row_maximum(t, &bad);
   if (bad) {
@@ -965,7 +1068,7 @@ __global__ __launch_bounds__(kThreads) void sample_choose_kernel(const float* __
         const ListView list{list_values, list_indices, n};
         chosen = choose(list, vocab, scaled_max, cut_k ? k : 0, p, u, cut_k ? -1.f : whole_s, 0.f, sc);
       } else {
-        const ListView list{t.list_values, t.list_indices, n};      // a long list stays where it is
+        const LongListView list{t.list_values, t.list_indices, n};      // a long list stays where it is
         chosen = choose(list, vocab, scaled_max, cut_k ? k : 0, p, u, cut_k ? -1.f : whole_s, 0.f, sc);
       }
       if (tid == 0) out[row] = chosen;
