@@ -8,6 +8,8 @@
 // One workgroup per output row.  The number of threads and the kernel variant
 // depend on the row length only, so a row's result never depends on the rest of
 // the batch.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace {
@@ -85,6 +87,77 @@ __global__ void rmsnorm_registers_kernel(TIn* __restrict__ x, const T* __restric
   }
 }
 
+// Four values of the storage type to and from floats, as one 8- or 16-byte access.
+__device__ __forceinline__ void load4(const float* p, float (&f)[4]) {
+  const float4 raw = *reinterpret_cast<const float4*>(p);
+  f[0] = raw.x, f[1] = raw.y, f[2] = raw.z, f[3] = raw.w;
+}
+__device__ __forceinline__ void load4(const ms::bf16* p, float (&f)[4]) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  f[0] = __uint_as_float(raw.x << 16), f[1] = __uint_as_float(raw.x & 0xffff0000u);
+  f[2] = __uint_as_float(raw.y << 16), f[3] = __uint_as_float(raw.y & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float (&f)[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+}
+__device__ __forceinline__ void store4(ms::bf16* p, const float (&f)[4]) {
+  uint2 raw;
+  raw.x = ms::float_to_bf16_bits(f[0]) | (static_cast<uint32_t>(ms::float_to_bf16_bits(f[1])) << 16);
+  raw.y = ms::float_to_bf16_bits(f[2]) | (static_cast<uint32_t>(ms::float_to_bf16_bits(f[3])) << 16);
+  *reinterpret_cast<uint2*>(p) = raw;
+}
+
+// The residual stream's norm for rows of a multiple of four values, every operand aligned
+// to 16 bytes: the row in registers as above, four consecutive values a thread and access
+// (one 16-byte read of the 32-bit row, one 8-byte write of the bfloat16 output), 256 threads
+// for any row up to 16,384.  VPT such groups per thread.
+template <typename T, int VPT>
+__global__ void rmsnorm_by_fours_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                        const T* __restrict__ weight, T* __restrict__ out,
+                                        const int32_t* __restrict__ rows, int dim, float eps, int write_back) {
+  __shared__ float scratch[16];
+  const int64_t out_row = blockIdx.x;
+  const int64_t in_row = rows ? static_cast<int64_t>(rows[out_row]) : out_row;
+  float* xr = x + in_row * dim;
+  const T* dr = delta ? delta + in_row * dim : nullptr;
+  T* yr = out + out_row * dim;
+  const int groups = dim / 4;
+
+  float v[VPT][4];
+  float partial = 0.f;
+#pragma unroll
+  for (int e = 0; e < VPT; ++e) {
+    const int i = threadIdx.x + e * blockDim.x;
+    if (i < groups) {
+      load4(xr + 4 * i, v[e]);
+      if (dr) {
+        float d[4];
+        load4(dr + 4 * i, d);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[e][c] += d[c];
+        if (write_back) store4(xr + 4 * i, v[e]);
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) partial = fmaf(v[e][c], v[e][c], partial);
+    }
+  }
+  const float total = ms::block_sum(partial, scratch);
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(dim) + eps);
+#pragma unroll
+  for (int e = 0; e < VPT; ++e) {
+    const int i = threadIdx.x + e * blockDim.x;
+    if (i < groups) {
+      float w[4], y[4];
+      load4(weight + 4 * i, w);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) y[c] = w[c] * ms::round_to<T>(v[e][c] * inv);
+      store4(yr + 4 * i, y);
+    }
+  }
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
 template <typename TIn, typename T>
 void launch_rmsnorm(void* x, const void* delta, const void* weight, void* out, const void* rows, int n_out, int dim,
                     float eps, int write_back, hipStream_t stream) {
@@ -94,6 +167,22 @@ void launch_rmsnorm(void* x, const void* delta, const void* weight, void* out, c
   const T* wp = static_cast<const T*>(weight);
   T* op = static_cast<T*>(out);
   const int32_t* rp = static_cast<const int32_t*>(rows);
+  if constexpr (std::is_same<TIn, float>::value) {
+    // (the choice goes by the row's length and the operands' alignment, never by the number of rows)
+    if (dim % 4 == 0 && dim >= 256 && dim <= 16384 && aligned16(x) && aligned16(delta) && aligned16(weight) &&
+        aligned16(out)) {
+      const dim3 block(256);
+#define MS_NORM_BY_FOURS(VPT)                                                                                     \
+  hipLaunchKernelGGL((rmsnorm_by_fours_kernel<T, VPT>), grid, block, 0, stream, xp, dp, wp, op, rp, dim, eps, write_back)
+      if (dim <= 1024) MS_NORM_BY_FOURS(1);
+      else if (dim <= 2048) MS_NORM_BY_FOURS(2);
+      else if (dim <= 4096) MS_NORM_BY_FOURS(4);
+      else if (dim <= 8192) MS_NORM_BY_FOURS(8);
+      else MS_NORM_BY_FOURS(16);
+#undef MS_NORM_BY_FOURS
+      return;
+    }
+  }
   if (dim <= 64) {
     hipLaunchKernelGGL((rmsnorm_registers_kernel<TIn, T, 1>), grid, dim3(64), 0, stream, xp, dp, wp, op, rp, dim, eps, write_back);
   } else if (dim <= 256) {

@@ -79,10 +79,11 @@ def test_rmsnorm_shapes_of_the_reference_and_edges(ops, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_rmsnorm_residual_forms(ops, dtype):
-    residual = rand(6, 200, seed=1)
-    delta = rand(6, 200, seed=2, dtype=dtype)
-    weight = (1 + 0.1 * rand(200, seed=3)).to(dtype)
+@pytest.mark.parametrize("dim", [200, 256, 1028, 2056, 5120, 9000, 16388])      # both kernels, every number of groups a thread
+def test_rmsnorm_residual_forms(ops, dtype, dim):
+    residual = rand(6, dim, seed=1)
+    delta = rand(6, dim, seed=2, dtype=dtype)
+    weight = (1 + 0.1 * rand(dim, seed=3)).to(dtype)
     total = residual + delta.float()
     kept = residual.clone()
     out = ops.rmsnorm(kept, weight, 1e-5, delta=delta, write_back=True)
