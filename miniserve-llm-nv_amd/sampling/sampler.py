@@ -11,12 +11,13 @@ from __future__ import annotations
 
 import os
 from dataclasses import dataclass
-from typing import Sequence
+from typing import TYPE_CHECKING, Sequence
 
 import numpy as np
 import torch
 
-from ..engine.request import SamplingParams
+if TYPE_CHECKING:       # for the annotations only: the engine package imports this one
+    from ..engine.request import SamplingParams
 
 _BELOW_ONE = 1.0 - 2.0**-24      # largest float32 below 1
 
