@@ -839,6 +839,32 @@ def test_sampling_from_the_short_list_and_from_the_whole_row(ops):
         assert out[row] == expected, f"row {row}: T={temperature[row]} k={top_k[row]} p={top_p[row]} u={uniform[row]}"
 
 
+def test_sampling_from_flat_rows_of_the_served_vocabulary(ops):
+    """Rows without outstanding tokens (a model with random weights gives such rows), 151,936
+    tokens wide: no distance below the maximum holds the tokens that can stay, so the choice
+    walks a list as long as the row or the row itself; with a small top-k the list is short
+    again.  Every row gives the plain implementation's token."""
+
+    vocab = 151936
+    generator = torch.Generator().manual_seed(21)
+    options = [(0.8, 0, 0.9), (0.8, 0, 0.5), (1.0, 5000, 1.0), (0.8, 50, 0.9), (1.5, 0, 0.99), (0.7, 20000, 0.7),
+               (1.0, 0, 1.0), (0.8, 1, 0.9)]
+    rows = len(options)
+    logits = torch.randn(rows, vocab, generator=generator) * torch.tensor([0.2, 0.64] * (rows // 2))[:, None]
+    temperature = torch.tensor([o[0] for o in options])
+    top_k = torch.tensor([o[1] for o in options], dtype=torch.int32)
+    top_p = torch.tensor([o[2] for o in options])
+    for trial in range(3):
+        uniform = torch.rand(rows, generator=generator)
+        out = ops.sample_rows(logits.to(DEVICE), temperature=temperature.to(DEVICE), top_k=top_k.to(DEVICE),
+                              top_p=top_p.to(DEVICE), uniform=uniform.to(DEVICE)).cpu().tolist()
+        for row in range(rows):
+            expected = plain_sampling.sample_row(
+                logits[row], float(temperature[row]), int(top_k[row]), float(top_p[row]), float(uniform[row])
+            )
+            assert out[row] == expected, f"trial {trial} row {row}: T={temperature[row]} k={top_k[row]} p={top_p[row]} u={uniform[row]}"
+
+
 def test_equal_values_at_the_edge_of_top_k_keep_the_lowest_indices(ops):
     """A hundred tokens share the k-th largest value, spread over a long row: exactly k
     tokens stay, the equal ones with the lowest indices, and every one of them can be drawn."""
