@@ -219,11 +219,14 @@ __device__ __forceinline__ void for_each_in_order(const View& view, int begin, i
 // every token's; `whole_mass`: the mass of all tokens where the view holds only some
 // of them and top-k is off (top_p is a share of that), else negative; `mass_before`:
 // with top-k and top-p off and a view that is one part of the row, the mass of the
-// tokens before it (the draw is then at uniform * whole_mass).  All threads of the
-// workgroup call it and get the same result.
+// tokens before it (the draw is then at uniform * whole_mass).  `preset_p_threshold`: the
+// threshold of top-p where it was found elsewhere (p is 1 then, and whole_mass and
+// mass_before are those of the kept tokens).  All threads of the workgroup call it and get
+// the same result.
 template <typename View>
 __device__ int choose(const View& view, int limit_index, float scaled_max, int k, float p, float uniform,
-                      float whole_mass, float mass_before, const Scratch& sc) {
+                      float whole_mass, float mass_before, const Scratch& sc,
+                      const uint32_t* preset_p_threshold = nullptr) {
   const int tid = threadIdx.x;
   const int n = view.size;
   // Contiguous segment of this thread, for everything that needs token order.
@@ -231,12 +234,13 @@ __device__ int choose(const View& view, int limit_index, float scaled_max, int k
   const int seg_begin = min(tid * seg, n);
   const int seg_end = min(seg_begin + seg, n);
 
-  if (n <= kSmallView) return choose_among_few(view, limit_index, scaled_max, k, p, uniform, whole_mass, mass_before, sc);
+  if (n <= kSmallView && preset_p_threshold == nullptr)
+    return choose_among_few(view, limit_index, scaled_max, k, p, uniform, whole_mass, mass_before, sc);
 
   Keep keep;
   keep.k_threshold = 0u;
   keep.tie_limit = limit_index;
-  keep.p_threshold = 0u;
+  keep.p_threshold = preset_p_threshold ? *preset_p_threshold : 0u;
 
   // ---- top-k ----------------------------------------------------------------
   if (k > 0 && k < n) {
@@ -753,17 +757,38 @@ constexpr int kRowChunks = 32;
 constexpr int kChunkThreads = 256;
 constexpr int kChunkWaves = kChunkThreads / ms::kWave;
 
+// Top-p alone over a row whose nucleus is no short list (a flat row: most of the vocabulary
+// stays): the threshold is searched by all chunks together, eight bits a pass.  A pass adds
+// the mass of every token to the bin of its next eight bits, in integers (a token's weight
+// times 2^40, rounded down), so that the sums do not depend on the order in which the
+// workgroups add; the tables of the passes and what the search leaves for the choice:
+constexpr int kNucleusPasses = 4;
+constexpr int kNucleusBins = 256;
+constexpr float kNucleusScale = 1099511627776.0f;      // 2^40
+// A list of up to this many tokens is searched by the one workgroup of the choice (about
+// 5 us per thousand tokens); a longer one, or none, by the chunks (some 80 us whatever the length).
+constexpr int kNucleusFrom = 24576;
+
 struct RowTables {
   float* chunk_max;
   int* chunk_arg;
   int* ladder_count;
   float* ladder_mass;
+  int* nucleus_flag;                  // 1: the row's threshold is searched by the chunks together
+  uint32_t* nucleus_threshold;        // the result: tokens whose ordered value reaches it stay
+  float* kept_mass;                   // [chunks]: the mass of the tokens that stay
+  unsigned long long* histogram;      // [kNucleusPasses][kNucleusBins]
+  unsigned long long* search_state;   // [kNucleusPasses][3]: what the search knew after each pass (NucleusSearch)
   float* list_values;
   int* list_indices;
 };
 
+constexpr size_t kRowFixedFloats = static_cast<size_t>(kRowChunks) * (2 + kLadder + kLadder + 1) + 2 + kRowChunks +
+                                   2 * static_cast<size_t>(kNucleusPasses) * (kNucleusBins + 3);
+static_assert((kRowChunks * (2 + kLadder + kLadder + 1) + 2 + kRowChunks) % 2 == 0, "the histogram is read as 64-bit words");
+
 __host__ __device__ inline size_t row_table_floats(int vocab) {
-  return static_cast<size_t>(kRowChunks) * (2 + kLadder + kLadder + 1) + 2 * static_cast<size_t>(vocab);
+  return kRowFixedFloats + 2 * static_cast<size_t>(vocab);
 }
 
 __device__ __forceinline__ RowTables row_tables(float* workspace, int row, int vocab) {
@@ -773,7 +798,13 @@ __device__ __forceinline__ RowTables row_tables(float* workspace, int row, int v
   t.chunk_arg = reinterpret_cast<int*>(base + kRowChunks);
   t.ladder_count = reinterpret_cast<int*>(base + 2 * kRowChunks);
   t.ladder_mass = base + 2 * kRowChunks + kRowChunks * kLadder;
-  t.list_values = base + 2 * kRowChunks + kRowChunks * (2 * kLadder + 1);
+  float* next = base + 2 * kRowChunks + kRowChunks * (2 * kLadder + 1);
+  t.nucleus_flag = reinterpret_cast<int*>(next);
+  t.nucleus_threshold = reinterpret_cast<uint32_t*>(next + 1);
+  t.kept_mass = next + 2;
+  t.histogram = reinterpret_cast<unsigned long long*>(next + 2 + kRowChunks);
+  t.search_state = t.histogram + kNucleusPasses * kNucleusBins;
+  t.list_values = base + kRowFixedFloats;
   t.list_indices = reinterpret_cast<int*>(t.list_values + vocab);
   return t;
 }
@@ -836,7 +867,11 @@ __global__ __launch_bounds__(kChunkThreads) void sample_scan_kernel(const float*
     for (int w = 0; w < kChunkWaves; ++w) any_bad += i_scratch[w];
     t.chunk_max[chunk] = chunk_best;                 // -inf for a chunk past the row's end
     t.chunk_arg[chunk] = any_bad ? -1 : shared_index;
+    if (chunk == 0) *t.nucleus_flag = 0;
   }
+  // every chunk clears its share of the tables that the search of a nucleus adds into
+  constexpr int kShare = kNucleusPasses * kNucleusBins / kRowChunks;
+  if (tid < kShare) t.histogram[chunk * kShare + tid] = 0ull;
 }
 
 // The row's maximum and whether any chunk met a non-finite value, from stage 1's table.
@@ -914,7 +949,8 @@ __global__ __launch_bounds__(kChunkThreads) void sample_gather_kernel(const floa
                                                                       const float* __restrict__ temperature,
                                                                       const int32_t* __restrict__ top_k,
                                                                       const float* __restrict__ top_p,
-                                                                      float* __restrict__ workspace, int vocab) {
+                                                                      float* __restrict__ workspace, int vocab,
+                                                                      int search_nucleus) {
   __shared__ int rung_s, base_s;
   __shared__ int wave_count[kChunkWaves];
   const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
@@ -935,7 +971,11 @@ __global__ __launch_bounds__(kChunkThreads) void sample_gather_kernel(const floa
     int base = 0;
     if (rung >= 0)
       for (int c = 0; c < chunk; ++c) base += t.ladder_count[c * kLadder + rung];
-    rung_s = rung;
+    // top-p alone and no short list: the chunks search the threshold together (the kernels
+    // after this one), nothing is gathered
+    const bool together = search_nucleus && !cut_k && (rung < 0 || total > kNucleusFrom);
+    if (together && chunk == 0) *t.nucleus_flag = 1;
+    rung_s = together ? -1 : rung;
     base_s = base;
   }
   __syncthreads();
@@ -977,6 +1017,130 @@ __global__ __launch_bounds__(kChunkThreads) void sample_gather_kernel(const floa
       }
     }
     written += round_total;
+  }
+}
+
+// What the search knows after some of its passes: the bits of the threshold found so far,
+// the mass of the tokens that lie above every value with those bits, and the mass that the
+// kept tokens must exceed.
+struct NucleusSearch {
+  uint32_t prefix;
+  unsigned long long above;
+  unsigned long long limit;
+};
+
+// Inclusive sum over this lane and the higher lanes of the wave.
+__device__ __forceinline__ unsigned long long wave_sum_from_here_up(unsigned long long v) {
+  const int lane = threadIdx.x & (ms::kWave - 1);
+#pragma unroll
+  for (int step = 1; step < ms::kWave; step <<= 1) {
+    const unsigned low = __shfl_down(static_cast<unsigned>(v), step, ms::kWave);
+    const unsigned high = __shfl_down(static_cast<unsigned>(v >> 32), step, ms::kWave);
+    if (lane + step < ms::kWave) v += (static_cast<unsigned long long>(high) << 32) | low;
+  }
+  return v;
+}
+
+// The state after pass `pass`, from the state before it (kept in the row's tables by the
+// kernel before this one; nothing before pass 0) and the pass's histogram.  All 256 threads
+// of the workgroup call it, a thread a bin, and get the same answer; chunk 0 keeps it for
+// the next kernel.
+__device__ NucleusSearch nucleus_search_after(const RowTables& t, int pass, float p, bool keep_it,
+                                              unsigned long long* group_s, unsigned long long* word_s, int* digit_s) {
+  const int tid = threadIdx.x;
+  NucleusSearch state{0u, 0ull, 0ull};
+  if (pass > 0) {
+    state.prefix = static_cast<uint32_t>(t.search_state[3 * (pass - 1)]);
+    state.above = t.search_state[3 * (pass - 1) + 1];
+    state.limit = t.search_state[3 * (pass - 1) + 2];
+  }
+  const unsigned long long bin = t.histogram[pass * kNucleusBins + tid];
+  unsigned long long reached = wave_sum_from_here_up(bin);      // this bin and the higher ones of its wave
+  if ((tid & (ms::kWave - 1)) == 0) group_s[tid / ms::kWave] = reached;
+  if (tid == 0) *digit_s = 0;
+  __syncthreads();
+  for (int g = tid / ms::kWave + 1; g < kChunkWaves; ++g) reached += group_s[g];
+  reached += state.above;
+  if (pass == 0) {
+    if (tid == 0) *word_s = reached;                 // the whole row's mass
+    __syncthreads();
+    state.limit = static_cast<unsigned long long>(static_cast<double>(p) * static_cast<double>(*word_s));
+    __syncthreads();
+  }
+  // the threshold's next eight bits: the highest bin from which on the mass still exceeds the limit
+  if (reached > state.limit) atomicMax(digit_s, tid);
+  __syncthreads();
+  const int digit = *digit_s;
+  if (tid == digit) *word_s = reached - bin;
+  __syncthreads();
+  state.above = *word_s;
+  state.prefix |= static_cast<uint32_t>(digit) << (24 - 8 * pass);
+  if (keep_it && tid == 0) {
+    t.search_state[3 * pass] = state.prefix;
+    t.search_state[3 * pass + 1] = state.above;
+    t.search_state[3 * pass + 2] = state.limit;
+  }
+  __syncthreads();
+  return state;
+}
+
+// One pass of the search (pass 0 .. kNucleusPasses - 1), or (pass == kNucleusPasses) what
+// the choice needs of its result: the threshold and every chunk's mass of kept tokens.
+__global__ __launch_bounds__(kChunkThreads) void sample_nucleus_kernel(const float* __restrict__ logits,
+                                                                       const float* __restrict__ temperature,
+                                                                       const float* __restrict__ top_p,
+                                                                       float* __restrict__ workspace, int vocab,
+                                                                       int pass) {
+  static_assert(kChunkThreads == kNucleusBins, "a thread a bin");
+  __shared__ unsigned long long mine_s[kNucleusBins];
+  __shared__ unsigned long long group_s[kChunkWaves];
+  __shared__ unsigned long long word_s;
+  __shared__ int digit_s;
+  __shared__ float mass_s[kChunkWaves];
+  const int row = blockIdx.y, chunk = blockIdx.x, tid = threadIdx.x;
+  const RowTables t = row_tables(workspace, row, vocab);
+  if (*t.nucleus_flag == 0) return;
+  const float temp = temperature[row];
+  const float p = top_p[row];
+  bool bad;
+  const float scaled_max = row_maximum(t, &bad) / temp;
+  // (kernel `pass` works out what pass - 1 found; the first has nothing to work out)
+  NucleusSearch found{0u, 0ull, 0ull};
+  if (pass > 0) found = nucleus_search_after(t, pass - 1, p, chunk == 0, group_s, &word_s, &digit_s);
+  const int length = chunk_length(vocab);
+  const int begin = min(chunk * length, vocab), end = min(begin + length, vocab);
+  const float* x = logits + static_cast<int64_t>(row) * vocab;
+  if (pass < kNucleusPasses) {
+    const int shift = 24 - 8 * pass;
+    mine_s[tid] = 0ull;
+    __syncthreads();
+    for (int i = begin + tid; i < end; i += kChunkThreads) {
+      const float v = x[i] / temp;
+      const uint32_t o = ordered(v);
+      // (in pass 0 every token has the bits above the pass's: there are none)
+      if (pass == 0 || ((o ^ found.prefix) >> (shift + 8)) == 0u) {
+        const unsigned long long weight = static_cast<unsigned long long>(expf(v - scaled_max) * kNucleusScale);
+        if (weight != 0ull) atomicAdd(&mine_s[(o >> shift) & 255u], weight);
+      }
+    }
+    __syncthreads();
+    if (mine_s[tid] != 0ull) atomicAdd(&t.histogram[pass * kNucleusBins + tid], mine_s[tid]);
+    return;
+  }
+  // the search is over: found.prefix is the threshold
+  float mass = 0.f;
+  for (int i = begin + tid; i < end; i += kChunkThreads) {
+    const float v = x[i] / temp;
+    if (ordered(v) >= found.prefix) mass += expf(v - scaled_max);
+  }
+  mass = ms::wave_sum(mass);
+  if ((tid & (ms::kWave - 1)) == 0) mass_s[tid / ms::kWave] = mass;
+  __syncthreads();
+  if (tid == 0) {
+    float sum = 0.f;
+    for (int w = 0; w < kChunkWaves; ++w) sum += mass_s[w];
+    t.kept_mass[chunk] = sum;
+    if (chunk == 0) *t.nucleus_threshold = found.prefix;
   }
 }
 
@@ -1047,6 +1211,42 @@ __global__ __launch_bounds__(kThreads) void sample_choose_kernel(const float* __
   const bool cut_p = p < 1.f;
   const float u = uniform[row];
 
+  if (cut_p && !cut_k && *t.nucleus_flag != 0) {
+    // The chunks have searched the threshold together and left every chunk's mass of kept
+    // tokens: the chunk in which the running mass passes uniform * the kept mass is found
+    // from those, and the draw is made inside it, among its kept tokens.
+    if (tid == 0) {
+      float kept = 0.f;
+      for (int c = 0; c < kRowChunks; ++c) kept += t.kept_mass[c];
+      const float target = u * kept;
+      float running = 0.f, before = 0.f;
+      int chunk = -1, last_live = 0;
+      for (int c = 0; c < kRowChunks; ++c) {
+        const float mass = t.kept_mass[c];
+        if (mass > 0.f) last_live = c;
+        if (chunk < 0 && running + mass > target) {
+          chunk = c;
+          before = running;
+        }
+        running += mass;
+      }
+      if (chunk < 0) {                          // rounding: the target lies at the very end
+        chunk = last_live;
+        before = -INFINITY;                     // nothing in the chunk passes the target: its last kept token is taken
+      }
+      chunk_s = chunk;
+      before_s = before;
+      whole_s = kept;
+    }
+    __syncthreads();
+    const int length = chunk_length(vocab);
+    const int begin = min(chunk_s * length, vocab), end = min(begin + length, vocab);
+    const ChunkView part{x, temp, begin, end - begin};
+    const uint32_t threshold = *t.nucleus_threshold;
+    const int chosen = choose(part, vocab, scaled_max, 0, 1.f, u, whole_s, before_s, sc, &threshold);
+    if (tid == 0) out[row] = chosen;
+    return;
+  }
   if (cut_k || cut_p) {
     if (tid == 0) {
       float whole;
@@ -1136,18 +1336,23 @@ extern "C" size_t ms_sample_rows_workspace_bytes(int rows, int vocab) {
 
 // The same choice as ms_sample_rows for a large vocabulary, the passes over a row
 // shared by 32 workgroups; temperature is not null.  workspace: device memory of
-// ms_sample_rows_workspace_bytes(rows, vocab), aligned to 4 bytes, the caller's until the
-// call's work on the stream is done.
+// ms_sample_rows_workspace_bytes(rows, vocab), aligned to 8 bytes, the caller's until the
+// call's work on the stream is done.  search_nucleus: not 0 if some row may have top-p
+// without top-k (then the kernels that search such a row's threshold with all chunks are
+// launched; a row decides for itself whether it needs them); 0 spares their launches.
 extern "C" int ms_sample_rows_chunked(const void* logits, const void* temperature, const void* top_k,
                                       const void* top_p, const void* uniform, void* out, void* workspace,
-                                      size_t workspace_bytes, int rows, int vocab, hipStream_t stream) {
+                                      size_t workspace_bytes, int rows, int vocab, int search_nucleus,
+                                      hipStream_t stream) {
   MS_REQUIRE(rows > 0 && rows <= 65535 && vocab > 0, "sample_rows_chunked: bad shape %d x %d", rows, vocab);
   MS_REQUIRE(temperature && uniform, "sample_rows_chunked: temperature and uniform numbers are needed");
   MS_REQUIRE(workspace && workspace_bytes >= ms_sample_rows_workspace_bytes(rows, vocab),
              "sample_rows_chunked: the workspace has %zu bytes, %zu are needed", workspace_bytes,
              ms_sample_rows_workspace_bytes(rows, vocab));
+  MS_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7u) == 0, "sample_rows_chunked: the workspace is not aligned to 8 bytes");
   float* tables = static_cast<float*>(workspace);
   const dim3 grid(kRowChunks, rows);
+  const int together = search_nucleus != 0 && top_p != nullptr;
   hipLaunchKernelGGL(sample_scan_kernel, grid, dim3(kChunkThreads), 0, stream, static_cast<const float*>(logits),
                      tables, vocab);
   MS_CHECK_LAUNCH("sample_scan");
@@ -1156,8 +1361,15 @@ extern "C" int ms_sample_rows_chunked(const void* logits, const void* temperatur
   MS_CHECK_LAUNCH("sample_ladder");
   hipLaunchKernelGGL(sample_gather_kernel, grid, dim3(kChunkThreads), 0, stream, static_cast<const float*>(logits),
                      static_cast<const float*>(temperature), static_cast<const int32_t*>(top_k),
-                     static_cast<const float*>(top_p), tables, vocab);
+                     static_cast<const float*>(top_p), tables, vocab, together);
   MS_CHECK_LAUNCH("sample_gather");
+  if (together) {
+    for (int pass = 0; pass <= kNucleusPasses; ++pass) {
+      hipLaunchKernelGGL(sample_nucleus_kernel, grid, dim3(kChunkThreads), 0, stream, static_cast<const float*>(logits),
+                         static_cast<const float*>(temperature), static_cast<const float*>(top_p), tables, vocab, pass);
+      MS_CHECK_LAUNCH("sample_nucleus");
+    }
+  }
   hipLaunchKernelGGL(sample_choose_kernel, dim3(rows), dim3(kThreads), 0, stream, static_cast<const float*>(logits),
                      static_cast<const float*>(temperature), static_cast<const int32_t*>(top_k),
                      static_cast<const float*>(top_p), static_cast<const float*>(uniform), tables,

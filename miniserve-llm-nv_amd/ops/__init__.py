@@ -635,7 +635,7 @@ SAMPLE_CHUNKED_FROM = 8192
 def _sample_row_table_bytes(vocab: int) -> int:
     """Bytes a row that the stages of the chunked choice share (csrc/sampling.hip: row_table_floats)."""
 
-    return 4 * (32 * (2 + 8 + 8 + 1) + 2 * vocab)
+    return 4 * (32 * (2 + 8 + 8 + 1) + 2 + 32 + 2 * 4 * (256 + 3) + 2 * vocab)
 
 
 def sample_rows(
@@ -645,12 +645,14 @@ def sample_rows(
     top_k: torch.Tensor | None = None,
     top_p: torch.Tensor | None = None,
     uniform: torch.Tensor | None = None,
+    top_p_alone: bool = True,
 ) -> torch.Tensor:
     """One token per row of float32 ``logits [R, V]`` -> int32 ``[R]``.
 
     ``temperature`` None or 0 in a row: argmax.  Otherwise temperature, top-k
     (0 = off), top-p (1 = off), then the inverse CDF at ``uniform[r]`` in token
-    order.  A row with a non-finite logit gives -1."""
+    order.  A row with a non-finite logit gives -1.  ``top_p_alone``: False when the
+    caller knows that no row has top-p without top-k (a few small launches are spared)."""
 
     _check(logits, "logits", dtype=torch.float32)
     if logits.ndim != 2 or logits.numel() == 0:
@@ -679,7 +681,7 @@ def sample_rows(
         # the list of the tokens that can stay
         workspace = torch.empty(rows * _sample_row_table_bytes(vocab), dtype=torch.uint8, device=logits.device)
         call("ms_sample_rows_chunked", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
-             _ptr(out), _ptr(workspace), workspace.numel(), rows, vocab, _stream())
+             _ptr(out), _ptr(workspace), workspace.numel(), rows, vocab, int(bool(top_p_alone) and top_p is not None), _stream())
         return out
     call("ms_sample_rows", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(out),
          rows, vocab, _stream())

@@ -42,7 +42,7 @@ _SIGNATURES: dict[str, list] = {
     "ms_sample_rows": [_P, _P, _P, _P, _P, _P, _I, _I, _P],
     "ms_argmax_rows": [_P, _P, _P, _P, _I, _I, _I, _P],
     "ms_sample_rows_workspace_bytes": [_I, _I],
-    "ms_sample_rows_chunked": [_P, _P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _P],
+    "ms_sample_rows_chunked": [_P, _P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _P],
 }
 
 _lock = threading.Lock()
