@@ -858,6 +858,11 @@ def test_sampling_from_flat_rows_of_the_served_vocabulary(ops):
         uniform = torch.rand(rows, generator=generator)
         out = ops.sample_rows(logits.to(DEVICE), temperature=temperature.to(DEVICE), top_k=top_k.to(DEVICE),
                               top_p=top_p.to(DEVICE), uniform=uniform.to(DEVICE)).cpu().tolist()
+        # (the rows with top-p alone were searched by their chunks together; without those kernels the one
+        # workgroup of the choice searches them, and finds the same)
+        alone = ops.sample_rows(logits.to(DEVICE), temperature=temperature.to(DEVICE), top_k=top_k.to(DEVICE),
+                                top_p=top_p.to(DEVICE), uniform=uniform.to(DEVICE), top_p_alone=False).cpu().tolist()
+        assert alone == out
         for row in range(rows):
             expected = plain_sampling.sample_row(
                 logits[row], float(temperature[row]), int(top_k[row]), float(top_p[row]), float(uniform[row])
