@@ -65,6 +65,7 @@ def _declare(lib: ctypes.CDLL) -> None:
             ) from None
         function.restype = c_int
         function.argtypes = argtypes
+    lib.ms_sample_rows_workspace_bytes.restype = c_size_t      # a size, not a status
 
 
 def load() -> ctypes.CDLL:

@@ -870,6 +870,18 @@ def test_sampling_from_flat_rows_of_the_served_vocabulary(ops):
             assert out[row] == expected, f"trial {trial} row {row}: T={temperature[row]} k={top_k[row]} p={top_p[row]} u={uniform[row]}"
 
 
+def test_the_sampling_workspace_has_the_size_the_library_asks_for(ops):
+    """The Python side sizes the workspace of the chunked choice from a formula of its own;
+    the library's entry point names the size it checks against.  They must agree."""
+
+    from miniserve_amd.ops import _sample_row_table_bytes
+    from miniserve_amd.ops.library import load
+
+    wanted = load().ms_sample_rows_workspace_bytes
+    for rows, vocab in [(1, 8192), (3, 50021), (64, 151936)]:
+        assert wanted(rows, vocab) == rows * _sample_row_table_bytes(vocab)
+
+
 def test_equal_values_at_the_edge_of_top_k_keep_the_lowest_indices(ops):
     """A hundred tokens share the k-th largest value, spread over a long row: exactly k
     tokens stay, the equal ones with the lowest indices, and every one of them can be drawn."""
