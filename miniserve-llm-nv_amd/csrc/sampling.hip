@@ -88,8 +88,8 @@ using LongListView = ListViewAt<true>;       // too long for that: where the gat
 constexpr int kListCap = 4096;      // tokens that the short list holds at most
 // Distances below the row's maximum (in units of logit / temperature) at which the
 // row is cut to make the short list: the first of them that keeps enough is taken.
-constexpr int kLadder = 8;
-constexpr float kLadderDepth[kLadder] = {1.f, 2.f, 4.f, 6.f, 9.f, 13.f, 18.f, 26.f};
+constexpr int kLadder = 10;
+constexpr float kLadderDepth[kLadder] = {0.25f, 0.5f, 1.f, 2.f, 4.f, 6.f, 9.f, 13.f, 18.f, 26.f};
 
 struct Scratch {
   float* f_scratch;       // [kWaves]

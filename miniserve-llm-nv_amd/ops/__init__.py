@@ -635,7 +635,7 @@ SAMPLE_CHUNKED_FROM = 8192
 def _sample_row_table_bytes(vocab: int) -> int:
     """Bytes a row that the stages of the chunked choice share (csrc/sampling.hip: row_table_floats)."""
 
-    return 4 * (32 * (2 + 8 + 8 + 1) + 2 + 32 + 2 * 4 * (256 + 3) + 2 * vocab)
+    return 4 * (32 * (2 + 10 + 10 + 1) + 2 + 32 + 2 * 4 * (256 + 3) + 2 * vocab)
 
 
 def sample_rows(
