@@ -750,9 +750,11 @@ extern "C" int ms_argmax_rows_static(const void* logits, void* out, int rows, in
 // the list, or, without top-k and top-p, inside the chunk that the running mass
 // singles out, or - no rung of the ladder holds the candidates - over the whole row as above.
 // The list lies in device memory and may be as long as the row; the last stage copies
-// it into LDS when it is short.  Tables between the stages (per row): chunk_max,
+// it into LDS when it is short.  Between (3) and (4), for rows with top-p alone and a long
+// nucleus, the chunks search the threshold together (sample_nucleus_kernel, below) and
+// nothing is gathered.  Tables between the stages (per row): chunk_max,
 // chunk_arg [chunks]; ladder_count [chunks][kLadder]; ladder_mass [chunks][kLadder + 1];
-// list_values, list_indices [vocab].
+// the tables of the search; list_values, list_indices [vocab].
 constexpr int kRowChunks = 32;
 constexpr int kChunkThreads = 256;
 constexpr int kChunkWaves = kChunkThreads / ms::kWave;
