@@ -33,6 +33,8 @@ struct Api {
   decltype(&hipblasLtMatmulPreferenceDestroy) pref_destroy = nullptr;
   decltype(&hipblasLtMatmulAlgoGetHeuristic) heuristic = nullptr;
   decltype(&hipblasLtMatmul) matmul = nullptr;
+  decltype(&hipblasLtMatmulDescDestroy) desc_destroy = nullptr;
+  decltype(&hipblasLtMatrixLayoutDestroy) layout_destroy = nullptr;
 };
 
 struct Plan {
@@ -49,11 +51,8 @@ std::map<std::tuple<int, int, int, int, int>, Plan> g_plans;            // (devi
 constexpr size_t kMaxPlans = 4096;
 
 constexpr int kCandidates = 8;
-// Row counts that share one timing: the solution that was fastest for the first row
-// count of a bucket is taken for the others where the library offers it for them, so
-// that a stream of ever new row counts (portions of prompts beside decode tokens) does
-// not stop to time each of them.  Few rows, where a decode step is nothing but these
-// products, in fine buckets; many rows in buckets of 256.
+// Row counts that share one choice of algorithm: few rows, where a decode step is
+// nothing but these products, in fine buckets; many rows in buckets of 256.
 int tune_bucket(int m) {
   if (m <= 8) return 0;
   if (m <= 16) return 1;
@@ -63,12 +62,13 @@ int tune_bucket(int m) {
   if (m < 256) return 5;
   return 5 + m / 256;
 }
-// The solution that timing chose for (device, n, k, out is float, tune_bucket(m)).
-std::map<std::tuple<int, int, int, int, int>, int> g_tuned;
-// What is written between two timed runs so that each finds the matrix in memory, not
-// in the caches (the last-level cache holds 256 MiB): a decode step meets every matrix
-// cold, and among candidates that are timed warm the wrong one wins.
-constexpr size_t kFlushBytes = static_cast<size_t>(384) << 20;
+// Which of the library's candidates runs a product is a fixed rule, so that the same
+// model gives the same 32-bit sums in every process: the solution that was pinned for
+// (n, k, out is float, tune_bucket(m)) where the library offers it among its candidates
+// for the shape, else the library's own first choice.  Nothing is timed while the engine
+// serves; the pins come from a table that was measured once (ms_gemm_library_time) and
+// is kept with the sources.
+std::map<std::tuple<int, int, int, int>, int> g_pinned;
 
 // What the library itself calls the index of an algorithm: the first integer of its
 // opaque data.  Used only to recognise a candidate among those offered for a shape.
@@ -78,64 +78,45 @@ int solution_index(const hipblasLtMatmulAlgo_t& algo) {
   return index;
 }
 
-// Index of the candidate that runs this product fastest: the least of three timed runs
-// each, after one that is not counted, the caches flushed before every timed run (where
-// the memory for that is to be had).  The output goes to memory of its own, so that
-// `out` is written once, by the call.
-int fastest_candidate(hipblasLtHandle_t handle, const Plan& plan, const hipblasLtMatmulHeuristicResult_t* candidates,
-                      int count, const void* x, const void* w, int m, int n, int out_float, void* workspace,
-                      size_t workspace_bytes, hipStream_t stream) {
-  void* scratch = nullptr;
-  const size_t bytes = static_cast<size_t>(m) * n * (out_float ? 4 : 2);
-  if (hipMalloc(&scratch, bytes) != hipSuccess) return 0;
-  void* flush = nullptr;
-  if (hipMalloc(&flush, kFlushBytes) != hipSuccess) {
-    flush = nullptr;
-    (void)hipGetLastError();      // timed warm then
+struct Candidates {
+  hipblasLtMatmulHeuristicResult_t result[kCandidates];
+  int count = 0;
+};
+
+// Descriptors of out[m, n] = x[m, k] . w[n, k]^T and the library's candidates for it.
+int describe(hipblasLtHandle_t handle, int m, int n, int k, int out_float, size_t workspace_bytes, Plan& plan,
+             Candidates& candidates) {
+  const hipDataType out_type = out_float ? HIP_R_32F : HIP_R_16BF;
+  const int32_t transpose = HIPBLAS_OP_T, keep = HIPBLAS_OP_N;
+  bool ok = g_api.desc_create(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && g_api.desc_set(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &transpose, sizeof(transpose)) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && g_api.desc_set(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &keep, sizeof(keep)) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && g_api.layout_create(&plan.a, HIP_R_16BF, k, n, k) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && g_api.layout_create(&plan.b, HIP_R_16BF, k, m, k) == HIPBLAS_STATUS_SUCCESS;
+  ok = ok && g_api.layout_create(&plan.c, out_type, n, m, n) == HIPBLAS_STATUS_SUCCESS;
+  MS_REQUIRE(ok, "gemm_library: cannot describe %d x %d x %d", m, n, k);
+  hipblasLtMatmulPreference_t preference = nullptr;
+  MS_REQUIRE(g_api.pref_create(&preference) == HIPBLAS_STATUS_SUCCESS, "gemm_library: no preference object");
+  const uint64_t limit = workspace_bytes;
+  g_api.pref_set(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit));
+  const hipblasStatus_t status = g_api.heuristic(handle, plan.desc, plan.a, plan.b, plan.c, plan.c, preference,
+                                                 kCandidates, candidates.result, &candidates.count);
+  g_api.pref_destroy(preference);
+  MS_REQUIRE(status == HIPBLAS_STATUS_SUCCESS && candidates.count > 0, "gemm_library: no algorithm for %d x %d x %d", m, n, k);
+  return 0;
+}
+
+int handle_of_current_device(hipblasLtHandle_t** out) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return ms_fail("gemm_library: no current device");
+  MS_REQUIRE(g_api.library != nullptr, "gemm_library: ms_gemm_library_open was not called");
+  hipblasLtHandle_t& handle = g_handles[device];
+  if (handle == nullptr && g_api.create(&handle) != HIPBLAS_STATUS_SUCCESS) {
+    g_handles.erase(device);
+    return ms_fail("gemm_library: hipblasLtCreate failed");
   }
-  hipEvent_t begin = nullptr, end = nullptr;
-  int best = 0;
-  if (hipEventCreate(&begin) == hipSuccess && hipEventCreate(&end) == hipSuccess) {
-    const float alpha = 1.0f, beta = 0.0f;
-    float least[kCandidates];
-    bool usable[kCandidates];
-    const auto run = [&](int i) {
-      return g_api.matmul(handle, plan.desc, &alpha, w, plan.a, x, plan.b, &beta, scratch, plan.c, scratch, plan.c,
-                          &candidates[i].algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
-    };
-    for (int i = 0; i < count && i < kCandidates; ++i) {
-      least[i] = 0.f;
-      usable[i] = candidates[i].state == HIPBLAS_STATUS_SUCCESS && candidates[i].workspaceSize <= workspace_bytes && run(i);
-    }
-    for (int trial = 0; trial < 3; ++trial) {
-      for (int i = 0; i < count && i < kCandidates; ++i) {
-        if (!usable[i]) continue;
-        float ms = 0.f;
-        bool ok = flush == nullptr || hipMemsetAsync(flush, trial, kFlushBytes, stream) == hipSuccess;
-        ok = ok && hipEventRecord(begin, stream) == hipSuccess && run(i) && hipEventRecord(end, stream) == hipSuccess &&
-             hipEventSynchronize(end) == hipSuccess && hipEventElapsedTime(&ms, begin, end) == hipSuccess;
-        if (!ok) {
-          usable[i] = false;
-          (void)hipGetLastError();
-        } else if (least[i] == 0.f || ms < least[i]) {
-          least[i] = ms;
-        }
-      }
-    }
-    float best_ms = 0.f;
-    for (int i = 0; i < count && i < kCandidates; ++i) {
-      if (usable[i] && least[i] > 0.f && (best_ms == 0.f || least[i] < best_ms)) {
-        best_ms = least[i];
-        best = i;
-      }
-    }
-  }
-  if (begin) hipEventDestroy(begin);
-  if (end) hipEventDestroy(end);
-  hipStreamSynchronize(stream);
-  if (flush) hipFree(flush);
-  hipFree(scratch);
-  return best;
+  *out = &handle;
+  return 0;
 }
 
 template <typename F>
@@ -160,7 +141,9 @@ extern "C" int ms_gemm_library_open(const char* path) {
                   resolve(g_api.pref_create, "hipblasLtMatmulPreferenceCreate") &&
                   resolve(g_api.pref_set, "hipblasLtMatmulPreferenceSetAttribute") &&
                   resolve(g_api.pref_destroy, "hipblasLtMatmulPreferenceDestroy") &&
-                  resolve(g_api.heuristic, "hipblasLtMatmulAlgoGetHeuristic") && resolve(g_api.matmul, "hipblasLtMatmul");
+                  resolve(g_api.heuristic, "hipblasLtMatmulAlgoGetHeuristic") && resolve(g_api.matmul, "hipblasLtMatmul") &&
+                  resolve(g_api.desc_destroy, "hipblasLtMatmulDescDestroy") &&
+                  resolve(g_api.layout_destroy, "hipblasLtMatrixLayoutDestroy");
   if (!ok) {
     g_api = Api{};
     return ms_fail("gemm_library: %s lacks a hipBLASLt entry point", path);
@@ -168,10 +151,22 @@ extern "C" int ms_gemm_library_open(const char* path) {
   return 0;
 }
 
+// Pins the solution for products against a matrix [n, k] with row counts of `bucket`
+// (ms_gemm_library_bucket) and the given output type.  Plans made before the call keep
+// what they chose, so pins are set before the first product.
+extern "C" int ms_gemm_library_pin(int n, int k, int out_float, int bucket, int solution) {
+  std::lock_guard<std::mutex> guard(g_mutex);
+  g_pinned[std::make_tuple(n, k, out_float != 0, bucket)] = solution;
+  return 0;
+}
+
+// The bucket of row counts that m falls into (a plain number, not a status).
+extern "C" int ms_gemm_library_bucket(int m) { return tune_bucket(m); }
+
 // x: bfloat16 [m, k]; w: bfloat16 [n, k]; out: [m, n], bfloat16 or (out_float) float.
 // accumulate (float output only): out += product.  workspace: device memory of
 // workspace_bytes for the library's use, the caller's for the duration of the call
-// on this stream.
+// on this stream.  The call allocates no device memory and waits for nothing.
 extern "C" int ms_gemm_library(const void* x, const void* w, void* out, int m, int n, int k, int out_float,
                                int accumulate, void* workspace, size_t workspace_bytes, hipStream_t stream) {
   MS_REQUIRE(m > 0 && n > 0 && k > 0, "gemm_library: empty shape %d x %d x %d", m, n, k);
@@ -181,69 +176,94 @@ extern "C" int ms_gemm_library(const void* x, const void* w, void* out, int m, i
   if (hipGetDevice(&device) != hipSuccess) return ms_fail("gemm_library: no current device");
 
   std::lock_guard<std::mutex> guard(g_mutex);
-  MS_REQUIRE(g_api.library != nullptr, "gemm_library: ms_gemm_library_open was not called");
-  hipblasLtHandle_t& handle = g_handles[device];
-  if (handle == nullptr && g_api.create(&handle) != HIPBLAS_STATUS_SUCCESS) {
-    g_handles.erase(device);
-    return ms_fail("gemm_library: hipblasLtCreate failed");
-  }
+  hipblasLtHandle_t* handle = nullptr;
+  if (const int failed = handle_of_current_device(&handle)) return failed;
 
   const auto key = std::make_tuple(device, m, n, k, out_float);
   auto found = g_plans.find(key);
   if (found == g_plans.end()) {
     if (g_plans.size() >= kMaxPlans) g_plans.clear();   // descriptors of shapes long gone; a few hundred bytes each
     Plan plan;
-    const hipDataType out_type = out_float ? HIP_R_32F : HIP_R_16BF;
-    const int32_t transpose = HIPBLAS_OP_T, keep = HIPBLAS_OP_N;
-    bool ok = g_api.desc_create(&plan.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && g_api.desc_set(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &transpose, sizeof(transpose)) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && g_api.desc_set(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &keep, sizeof(keep)) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && g_api.layout_create(&plan.a, HIP_R_16BF, k, n, k) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && g_api.layout_create(&plan.b, HIP_R_16BF, k, m, k) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && g_api.layout_create(&plan.c, out_type, n, m, n) == HIPBLAS_STATUS_SUCCESS;
-    MS_REQUIRE(ok, "gemm_library: cannot describe %d x %d x %d", m, n, k);
-    hipblasLtMatmulPreference_t preference = nullptr;
-    MS_REQUIRE(g_api.pref_create(&preference) == HIPBLAS_STATUS_SUCCESS, "gemm_library: no preference object");
-    const uint64_t limit = workspace_bytes;
-    g_api.pref_set(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &limit, sizeof(limit));
-    hipblasLtMatmulHeuristicResult_t result[kCandidates];
-    int returned = 0;
-    const hipblasStatus_t status =
-        g_api.heuristic(handle, plan.desc, plan.a, plan.b, plan.c, plan.c, preference, kCandidates, result, &returned);
-    g_api.pref_destroy(preference);
-    MS_REQUIRE(status == HIPBLAS_STATUS_SUCCESS && returned > 0, "gemm_library: no algorithm for %d x %d x %d", m, n, k);
-    int best = 0;
-    // The library's first choice is not always its fastest (25600 x 5120 against 8 rows:
-    // 138 us, its third candidate 58).  The candidates are timed once for a bucket of row
-    // counts, on scratch output, unless the stream is recording (no waiting there).
-    if (returned > 1) {
-      const auto bucket = std::make_tuple(device, n, k, out_float, tune_bucket(m));
-      const auto tuned = g_tuned.find(bucket);
-      hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-      if (tuned != g_tuned.end()) {
-        for (int i = 0; i < returned; ++i) {
-          if (result[i].state == HIPBLAS_STATUS_SUCCESS && result[i].workspaceSize <= workspace_bytes &&
-              solution_index(result[i].algo) == tuned->second) {
-            best = i;
-            break;
-          }
-        }
-      } else if (hipStreamIsCapturing(stream, &capture) == hipSuccess && capture == hipStreamCaptureStatusNone) {
-        best = fastest_candidate(handle, plan, result, returned, x, w, m, n, out_float, workspace, workspace_bytes, stream);
-        g_tuned[bucket] = solution_index(result[best].algo);
+    Candidates candidates;
+    if (const int failed = describe(*handle, m, n, k, out_float, workspace_bytes, plan, candidates)) return failed;
+    int best = -1;
+    const auto pinned = g_pinned.find(std::make_tuple(n, k, out_float != 0, tune_bucket(m)));
+    for (int i = 0; i < candidates.count; ++i) {
+      const auto& candidate = candidates.result[i];
+      if (candidate.state != HIPBLAS_STATUS_SUCCESS || candidate.workspaceSize > workspace_bytes) continue;
+      if (best < 0) best = i;                           // the library's first usable choice
+      if (pinned != g_pinned.end() && solution_index(candidate.algo) == pinned->second) {
+        best = i;
+        break;
       }
     }
-    plan.algo = result[best].algo;
-    plan.workspace = result[best].workspaceSize;
+    MS_REQUIRE(best >= 0, "gemm_library: no usable algorithm for %d x %d x %d", m, n, k);
+    plan.algo = candidates.result[best].algo;
+    plan.workspace = candidates.result[best].workspaceSize;
     found = g_plans.emplace(key, plan).first;
   }
   const Plan& plan = found->second;
   MS_REQUIRE(plan.workspace <= workspace_bytes, "gemm_library: the algorithm wants %zu bytes of workspace, %zu given",
              plan.workspace, workspace_bytes);
   const float alpha = 1.0f, beta = accumulate ? 1.0f : 0.0f;
-  const hipblasStatus_t status = g_api.matmul(handle, plan.desc, &alpha, w, plan.a, x, plan.b, &beta, out, plan.c, out,
+  const hipblasStatus_t status = g_api.matmul(*handle, plan.desc, &alpha, w, plan.a, x, plan.b, &beta, out, plan.c, out,
                                               plan.c, &plan.algo, workspace, workspace_bytes, stream);
   MS_REQUIRE(status == HIPBLAS_STATUS_SUCCESS, "gemm_library: hipblasLtMatmul failed with status %d for %d x %d x %d",
              static_cast<int>(status), m, n, k);
+  return 0;
+}
+
+// For the tool that measures the table of pins, never called while the engine serves:
+// times the library's candidates for x[m, k] . w[n, k]^T -> scratch_out [m, n] (memory of
+// the caller's, not the product's true output) and reports, per candidate, its solution
+// and the least of three timed runs in milliseconds (0 = not usable), each run after
+// `flush` (flush_bytes of the caller's memory, more than the caches hold, or null) has
+// been overwritten: a decode step meets every matrix in memory, not in the caches, and
+// among candidates that are timed warm the wrong one wins.  solutions and milliseconds
+// hold `capacity` entries; *count receives how many were filled.  Waits for the stream.
+extern "C" int ms_gemm_library_time(const void* x, const void* w, void* scratch_out, int m, int n, int k, int out_float,
+                                    void* workspace, size_t workspace_bytes, void* flush, size_t flush_bytes,
+                                    int* solutions, float* milliseconds, int capacity, int* count, hipStream_t stream) {
+  MS_REQUIRE(m > 0 && n > 0 && k > 0 && x && w && scratch_out && solutions && milliseconds && count && capacity > 0,
+             "gemm_library_time: bad arguments");
+  std::lock_guard<std::mutex> guard(g_mutex);
+  hipblasLtHandle_t* handle = nullptr;
+  if (const int failed = handle_of_current_device(&handle)) return failed;
+  Plan plan;
+  Candidates candidates;
+  if (const int failed = describe(*handle, m, n, k, out_float, workspace_bytes, plan, candidates)) return failed;
+  hipEvent_t begin = nullptr, end = nullptr;
+  MS_REQUIRE(hipEventCreate(&begin) == hipSuccess && hipEventCreate(&end) == hipSuccess, "gemm_library_time: no events");
+  const float alpha = 1.0f, beta = 0.0f;
+  const auto run = [&](int i) {
+    return g_api.matmul(*handle, plan.desc, &alpha, w, plan.a, x, plan.b, &beta, scratch_out, plan.c, scratch_out, plan.c,
+                        &candidates.result[i].algo, workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
+  };
+  const int filled = candidates.count < capacity ? candidates.count : capacity;
+  for (int i = 0; i < filled; ++i) {
+    solutions[i] = solution_index(candidates.result[i].algo);
+    milliseconds[i] = 0.f;
+    bool usable = candidates.result[i].state == HIPBLAS_STATUS_SUCCESS &&
+                  candidates.result[i].workspaceSize <= workspace_bytes && run(i);      // one run that is not counted
+    for (int trial = 0; usable && trial < 3; ++trial) {
+      float ms = 0.f;
+      usable = (flush == nullptr || hipMemsetAsync(flush, trial, flush_bytes, stream) == hipSuccess) &&
+               hipEventRecord(begin, stream) == hipSuccess && run(i) && hipEventRecord(end, stream) == hipSuccess &&
+               hipEventSynchronize(end) == hipSuccess && hipEventElapsedTime(&ms, begin, end) == hipSuccess;
+      if (usable && (milliseconds[i] == 0.f || ms < milliseconds[i])) milliseconds[i] = ms;
+    }
+    if (!usable) {
+      milliseconds[i] = 0.f;
+      (void)hipGetLastError();
+    }
+  }
+  *count = filled;
+  g_api.desc_destroy(plan.desc);
+  g_api.layout_destroy(plan.a);
+  g_api.layout_destroy(plan.b);
+  g_api.layout_destroy(plan.c);
+  (void)hipEventDestroy(begin);
+  (void)hipEventDestroy(end);
+  (void)hipStreamSynchronize(stream);
   return 0;
 }

@@ -256,6 +256,9 @@ class ModelRunner:
         from .. import ops
 
         ops.load()
+        if model.dtype == torch.bfloat16:
+            # the library product's binding and workspace, before the pool is sized from what is free
+            ops.prepare_products(self.device)
         self.model = model
         self.spec = model.spec
         self.engine_config = engine_config.validate(max_positions=self.spec.max_positions)

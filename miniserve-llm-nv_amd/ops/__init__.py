@@ -7,8 +7,12 @@ torch is the allocator and gives the stream.
 from __future__ import annotations
 
 import contextlib
+import ctypes
 import dataclasses
+import json
+import os
 import warnings
+from pathlib import Path
 
 import torch
 
@@ -402,6 +406,13 @@ FUSED_NORM_GATED_BYTES = 48 << 20
 _GEMM_WORKSPACE_BYTES = 64 << 20
 _gemm_workspaces: dict[int, torch.Tensor] = {}
 _gemm_library_opened = False
+# The table of pinned solutions: for a matrix [n, k], an output type and a bucket of
+# row counts, the solution of hipBLASLt that was fastest when the table was measured
+# (``python -m miniserve_amd.ops.tune``).  It holds for one build of the library, which
+# the table names; with another build, or for a shape the table lacks, the library's own
+# first choice runs.  Either way nothing is timed in a serving process, and the same
+# model gives the same 32-bit sums in every process.
+LIBRARY_PRODUCTS_TABLE = Path(__file__).resolve().parent / "library_products.json"
 
 
 def _loaded_hipblaslt() -> str:
@@ -416,21 +427,104 @@ def _loaded_hipblaslt() -> str:
     raise KernelError("no hipBLASLt is loaded in this process (torch on ROCm brings it).")
 
 
+def hipblaslt_build(path: str) -> str:
+    """What names a build of the library in the table of pins: its file's name and size."""
+
+    real = os.path.realpath(path)
+    return f"{os.path.basename(real)}:{os.path.getsize(real)}"
+
+
+def open_gemm_library() -> str:
+    """Binds the product for many rows to the process's hipBLASLt and sets the pinned
+    solutions; returns the library's path.  Done once."""
+
+    global _gemm_library_opened
+    path = _loaded_hipblaslt()
+    if not _gemm_library_opened:
+        call("ms_gemm_library_open", path.encode())
+        if LIBRARY_PRODUCTS_TABLE.is_file():
+            table = json.loads(LIBRARY_PRODUCTS_TABLE.read_text())
+            if table.get("library") == hipblaslt_build(path):
+                for n, k, out_float, bucket, solution in table.get("pins", ()):
+                    call("ms_gemm_library_pin", int(n), int(k), int(out_float), int(bucket), int(solution))
+        _gemm_library_opened = True
+    return path
+
+
+def _gemm_workspace(device: torch.device) -> torch.Tensor:
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    workspace = _gemm_workspaces.get(index)
+    if workspace is None:
+        workspace = _gemm_workspaces[index] = torch.empty(_GEMM_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    return workspace
+
+
+def prepare_products(device: torch.device | str) -> None:
+    """What the matrix products allocate and set up once per process and device (the
+    library's binding, its pins and its workspace), done now: an engine calls this before
+    it sizes its cache pool from the free memory, so that no step allocates for them."""
+
+    open_gemm_library()
+    _gemm_workspace(torch.device(device))
+
+
 def _library_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
     """``out (+)= x @ weight^T`` through hipBLASLt; bfloat16 in, bfloat16 or float32 out."""
 
-    global _gemm_library_opened
     if not _gemm_library_opened:
-        call("ms_gemm_library_open", _loaded_hipblaslt().encode())
-        _gemm_library_opened = True
-    index = x.device.index if x.device.index is not None else torch.cuda.current_device()
-    workspace = _gemm_workspaces.get(index)
-    if workspace is None:
-        workspace = _gemm_workspaces[index] = torch.empty(_GEMM_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
+        open_gemm_library()
+    workspace = _gemm_workspace(x.device)
     m, k = x.shape
     product_calls["library"] += 1
+    if _noted_library_products is not None:
+        _noted_library_products.add((m, weight.shape[0], k, int(out.dtype == torch.float32)))
     call("ms_gemm_library", _ptr(x), _ptr(weight), _ptr(out), m, weight.shape[0], k, int(out.dtype == torch.float32),
          int(accumulate), _ptr(workspace), _GEMM_WORKSPACE_BYTES, _stream())
+
+
+_noted_library_products: set | None = None
+
+
+@contextlib.contextmanager
+def noting_library_products(into: set):
+    """Inside the block every product that hipBLASLt serves adds ``(m, n, k, out is
+    float32)`` to ``into`` (for the tool that measures the table of pins)."""
+
+    global _noted_library_products
+    previous, _noted_library_products = _noted_library_products, into
+    try:
+        yield into
+    finally:
+        _noted_library_products = previous
+
+
+def time_library_product(m: int, n: int, k: int, *, out_float32: bool = False, flush: torch.Tensor | None = None,
+                         device: torch.device | str = "cuda:0") -> list[tuple[int, float]]:
+    """For the tool that measures the table of pins: (solution, milliseconds) of every
+    candidate that hipBLASLt offers for ``x [m, k] @ w [n, k]^T``, each timed from
+    flushed caches (``flush``: a tensor larger than the caches, overwritten before every
+    run); 0 ms marks a candidate that did not run."""
+
+    open_gemm_library()
+    device = torch.device(device)
+    x = torch.randn((m, k), device=device).to(torch.bfloat16)
+    w = (torch.randn((n, k), device=device) * 0.02).to(torch.bfloat16)
+    out = torch.empty((m, n), dtype=torch.float32 if out_float32 else torch.bfloat16, device=device)
+    workspace = _gemm_workspace(device)
+    capacity = 16
+    solutions = (ctypes.c_int * capacity)()
+    milliseconds = (ctypes.c_float * capacity)()
+    count = ctypes.c_int(0)
+    call("ms_gemm_library_time", _ptr(x), _ptr(w), _ptr(out), m, n, k, int(out_float32), _ptr(workspace),
+         _GEMM_WORKSPACE_BYTES, _ptr(flush), 0 if flush is None else flush.numel() * flush.element_size(),
+         solutions, milliseconds, capacity, ctypes.byref(count), _stream())
+    return [(int(solutions[i]), float(milliseconds[i])) for i in range(count.value)]
+
+
+def library_product_bucket(m: int) -> int:
+    """The bucket of row counts that shares one pinned solution."""
+
+    return int(load().ms_gemm_library_bucket(int(m)))
 
 
 # Which of the two products serves a call that both can serve is a fixed rule of the
@@ -441,8 +535,9 @@ def _library_product(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, a
 # library's product streams a small matrix faster, the more so the fewer the rows;
 # hipBLASLt, with the fastest of its candidates for the shape, streams a large one
 # faster; the fused forms (norm as prologue, activation as epilogue) save one or two
-# kernels of some 5 us each.  (Which candidate the library runs is timed once per
-# process and shape; its candidates differ in the order of their 32-bit sums only.)
+# kernels of some 5 us each.  Which of its candidates the library runs is fixed as
+# well (the table of pins above, else its first choice), so two processes that run the
+# same model on the same steps give the same bits.
 _MIB = 1 << 20
 product_calls = {"skinny": 0, "library": 0}     # calls served by each since the import
 _forced_product: str | None = None

@@ -38,6 +38,9 @@ _SIGNATURES: dict[str, list] = {
     "ms_gemm_skinny_normed": [_P, _P, _F, _P, _P, _I, _I, _I, _I, _P],
     "ms_gemm_library_open": [c_char_p],
     "ms_gemm_library": [_P, _P, _P, _I, _I, _I, _I, _I, _P, c_size_t, _P],
+    "ms_gemm_library_pin": [_I, _I, _I, _I, _I],
+    "ms_gemm_library_bucket": [_I],
+    "ms_gemm_library_time": [_P, _P, _P, _I, _I, _I, _I, _P, c_size_t, _P, c_size_t, _P, _P, _I, _P, _P],
     "ms_silu_mul": [_P, _P, _I, _I, _I, _P],
     "ms_sample_rows": [_P, _P, _P, _P, _P, _P, _I, _I, _P],
     "ms_argmax_rows": [_P, _P, _P, _P, _I, _I, _I, _P],

@@ -1,8 +1,9 @@
 """Trace replay at the layer sizes that are served, against the plain implementation:
 the widths of Qwen3-0.6B (hidden 1024, 16 query and 8 key/value heads of 128, feed-forward
-3072, 151,936 tokens, tied head) with three layers, and the widths of Qwen3-8B (hidden
-4096, 32 and 8 heads, feed-forward 12288, untied head) with one layer and a shorter,
-odd vocabulary.  Requests of 90 to 700 tokens run whole, with the last 32 tokens one
+3072, 151,936 tokens, tied head) with three layers, the widths of Qwen3-8B (hidden
+4096, 32 and 8 heads, feed-forward 12288, untied head) and those of Qwen3-32B (hidden
+5120, 64 and 8 heads: eight query heads to a key/value head, feed-forward 25600) with
+one layer each and a shorter, odd vocabulary.  Requests of 90 to 700 tokens run whole, with the last 32 tokens one
 by one, in portions of changing size, and mixed on so few pages that they are used
 again; in 32-bit and in bfloat16, the latter with each of the two matrix products
 forced in turn.  The pools are filled with NaN before every run.
@@ -16,12 +17,14 @@ from __future__ import annotations
 
 import io
 import shutil
+import subprocess
+import sys
 
 import plain_qwen3 as plain
 import pytest
 import replay_shapes as shapes
 import torch
-from helpers import make_model_folder, random_tokens, read_config, read_weights
+from helpers import ROOT, make_model_folder, random_tokens, read_config, read_weights
 
 pytestmark = pytest.mark.gpu
 
@@ -44,7 +47,17 @@ def widths_8b() -> dict:
     }
 
 
-MODELS = {"0.6b": (widths_0p6b, (100, 700, 333, 257, 512)), "8b": (widths_8b, (150, 420, 90, 260, 330))}
+def widths_32b() -> dict:
+    return {
+        "architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "hidden_size": 5120, "intermediate_size": 25600,
+        "num_hidden_layers": 1, "num_attention_heads": 64, "num_key_value_heads": 8, "head_dim": 128,
+        "vocab_size": 20011, "max_position_embeddings": 2048, "rms_norm_eps": 1e-6, "rope_theta": 1000000.0,
+        "tie_word_embeddings": False, "hidden_act": "silu", "attention_bias": False, "attention_dropout": 0.0,
+    }
+
+
+MODELS = {"0.6b": (widths_0p6b, (100, 700, 333, 257, 512)), "8b": (widths_8b, (150, 420, 90, 260, 330)),
+          "32b": (widths_32b, (130, 300, 70, 200, 150))}
 BLOCK = 16
 # portions that end on, before and after the edges of pages (16) and of the attention kernel's tiles (64)
 PORTIONS = (64, 2, 130, 17, 255, 2, 33, 1, 96, 300, 15, 49)
@@ -185,3 +198,27 @@ def test_replay_at_served_widths_in_bfloat16(name, product, sized, tmp_path):
     assert used[product] > 0
     if product == "library":
         assert used["skinny"] == 0
+
+
+def test_two_processes_give_the_same_bfloat16_logits_to_the_bit(sized, tmp_path):
+    """Which kernel and which of the library's algorithms serves a product is a fixed rule
+    of its shape: nothing is timed in a serving process.  The replay program, run twice in
+    fresh processes on the same model and steps, writes the same bits."""
+
+    folder, config, requests, wanted, _, _, _ = sized("0.6b")
+    steps = the_shapes(requests, wanted)["mixed"]
+    lines = "".join(line + "\n" for line in shapes.to_lines(steps))
+    outs = []
+    for run in range(2):
+        out = tmp_path / f"run{run}"
+        process = subprocess.run(
+            [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype", "bfloat16", "--out", str(out),
+             "--max-tokens", str(shapes.max_live_tokens(steps))],
+            input=lines, capture_output=True, text=True, timeout=600,
+        )
+        assert process.returncode == 0, process.stderr[-2000:]
+        outs.append(out)
+    files = sorted(path.name for path in outs[0].iterdir())
+    assert files and files == sorted(path.name for path in outs[1].iterdir())
+    for name in files:
+        assert (outs[0] / name).read_bytes() == (outs[1] / name).read_bytes(), f"step file {name} differs between the runs"
