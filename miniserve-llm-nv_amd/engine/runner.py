@@ -10,6 +10,8 @@ from __future__ import annotations
 
 import gc
 import weakref
+
+import numpy as np
 from dataclasses import dataclass
 from pathlib import Path
 from typing import Sequence
@@ -20,7 +22,7 @@ from ..cache import CacheLayout, CacheManager, StepItem
 from ..config import EngineConfig, load_config
 from ..parts.model import TORCH_DTYPES, DecoderModel
 from ..weights import WeightLoadReport, load_weights, random_device_tensors
-from ..parts.base import GroupStepView, StepContext
+from ..parts.base import GroupStepView, HostBatch, StepContext
 from .batch import BuiltStep, StepEntry, build_step
 
 
@@ -41,19 +43,34 @@ def recorded_batch_size(batch: int) -> int:
     return -(-batch // step) * step
 
 
+def recorded_context_bound(longest: int, limit: int) -> int:
+    """The context bound of the recorded step that serves rows of up to ``longest``
+    tokens: 256, 512, 1024, ... up to ``limit`` (the longest request the engine admits).
+    Kernels inside a recording size their launches by the bound (the parts that the keys
+    of a row are cut into, say), and the block tables have its width, so a short context
+    is not served by a step made for the longest one; a request that grows past a bound
+    moves on to the next recording."""
+
+    bound = 256
+    while bound < longest:
+        bound *= 2
+    return min(bound, limit)
+
+
 _SPARE_ROW = object()       # marks a row of a host buffer that holds the values of a spare row
 
 
 class DecodeGraph:
-    """One decode step of a fixed batch size, recorded as a HIP graph.
+    """One decode step of a fixed batch size and context bound, recorded as a HIP graph.
 
     A step in which every request brings one token launches a few hundred small
     kernels; recorded once and replayed, the launches cost next to nothing.  The
     integer metadata of the step lives in one static device buffer that every
     replay reads; a step copies its own values there (one copy from pinned host
-    memory) and replays.  Block tables have the static width of the longest
-    request the engine admits.  The graph holds no memset node: nothing in the
-    recorded step clears memory.
+    memory) and replays.  Block tables have the static width of the step's context
+    bound.  The graph holds no memset node: nothing in the recorded step clears memory.
+    Integer tables that parts ask for (``step_tables``) are made once, from what holds
+    for every replay, and lie in the same buffer.
 
     A step of fewer requests than ``batch`` fills the other rows with spare ones:
     token 0 at position 0 of a sequence whose only page is the pools' spare page and
@@ -61,15 +78,21 @@ class DecodeGraph:
     holds, and their logits are not returned.
     """
 
-    def __init__(self, runner: "ModelRunner", batch: int) -> None:
+    def __init__(self, runner: "ModelRunner", batch: int, bound: int) -> None:
         self.batch = batch
+        self.bound = bound
         # no strong reference back: a runner that is dropped goes at once, with its graphs,
         # and not at some later collection of cycles
         self._runner = weakref.ref(runner)
         groups = len(runner.cache.layout.groups)
-        widths = runner.max_blocks_per_seq          # per group: pages of the longest request the engine admits
+        widths = tuple(-(-bound // size) for size in runner.cache.block_sizes)     # per group: pages of a row at the bound
+        # the parts' own tables, from what every replay shares: one token a row
+        host_batch = HostBatch((1,) * batch, tuple(range(batch + 1)), None, batch, recorded=True)
+        part_tables = {name: np.asarray(values, dtype=np.int64)
+                       for name, values in runner.model.step_tables(host_batch).items()}
         sizes = [("token_ids", batch), ("positions", batch), ("seq_of_token", batch), ("query_start", batch + 1),
                  ("context_lens", batch), ("state_slots", batch), ("logit_rows", batch)]
+        sizes += [(f"part:{name}", values.size) for name, values in part_tables.items()]
         for group in range(groups):
             sizes += [(f"slots{group}", batch), (f"table{group}", batch * widths[group])]
         self.offsets: dict[str, tuple[int, int]] = {}
@@ -81,6 +104,10 @@ class DecodeGraph:
         # copy of this step's is still on its way
         self.hosts = [torch.zeros(total, dtype=torch.int32).pin_memory() for _ in range(2)]
         self.hosts_np = [host.numpy() for host in self.hosts]
+        for host in self.hosts_np:
+            for name, values in part_tables.items():
+                start, size = self.offsets[f"part:{name}"]
+                host[start : start + size] = values
         self._turn = 0
         self.meta = torch.zeros(total, dtype=torch.int32, device=runner.device)
         self.widths = widths
@@ -107,7 +134,8 @@ class DecodeGraph:
             first_positions_host=None,
             decode_prefix=batch,
             recorded=True,
-            context_bound=runner.max_model_len,
+            context_bound=bound,
+            tables={name: view(f"part:{name}") for name in part_tables},
         )
         self.rows = view("logit_rows")
         # the table object that each row of the host buffer was last filled from: a request's
@@ -135,6 +163,8 @@ class DecodeGraph:
         spare = batch - len(metas)
         if spare < 0:
             raise ValueError(f"{len(metas)} requests do not fit a recorded step of {batch}.")
+        if any(meta.after > self.bound for meta in metas):
+            raise ValueError(f"a request is longer than the {self.bound} tokens this recorded step was made for.")
         runner = self._runner()
         put("positions", [meta.before for meta in metas] + [0] * spare)
         put("seq_of_token", range(batch))
@@ -284,7 +314,7 @@ class ModelRunner:
         self.cache.allocate_storage(self.dtype, self.device)
         self._call_views = self.cache.call_views()
         self.max_blocks_per_seq = tuple(-(-self.max_model_len // size) for size in self.cache.block_sizes)
-        self._decode_graphs: dict[int, DecodeGraph] = {}
+        self._decode_graphs: dict[tuple[int, int], DecodeGraph] = {}     # by (rows, context bound)
         self._graph_pool = None
         self.steps_run = 0
         self.tokens_run = 0
@@ -336,6 +366,12 @@ class ModelRunner:
         blocks = max(1, min(by_memory, by_need))
         return blocks
 
+    def _recorded_step_key(self, batch: int, longest: int) -> tuple[int, int]:
+        """(rows, context bound) of the recorded step that serves ``batch`` single tokens
+        whose longest row has ``longest`` tokens after the step."""
+
+        return recorded_batch_size(batch), recorded_context_bound(longest, self.max_model_len)
+
     def _decode_graph_step(self, entries: Sequence[StepEntry], reservation, prepared: int | None = None) -> torch.Tensor | None:
         """A step of single tokens through the recorded graph of its batch size.  The
         graph computes the logits of every row; the wanted ones are picked."""
@@ -344,12 +380,12 @@ class ModelRunner:
             if entry.token_ids[0] >= self.spec.vocab_size:
                 raise ValueError(f"entry {entry.request_id!r}: a token id is outside the vocabulary.")
         batch = len(entries)
-        recorded = recorded_batch_size(batch)
-        graph = self._decode_graphs.get(recorded)
+        key = self._recorded_step_key(batch, max(meta.after for meta in reservation.sequences))
+        graph = self._decode_graphs.get(key)
         if graph is None:
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
-            graph = self._decode_graphs[recorded] = DecodeGraph(self, recorded)
+            graph = self._decode_graphs[key] = DecodeGraph(self, *key)
         logits = graph.run(entries, reservation, prepared)
         wanted = [index for index, entry in enumerate(entries) if entry.want]
         if len(wanted) == batch:
@@ -376,13 +412,13 @@ class ModelRunner:
 
         if not self.engine_config.decode_graphs or not request_ids:
             return None
-        graph = self._decode_graphs.get(recorded_batch_size(len(request_ids)))
-        if graph is None or graph.graph is None:
-            return None
         items = []
         for request_id in request_ids:
             start = self.cache.committed_tokens(request_id)
             items.append(StepItem(request_id, start, start + 1))
+        graph = self._decode_graphs.get(self._recorded_step_key(len(items), max(item.end for item in items)))
+        if graph is None or graph.graph is None:
+            return None
         reservation = self.cache.prepare_step(items)
         try:
             buffer = graph.prepare(reservation)

@@ -113,12 +113,16 @@ class GroupStepView:
 @dataclass(frozen=True)
 class HostBatch:
     """What a part may know of a step on the host, before anything is sent: the
-    sequences in the order of the batch (those that bring one token first)."""
+    sequences in the order of the batch (those that bring one token first).
+    ``recorded``: the batch stands for every replay of a recorded step of single
+    tokens; then the positions are not known (``first_positions`` is None) and the
+    tables made from it are made once."""
 
     query_lens: tuple[int, ...]         # tokens that each sequence brings
     query_start: tuple[int, ...]        # index of each sequence's first token in the batch, and the total
-    first_positions: tuple[int, ...]    # absolute position of each sequence's first token
+    first_positions: tuple[int, ...] | None    # absolute position of each sequence's first token
     decode_prefix: int                  # sequences at the front that bring exactly one token
+    recorded: bool = False
 
 
 @dataclass

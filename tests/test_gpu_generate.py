@@ -325,7 +325,7 @@ def test_decode_graphs_replay_like_eager_steps(dtype, model_folders):
         both({"a": 1, "b": 1, "c": 1, "d": 1})     # crosses page edges of 16
     both({"b": 1})
     assert runners[0].graph_steps == 33 and runners[1].graph_steps == 0
-    assert sorted(runners[0]._decode_graphs) == [1, 2, 4]           # three requests ran in the step of four
+    assert sorted(runners[0]._decode_graphs) == [(1, 256), (2, 256), (4, 256)]    # three requests ran in the step of four
 
 
 def test_steps_planned_ahead_on_the_device_change_no_token(model_folders):
@@ -439,7 +439,7 @@ def test_recorded_steps_filled_up_with_spare_rows(dtype, live, recorded, model_f
         runner.release("r0")
     for _ in range(10):
         both({name: 1 for name in names if name not in ("r0", "r4")})    # nine live, across page edges of 8
-    assert sorted(runners[0]._decode_graphs) == recorded and runners[0].graph_steps == 23
+    assert sorted(runners[0]._decode_graphs) == [(rows, 256) for rows in recorded] and runners[0].graph_steps == 23
     cache = runners[0].cache
     assert all(cache.spare_page(0) not in cache.block_table(name) for name in cache.live_requests())
 
@@ -472,7 +472,7 @@ def test_a_dropped_runner_is_freed_at_once_and_recording_survives_a_collection(m
     expected = decode_once(first)
     assert first.graph_steps == 1
     gone = weakref.ref(first)
-    graph_gone = weakref.ref(first._decode_graphs[1])
+    graph_gone = weakref.ref(first._decode_graphs[(1, 256)])
     del first
     assert gone() is None and graph_gone() is None
 

@@ -418,7 +418,7 @@ def test_state_in_recorded_steps(toy):
             runner.release(rid)
             live.remove(rid)
         steps += 1
-    assert runner.graph_steps == steps and sorted(runner._decode_graphs) == [1, 2, 4]      # three, two, one request
+    assert runner.graph_steps == steps and sorted(runner._decode_graphs) == [(1, 256), (2, 256), (4, 256)]      # three, two, one request
 
 
 def test_an_aborted_step_puts_the_state_back(toy):

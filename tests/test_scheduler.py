@@ -535,3 +535,11 @@ def test_cancel_gives_everything_back():
     engine.cancel("a")
     assert runner.cache.capacity().free_blocks == (64,) and not engine.has_unfinished()
     assert engine.pop_result("a").finish_reason == "cancelled"
+
+
+def test_recorded_context_bounds():
+    from miniserve_amd.engine.runner import recorded_context_bound
+
+    assert [recorded_context_bound(n, 40960) for n in (1, 100, 256, 257, 2049, 4096, 33000, 40960)] == [
+        256, 256, 256, 512, 4096, 4096, 40960, 40960]
+    assert recorded_context_bound(100, 128) == 128
