@@ -120,7 +120,10 @@ def parity_run(sizes, layers, device, prompt_len=300, tail=32):
 
     import torch
 
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    tests = os.path.join(ROOT, "tests")
+    if not os.path.isfile(os.path.join(tests, "plain_qwen3.py")):
+        raise SystemExit(f"--parity compares with the plain implementation in {tests}/plain_qwen3.py, which this checkout lacks.")
+    sys.path.insert(0, tests)
     import plain_qwen3
 
     from miniserve_amd.config import EngineConfig, config_from_dict

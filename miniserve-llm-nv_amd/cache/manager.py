@@ -151,16 +151,19 @@ class CacheManager:
         self._next_step_id = 0
         self._open: StepReservation | None = None
         # storage, attached by allocate_storage()
-        self.key_pools: list = []
+        self.pools: list[dict] = []        # per group: plane name -> [calls, pages + 1, *plane shape]
+        self.key_pools: list = []          # the "key" and "value" planes of the groups that have them
         self.value_pools: list = []
         self.state_tensors: list = []
 
     # ---- storage --------------------------------------------------------------------
     def allocate_storage(self, dtype, device) -> None:
-        """Per group a key pool ``[calls, pages + 1, kv_heads, block_size, head_dim]`` and a
-        value pool ``[calls, pages + 1, kv_heads, head_dim, block_size]`` (values lie
+        """Per group one pool for every plane that the group's need names,
+        ``[calls, pages + 1, *plane shape]``; with the default planes a key pool
+        ``[calls, pages + 1, kv_heads, block_size, head_dim]`` and a value pool
+        ``[calls, pages + 1, kv_heads, head_dim, block_size]`` (values lie
         transposed inside a page: the matrix-core kernels read 4 consecutive keys
-        of one column in one load), allocated once and never initialised (a page's content is read only below the
+        of one column in one load).  Allocated once and never initialised (a page's content is read only below the
         committed length; reference: miniserve/kv/paged.py:39-41), and zeroed
         state tensors ``[slots + 1, *shape]``.  The last page of a pool and the last
         state slot are spare: no request ever holds them, and rows that only fill a
@@ -169,13 +172,24 @@ class CacheManager:
 
         import torch
 
-        self.key_pools, self.value_pools, self.state_tensors = [], [], []
+        self.pools, self.key_pools, self.value_pools, self.state_tensors = [], [], [], []
         for group, count, page in zip(self.layout.groups, self.num_blocks, self.block_sizes):
-            heads, dim = group.need.num_kv_heads, group.need.head_dim
-            self.key_pools.append(torch.empty((len(group.calls), count + 1, heads, page, dim), dtype=dtype, device=device))
-            self.value_pools.append(torch.empty((len(group.calls), count + 1, heads, dim, page), dtype=dtype, device=device))
+            made = {
+                plane.name: torch.empty((len(group.calls), count + 1, *plane.shape(page)), dtype=dtype, device=device)
+                for plane in group.need.page_planes()
+            }
+            self.pools.append(made)
+            if "key" in made:
+                self.key_pools.append(made["key"])
+            if "value" in made:
+                self.value_pools.append(made["value"])
         for need in self.layout.states:
             self.state_tensors.append(torch.zeros((self.max_num_seqs + 1, *need.shape), dtype=need.dtype, device=device))
+
+    def page_pools(self) -> list:
+        """Every page pool of every group (tests poison them before a run)."""
+
+        return [pool for made in self.pools for pool in made.values()]
 
     def spare_page(self, group: int) -> int:
         """The page of ``group``'s pools that belongs to no request."""
@@ -189,25 +203,27 @@ class CacheManager:
         return self.max_num_seqs
 
     def call_views(self) -> list:
-        """The cache of every call of the run order: ``KVCacheView``, ``StateView`` or None."""
+        """The cache of every call of the run order: ``KVCacheView``, ``StateView``, None,
+        or a tuple of them for a call with several needs."""
 
-        views = []
-        for placement in self.layout.placements:
+        def view(placement):
             if placement.kind == "kv":
-                views.append(
-                    KVCacheView(
-                        group=placement.group,
-                        key=self.key_pools[placement.group][placement.index],
-                        value=self.value_pools[placement.group][placement.index],
-                        block_size=self.block_sizes[placement.group],
-                        write=placement.write,
-                    )
+                planes = {name: pool[placement.index] for name, pool in self.pools[placement.group].items()}
+                return KVCacheView(
+                    group=placement.group,
+                    key=planes.get("key"),
+                    value=planes.get("value"),
+                    block_size=self.block_sizes[placement.group],
+                    write=placement.write,
+                    planes=planes,
                 )
-            elif placement.kind == "state":
-                views.append(StateView(self.state_tensors[placement.index]))
-            else:
-                views.append(None)
-        return views
+            if placement.kind == "state":
+                return StateView(self.state_tensors[placement.index])
+            if placement.kind == "many":
+                return tuple(view(part) for part in placement.parts)
+            return None
+
+        return [view(placement) for placement in self.layout.placements]
 
     # ---- admission and release --------------------------------------------------------
     def admit(self, request_id: str) -> int:

@@ -6,8 +6,11 @@
 // csrc/rmsnorm.cu:92-105).  In 32-bit storage the rounding is the identity.
 //
 // One workgroup per output row.  The number of threads and the kernel variant
-// depend on the row length only, so a row's result never depends on the rest of
-// the batch.
+// depend on the row length and the input type only, so a row's result never depends
+// on the rest of the batch nor on where its operands lie.  (The variant for the 32-bit
+// residual stream in rows of a multiple of four reads 16 bytes at a time; operands
+// that are not 16-byte aligned are refused there rather than served by another variant
+// whose sums have another order.)
 #include <type_traits>
 
 #include "common.hpp"
@@ -158,6 +161,9 @@ __global__ void rmsnorm_by_fours_kernel(float* __restrict__ x, const T* __restri
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Whether a row of `dim` 32-bit values goes four values a thread and access.
+bool by_fours(int dim) { return dim % 4 == 0 && dim >= 256 && dim <= 16384; }
+
 template <typename TIn, typename T>
 void launch_rmsnorm(void* x, const void* delta, const void* weight, void* out, const void* rows, int n_out, int dim,
                     float eps, int write_back, hipStream_t stream) {
@@ -168,9 +174,8 @@ void launch_rmsnorm(void* x, const void* delta, const void* weight, void* out, c
   T* op = static_cast<T*>(out);
   const int32_t* rp = static_cast<const int32_t*>(rows);
   if constexpr (std::is_same<TIn, float>::value) {
-    // (the choice goes by the row's length and the operands' alignment, never by the number of rows)
-    if (dim % 4 == 0 && dim >= 256 && dim <= 16384 && aligned16(x) && aligned16(delta) && aligned16(weight) &&
-        aligned16(out)) {
+    // (the choice goes by the row's length, never by the number of rows; the entry point has checked the alignment)
+    if (by_fours(dim)) {
       const dim3 block(256);
 #define MS_NORM_BY_FOURS(VPT)                                                                                     \
   hipLaunchKernelGGL((rmsnorm_by_fours_kernel<T, VPT>), grid, block, 0, stream, xp, dp, wp, op, rp, dim, eps, write_back)
@@ -210,6 +215,11 @@ extern "C" int ms_rmsnorm(void* x, const void* delta, const void* weight, void* 
   MS_REQUIRE(eps > 0.f, "rmsnorm: eps must be positive");
   MS_REQUIRE(!(write_back && rows), "rmsnorm: write_back with gathered rows is not defined");
   MS_REQUIRE(!(write_back && !delta), "rmsnorm: write_back needs a delta");
+  if (x_is_f32 || dtype == MS_F32) {
+    MS_REQUIRE(!by_fours(dim) || (aligned16(x) && aligned16(delta) && aligned16(weight) && aligned16(out)),
+               "rmsnorm: 32-bit rows of %d values are read 16 bytes at a time; x, delta, weight and out must be "
+               "16-byte aligned (a view that starts inside a row is not)", dim);
+  }
   if (dtype == MS_F32) {
     launch_rmsnorm<float, float>(x, delta, weight, out, rows, n_out, dim, eps, write_back, stream);
   } else if (dtype == MS_BF16) {

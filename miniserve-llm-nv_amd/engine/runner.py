@@ -21,7 +21,7 @@ import torch
 from ..cache import CacheLayout, CacheManager, StepItem
 from ..config import EngineConfig, load_config
 from ..parts.model import TORCH_DTYPES, DecoderModel
-from ..weights import WeightLoadReport, load_weights, random_device_tensors
+from ..weights import WeightLoadReport, load_weights, random_model_tensors
 from ..parts.base import GroupStepView, HostBatch, StepContext
 from .batch import BuiltStep, StepEntry, build_step
 
@@ -343,11 +343,12 @@ class ModelRunner:
     def from_random(
         cls, config, engine_config: EngineConfig, *, seed: int = 0, device: torch.device | str = "cuda:0"
     ) -> "ModelRunner":
-        """Random weights drawn on the device (for sizes that should not pass through a file)."""
+        """Random weights from ``seed``: a small model gets the values that
+        ``write_random_model`` writes for the seed, a large one is drawn on the device."""
 
         _require_gpu(torch.device(device))
         model = DecoderModel(config.model_spec(), engine_config.dtype)
-        tensors = random_device_tensors(model.weight_specs(), seed=seed, dtype=model.dtype, device=device)
+        tensors = random_model_tensors(model.weight_specs(), seed=seed, dtype=model.dtype, device=device)
         runner = cls(model, tensors, engine_config, device=device)
         runner.config = config
         runner.load_report = WeightLoadReport(model_dir="<random>")

@@ -50,14 +50,14 @@ class LLM:
         if isinstance(model, (str, os.PathLike)):
             self.runner = ModelRunner.from_folder(model, self.engine_config, device=device)
         else:
-            # a configuration object: random weights, drawn on the device from ``seed``
+            # a configuration object: random weights from ``seed`` (the model that ``write_random_model``
+            # writes for it, unless it is so large that it is drawn on the device)
             self.runner = ModelRunner.from_random(model, self.engine_config, seed=seed, device=device)
         self.engine = Engine(self.runner)
 
     @classmethod
     def from_random(cls, config, *, seed: int = 0, layers: int | None = None, **options) -> "LLM":
-        """An engine over random weights, drawn on the device: for sizes that should
-        not pass through a file.  ``config`` is a configuration object of a
+        """An engine over random weights without a file.  ``config`` is a configuration object of a
         registered architecture, the name of a preset (``"qwen3-0.6b"``) or the path
         of a ``config.json``; ``layers`` replaces the number of layers of a preset or
         file.  ``options`` as for the constructor."""

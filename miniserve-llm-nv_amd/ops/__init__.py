@@ -727,12 +727,6 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
 SAMPLE_CHUNKED_FROM = 8192
 
 
-def _sample_row_table_bytes(vocab: int) -> int:
-    """Bytes a row that the stages of the chunked choice share (csrc/sampling.hip: row_table_floats)."""
-
-    return 4 * (32 * (2 + 10 + 10 + 1) + 2 + 32 + 2 * 4 * (256 + 3) + 2 * vocab)
-
-
 def sample_rows(
     logits: torch.Tensor,
     *,
@@ -774,7 +768,7 @@ def sample_rows(
     if temperature is not None and vocab >= SAMPLE_CHUNKED_FROM and rows <= 65535:
         # a long row: its passes are shared by many workgroups; between the stages small tables and room for
         # the list of the tokens that can stay
-        workspace = torch.empty(rows * _sample_row_table_bytes(vocab), dtype=torch.uint8, device=logits.device)
+        workspace = torch.empty(int(load().ms_sample_rows_workspace_bytes(rows, vocab)), dtype=torch.uint8, device=logits.device)
         call("ms_sample_rows_chunked", _ptr(logits), _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
              _ptr(out), _ptr(workspace), workspace.numel(), rows, vocab, int(bool(top_p_alone) and top_p is not None), _stream())
         return out

@@ -11,15 +11,19 @@ Categories and what each must offer:
                       ``residual + delta``; the sum is stored into the 32-bit
                       ``residual`` when ``write_back``.
 ``position``          ``apply(x [N, heads, dim], positions [N]) -> x'``; no weights.
-``mixer``             ``cache_need() -> KVCacheNeed | StateNeed | None`` and
+``mixer``             ``cache_need() -> KVCacheNeed | StateNeed | None`` (or a tuple of
+                      needs: pages and a state row, say) and
                       ``forward(x [N, H], ctx: StepContext, cache) -> [N, H]``,
-                      ``cache`` being a ``KVCacheView``, a ``StateView`` or None.
+                      ``cache`` being a ``KVCacheView``, a ``StateView``, None, or a
+                      tuple of views in the order of the needs.
 ``feed_forward``      ``forward(x [N, H], ctx) -> [N, H]``.
 ``block``             the arrangement of one layer's parts around the residual
                       stream: ``forward(residual, delta, ctx, cache) ->
                       (residual, delta)``; the sum ``residual + delta`` is what
                       the next block (or the final norm) starts from.
-``embedding``         ``forward(token_ids [N]) -> float32 [N, H]``.
+``embedding``         ``forward(token_ids [N], ctx) -> float32 [N, H]`` (``ctx``: the
+                      step's ``StepContext``, for an embedding that adds a term of
+                      the position or of another per-token input).
 ``head``              ``forward(x [R, H]) -> float32 logits [R, V]``.
 """
 
@@ -60,17 +64,54 @@ class WeightSpec:
 
 # ---- what a mixer says about its cache -------------------------------------------
 
+PAGE_TOKENS = "tokens"      # in a plane's dims: the number of tokens a page holds
+
+
+@dataclass(frozen=True)
+class PagePlane:
+    """One tensor that a mixer keeps per page: ``dims`` is the shape of one page's
+    share, with ``PAGE_TOKENS`` where the page's tokens go (``("tokens", 48)``: a vector
+    of 48 a token; ``(heads, dim, "tokens")``: tokens innermost)."""
+
+    name: str
+    dims: tuple
+
+    def shape(self, block_size: int) -> tuple[int, ...]:
+        if sum(1 for dim in self.dims if dim == PAGE_TOKENS) != 1:
+            raise ValueError(f"plane {self.name!r}: its dims must name the page's tokens exactly once.")
+        return tuple(block_size if dim == PAGE_TOKENS else int(dim) for dim in self.dims)
+
+    def elements_per_token(self) -> int:
+        count = 1
+        for dim in self.dims:
+            count *= 1 if dim == PAGE_TOKENS else int(dim)
+        return count
+
+
 @dataclass(frozen=True)
 class KVCacheNeed:
-    """Keys and values in pages.  ``window`` None: all keys are kept; an int: only
-    the last ``window`` keys of a position are ever read, older pages go back.
-    ``block_size``: tokens a page of this mixer's group holds; None = the engine's
-    ``kv_block_size`` (a mixer with a short window may want smaller pages)."""
+    """What a mixer keeps per token, in pages.  ``window`` None: all tokens are kept; an
+    int: only the last ``window`` tokens of a position are ever read, older pages go
+    back.  ``block_size``: tokens a page of this mixer's group holds; None = the
+    engine's ``kv_block_size`` (a mixer with a short window may want smaller pages).
+    ``planes``: the tensors of a page, named by the mixer; None = keys ``[kv_heads,
+    tokens, head_dim]`` and values ``[kv_heads, head_dim, tokens]``, what the attention
+    kernels of this package read.  A mixer with planes of its own (one latent vector a
+    token, keys only) finds them by name in its ``KVCacheView.planes``."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
     block_size: int | None = None
+    planes: tuple[PagePlane, ...] | None = None
+
+    def page_planes(self) -> tuple[PagePlane, ...]:
+        if self.planes is not None:
+            if not self.planes or len({plane.name for plane in self.planes}) != len(self.planes):
+                raise ValueError("a cache need names at least one plane, each once.")
+            return self.planes
+        return (PagePlane("key", (self.num_kv_heads, PAGE_TOKENS, self.head_dim)),
+                PagePlane("value", (self.num_kv_heads, self.head_dim, PAGE_TOKENS)))
 
 
 @dataclass(frozen=True)
@@ -84,13 +125,21 @@ class StateNeed:
 @dataclass
 class KVCacheView:
     """One call's slice of its group's pools: keys ``[pages, kv_heads, block_size,
-    head_dim]``, values ``[pages, kv_heads, head_dim, block_size]``."""
+    head_dim]``, values ``[pages, kv_heads, head_dim, block_size]``; for a need with
+    planes of its own ``key`` and ``value`` are None and ``planes`` holds each plane's
+    ``[pages, *dims]`` under its name (the default planes are there too, as "key" and
+    "value")."""
 
     group: int
-    key: torch.Tensor
-    value: torch.Tensor
+    key: torch.Tensor | None
+    value: torch.Tensor | None
     block_size: int
     write: bool = True     # False: this call reads another call's cache
+    planes: dict[str, torch.Tensor] = field(default_factory=dict)
+
+    def __post_init__(self) -> None:
+        if not self.planes:
+            self.planes = {name: tensor for name, tensor in (("key", self.key), ("value", self.value)) if tensor is not None}
 
 
 @dataclass

@@ -27,7 +27,10 @@ class TokenEmbedding(Part):
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.weight = tensors[self.weight_name]
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, token_ids: torch.Tensor, ctx=None) -> torch.Tensor:
+        """``ctx``: the step's context, which every embedding part is handed (one that
+        adds a term of the position reads it there); this one needs the ids alone."""
+
         return ops.embedding_gather(token_ids, self.weight)
 
 

@@ -30,7 +30,7 @@ class CallCacheNeed:
     """What entry ``call`` of the run order needs of the cache manager."""
 
     call: int
-    need: KVCacheNeed | StateNeed | None
+    need: KVCacheNeed | StateNeed | None | tuple     # a tuple: several needs at once (pages and a state row)
     cache_from: int | None
 
 
@@ -114,7 +114,7 @@ class DecoderModel:
         tokens), or None when no row is wanted; the final norm and the head run
         on those rows alone."""
 
-        residual = self.embedding.forward(ctx.token_ids)
+        residual = self.embedding.forward(ctx.token_ids, ctx)
         delta = None
         for index, call in enumerate(self.order):
             residual, delta = self.layers[call.layer].forward(residual, delta, ctx, caches[index])

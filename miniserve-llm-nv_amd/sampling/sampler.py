@@ -100,7 +100,8 @@ class Sampler:
             numbers[2] = uniforms
             numbers[3].view(np.int32)[:] = [p.top_k for _, p in requests]
             sent = host.to(logits.device, non_blocking=True)
-            alone = any(p.temperature > 0 and p.top_p < 1 and p.top_k == 0 for _, p in requests)
+            # (a top-k of the whole vocabulary cuts nothing: the kernel treats it as off)
+            alone = any(p.temperature > 0 and p.top_p < 1 and (p.top_k == 0 or p.top_k >= vocab) for _, p in requests)
             tokens = ops.sample_rows(
                 logits, temperature=sent[0], top_p=sent[1], uniform=sent[2], top_k=sent[3].view(torch.int32),
                 top_p_alone=alone,

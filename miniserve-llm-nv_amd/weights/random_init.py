@@ -84,6 +84,31 @@ def write_random_model(config, folder: str | Path, *, seed: int, store_dtype: st
     return folder
 
 
+# Up to this many float32 bytes a random model is drawn by the CPU generator, so that a
+# seed names the model that ``write_random_model`` writes; larger ones are drawn on the device.
+HOST_DRAW_BYTES = 1 << 30
+
+
+def random_model_tensors(
+    specs: Sequence[WeightSpec], *, seed: int, dtype: torch.dtype, device: torch.device | str
+) -> dict[str, torch.Tensor]:
+    """Random weights on ``device`` in the engine's types.  A model of up to
+    ``HOST_DRAW_BYTES`` is drawn by :func:`random_tensors` (the CPU generator: the same
+    values as a folder written by :func:`write_random_model` with this seed holds); a
+    larger one by :func:`random_device_tensors`, whose values differ."""
+
+    drawn = [spec for spec in specs if spec.same_as is None]
+    size = sum(4 * int(torch.Size(spec.shape).numel()) for spec in drawn)
+    if size > HOST_DRAW_BYTES:
+        return random_device_tensors(specs, seed=seed, dtype=dtype, device=device)
+    tensors = {}
+    for spec, (name, tensor) in zip(drawn, random_tensors(specs, seed).items()):
+        if tensor.is_floating_point() and spec.keep == "compute":
+            tensor = tensor.to(dtype)
+        tensors[name] = tensor.to(device)
+    return tensors
+
+
 def random_device_tensors(
     specs: Sequence[WeightSpec], *, seed: int, dtype: torch.dtype, device: torch.device | str
 ) -> dict[str, torch.Tensor]:

@@ -34,6 +34,22 @@ def filter_top_p(logits: torch.Tensor, top_p: float) -> torch.Tensor:
     return torch.empty_like(sorted_logits).scatter(-1, sorted_indices, sorted_logits)
 
 
+def running_sums(logits: torch.Tensor, temperature: float, top_k: int, top_p: float) -> torch.Tensor:
+    """The running probability sums (float64, token order) that the draw is made from."""
+
+    filtered = logits.to(torch.float32) / temperature
+    filtered = filter_top_p(filter_top_k(filtered, top_k), top_p)
+    return torch.cumsum(torch.softmax(filtered.to(torch.float64), dim=-1), dim=-1)
+
+
+def edge_distance(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, uniform: float) -> float:
+    """How close ``uniform`` lies to an edge between two tokens' shares: a draw closer
+    than an implementation's rounding of its sums may fall to either neighbour."""
+
+    running = running_sums(logits, temperature, top_k, top_p)
+    return float((running / running[-1] - uniform).abs().min())
+
+
 def sample_row(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, uniform: float) -> int:
     """temperature == 0: argmax.  Else temperature, top-k, top-p, softmax
     (reference: sampling.py:69-79), then the first index whose running
