@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--size 0.6B|8B|32B] [--parity]
+                    [--also-sizes 8B,32B|none]
 
 A "step" is one decode step of the engine loop (schedule, the step function over
 the paged cache, sampling) with ``--batch`` live requests, each after a prompt of
@@ -21,7 +22,8 @@ budget of 2,048 tokens a step, through the scheduler; all tokens over the wall t
 and by device events per step the share of steps that only decode (as a fraction
 of the HBM peak) and of steps that run prompt portions (as a fraction of the MFMA
 peak).  ``measured``: what the card reaches on a plain device copy and a large
-library product.  ``--parity`` adds a 32-bit run of the same layer sizes (two layers
+library product.  ``sizes``: with the default size, the same decode points and prefill at
+the layer sizes of Qwen3-8B and Qwen3-32B (all their layers), and for 32B the mixed run.  ``--parity`` adds a 32-bit run of the same layer sizes (two layers
 unless ``--layers`` says otherwise) against the plain float64 implementation of
 ``tests/plain_qwen3.py``: a prompt whole, then 32 tokens one by one.
 
@@ -63,6 +65,10 @@ def parse_args():
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points and the mixed run")
+    parser.add_argument("--no-mixed", action="store_true", help="skip the mixed run")
+    parser.add_argument("--also-sizes", default="8B,32B",
+                        help="with the default size: the sizes whose decode, prefill (and, for 32B, mixed) numbers are "
+                             "added under \"sizes\" ('none': the headline alone)")
     parser.add_argument("--mixed-requests", type=int, default=64, help="requests of the mixed continuous-batching run")
     parser.add_argument("--mixed-new-tokens", type=int, default=128, help="tokens each of them generates")
     parser.add_argument("--eager", action="store_true", help="no HIP graphs for decode steps")
@@ -228,14 +234,9 @@ def account_trace(path: str) -> None:
         table(mixed[len(mixed) // 2:], "step with prompt portions beside decode tokens")
 
 
-def main() -> int:
-    args = parse_args()
-    if args.account_trace:
-        account_trace(args.account_trace)
-        return 0
-    if args.gpus != 1:
-        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine does not span GPUs).")
-        return 2
+def measure(args, *, with_measured: bool = True) -> dict:
+    """Everything the line holds for the layer sizes ``args.size``."""
+
     import torch
 
     from miniserve_amd.config import EngineConfig, config_dict_from_preset_or_file, config_from_dict
@@ -430,15 +431,17 @@ def main() -> int:
         torch.cuda.synchronize()
         return (time.perf_counter() - begin) / repeats
 
-    source = torch.empty(1 << 30, dtype=torch.uint8, device=device)
-    target = torch.empty_like(source)
-    copy_gbps = 2 * source.numel() / rate(lambda: target.copy_(source)) / 1e9       # bytes read and written
-    del source, target
-    a = torch.randn(8192, 8192, device=device, dtype=torch.bfloat16)
-    b = torch.randn(8192, 8192, device=device, dtype=torch.bfloat16)
-    gemm_tflops = 2 * 8192**3 / rate(lambda: ops.linear(a, b)) / 1e12
-    del a, b
-    torch.cuda.empty_cache()
+    copy_gbps = gemm_tflops = None
+    if with_measured:
+        source = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+        target = torch.empty_like(source)
+        copy_gbps = 2 * source.numel() / rate(lambda: target.copy_(source)) / 1e9       # bytes read and written
+        del source, target
+        a = torch.randn(8192, 8192, device=device, dtype=torch.bfloat16)
+        b = torch.randn(8192, 8192, device=device, dtype=torch.bfloat16)
+        gemm_tflops = 2 * 8192**3 / rate(lambda: ops.linear(a, b)) / 1e12
+        del a, b
+        torch.cuda.empty_cache()
 
     points, points_frac = {}, {}
     if not args.no_points:
@@ -448,7 +451,7 @@ def main() -> int:
             point_bytes = step_bytes_of(batch, point_context, model_bytes, kv_bytes_per_token)
             points_frac[f"decode_b{batch}"] = round(point_bytes / (point_ms / 1000) / 1e9 / HBM_GBPS, 4)
     mixed = None
-    if not args.no_points:
+    if not args.no_points and not args.no_mixed:
         mixed = mixed_rate(args.mixed_requests, args.mixed_new_tokens)
 
     line = {
@@ -490,7 +493,6 @@ def main() -> int:
             "ms": round(1000 * prefill_s, 3),
             "samples_ms": [round(sample, 3) for sample in prefill_samples],
             "frac": round(flops / prefill_s / (PEAK_TFLOPS[args.dtype] * 1e12), 5),
-            "frac_of_measured_gemm": round(flops / prefill_s / (gemm_tflops * 1e12), 5),
         },
         "roofline": {
             "bound": "hbm",
@@ -498,15 +500,58 @@ def main() -> int:
             "peak": HBM_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_GBPS, 5),
-            "frac_of_measured_copy": round(achieved / copy_gbps, 5),
         },
         "points": points,
         "points_frac": points_frac,
         "mixed": mixed,
-        "measured": {"copy_GBps": round(copy_gbps, 1), "library_gemm_8192_TFLOPs": round(gemm_tflops, 1)},
     }
+    if with_measured:
+        line["prefill"]["frac_of_measured_gemm"] = round(flops / prefill_s / (gemm_tflops * 1e12), 5)
+        line["roofline"]["frac_of_measured_copy"] = round(achieved / copy_gbps, 5)
+        line["measured"] = {"copy_GBps": round(copy_gbps, 1), "library_gemm_8192_TFLOPs": round(gemm_tflops, 1)}
     if args.parity:
         line["parity"] = parity_run(sizes, args.layers if args.layers is not None else 2, device)
+    return line
+
+
+def summary_of(line: dict) -> dict:
+    """What the line of another size adds to the headline's: decode at batch 1, 8 and 64 with the fractions of
+    the HBM peak, the prefill with its fraction of the MFMA peak, the mixed run, and how many layers ran."""
+
+    batch = line["config"]["global_batch"]
+    short = {
+        "layers": line["config"]["layers"], "layers_of_model": line["config"]["layers_of_model"],
+        "decode": {f"decode_b{batch}": line["value"], **line["points"]},
+        "decode_frac_hbm": {f"decode_b{batch}": line["roofline"]["frac"], **line["points_frac"]},
+        "ms_per_step": line["ms_per_step"],
+        "prefill": {key: line["prefill"][key] for key in ("value", "tokens", "ms", "frac")},
+    }
+    if line.get("mixed"):
+        short["mixed"] = {key: line["mixed"][key] for key in ("value", "requests", "steps", "ms", "preemptions", "phases")}
+    return short
+
+
+def main() -> int:
+    args = parse_args()
+    if args.account_trace:
+        account_trace(args.account_trace)
+        return 0
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine does not span GPUs).")
+        return 2
+    line = measure(args)
+    others = [size for size in args.also_sizes.split(",") if size and size != "none"]
+    if others and (args.no_points or args.size != "0.6B"):
+        others = []             # the other sizes go with the default run only
+    for size in others:
+        if size not in SIZES:
+            raise SystemExit(f"--also-sizes knows {', '.join(SIZES)}; not {size!r}.")
+        print(f"[bench] Qwen3-{size} sizes ...", file=sys.stderr, flush=True)
+        other = argparse.Namespace(**vars(args))
+        other.size, other.layers, other.parity = size, None, False
+        other.steps, other.warmup = min(args.steps, 24), min(args.warmup, 4)
+        other.no_mixed = size != "32B"          # the mixed continuous batch is the 32B sizes' configuration
+        line.setdefault("sizes", {})[size] = summary_of(measure(other, with_measured=False))
     print(json.dumps(line))
     return 0
 
