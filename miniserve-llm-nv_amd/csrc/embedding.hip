@@ -6,9 +6,14 @@ namespace {
 
 template <typename T>
 __global__ void embedding_gather_kernel(const int32_t* __restrict__ token_ids, const T* __restrict__ table,
-                                        float* __restrict__ out, int hidden) {
+                                        float* __restrict__ out, int hidden, int vocab) {
   const int64_t token = blockIdx.x;
-  const T* row = table + static_cast<int64_t>(token_ids[token]) * hidden;
+  // Ids that come from the host are checked there.  An id may also come straight from the
+  // sampling kernel of the step before (a step launched before the host has read its
+  // tokens), which gives -1 for a row of logits that are not finite: such a step is thrown
+  // away by the host afterwards, and until then it must read inside the table.
+  const int id = min(max(token_ids[token], 0), vocab - 1);
+  const T* row = table + static_cast<int64_t>(id) * hidden;
   float* dst = out + token * hidden;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = ms::to_float(row[i]);
 }
@@ -22,11 +27,11 @@ extern "C" int ms_embedding_gather(const void* token_ids, const void* table, voi
   const dim3 grid(num_tokens);
   if (dtype == MS_F32) {
     hipLaunchKernelGGL((embedding_gather_kernel<float>), dim3(grid), dim3(threads), 0, stream, 
-        static_cast<const int32_t*>(token_ids), static_cast<const float*>(table), static_cast<float*>(out), hidden);
+        static_cast<const int32_t*>(token_ids), static_cast<const float*>(table), static_cast<float*>(out), hidden, vocab);
   } else if (dtype == MS_BF16) {
     hipLaunchKernelGGL((embedding_gather_kernel<ms::bf16>), dim3(grid), dim3(threads), 0, stream, 
         static_cast<const int32_t*>(token_ids), static_cast<const ms::bf16*>(table), static_cast<float*>(out),
-        hidden);
+        hidden, vocab);
   } else {
     return ms_fail("embedding_gather: unknown dtype code %d", dtype);
   }

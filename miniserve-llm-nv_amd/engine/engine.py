@@ -198,6 +198,7 @@ class Engine:
                     launched = self.sampler.launch(logits, requests)
                     # while the GPU runs the step: the next one, if it can be foreseen
                     next_ahead = self._prepare_step_ahead(plan, sampled)
+                    self._launch_chained(next_ahead, sampled, launched)
                     staged = self.sampler.finish(launched)
                 else:
                     staged = self.sampler.stage(logits, requests)
@@ -311,6 +312,24 @@ class Engine:
         if prepared is None:
             return None
         return _StepAhead(self._version, next_plan, prepared)
+
+    def _launch_chained(self, ahead: "_StepAhead | None", sampled: Sequence[SequenceState], launched) -> None:
+        """A recorded step of single tokens that was planned ahead is launched at once,
+        behind the running step, when its rows are the requests that the running step
+        samples, in that order: the sampling kernel's tokens go into its token ids on the
+        device, and the GPU does not wait while the host reads them and advances the
+        requests.  Should a request of it turn out to have ended (a stop token), or the set
+        of requests change before the next call, the step is thrown away like any step
+        planned ahead; it has then run for nothing."""
+
+        launch = getattr(self.runner, "launch_chained", None)
+        if ahead is None or launch is None or ahead.plan.prefill_items or not hasattr(ahead.prepared, "launched"):
+            return
+        tokens = launched[0]
+        rows = tuple(item.request_id for item in _longest_first(ahead.plan.decode_items))
+        if rows != tuple(state.request_id for state in sampled) or not getattr(tokens, "is_cuda", False):
+            return
+        launch(ahead.prepared, tokens)
 
     def _finalize(self, state: SequenceState) -> None:
         """A request that ended gives back its pages, its state slot and its random stream."""

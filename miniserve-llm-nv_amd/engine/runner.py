@@ -247,15 +247,32 @@ class DecodeGraph:
         self.replays += 1
         return self.logits[: len(entries)]
 
+    def launch_chained(self, which: int, tokens: torch.Tensor, count: int) -> None:
+        """Replays the step whose numbers :meth:`prepare` wrote into host buffer ``which``
+        with the token ids of its first ``count`` rows taken from ``tokens`` (int32, on
+        the device: what the sampling kernel of the step before chose, in row order)
+        instead of from the host, which has not read them yet.  Rows that only fill the
+        step up keep the ids they had (any id inside the vocabulary serves them)."""
 
-@dataclass(frozen=True)
+        start, size = self.offsets["token_ids"]
+        if start != 0 or self.graph is None:
+            raise RuntimeError("a chained step needs its recording, and the token ids at the front of its numbers.")
+        self.meta[size:].copy_(self.hosts[which][size:], non_blocking=True)
+        self.meta[:count].copy_(tokens[:count])
+        self.graph.replay()
+        self.replays += 1
+
+
+@dataclass
 class PreparedDecode:
     """A step of single tokens whose cache transaction is open and whose numbers are
-    written, but for the token ids."""
+    written, but for the token ids.  ``launched``: it runs already, its token ids fed on
+    the device from the sampling of the step before (:meth:`ModelRunner.launch_chained`)."""
 
     request_ids: tuple[str, ...]
     reservation: object
     buffer: int
+    launched: bool = False
 
 
 @dataclass(frozen=True)
@@ -321,6 +338,8 @@ class ModelRunner:
         self.graph_steps = 0
         self.prepared_steps = 0        # steps whose numbers were written while the step before ran
         self.prepared_mixed_steps = 0  # those of them that are not recorded steps
+        self.chained_steps = 0         # recorded steps launched before the host had read the tokens they run
+        self.voided_chained_steps = 0  # those of them that were thrown away (a request of theirs had ended)
 
     # ---- construction -----------------------------------------------------------------
     @classmethod
@@ -454,9 +473,31 @@ class ModelRunner:
             raise
         return PreparedStep(tuple(entry.request_id for entry in entries), reservation, built, tuple(admitted))
 
+    @torch.inference_mode()
+    def launch_chained(self, prepared: "PreparedDecode", tokens: torch.Tensor) -> None:
+        """Launches the prepared step of single tokens now, behind the step that is still
+        running: row ``i`` runs ``tokens[i]`` (int32 on the device, the sampling kernel's
+        output of the running step, whose rows are this step's requests in this order).
+        The host reads those tokens afterwards; :meth:`step` with this ``prepared`` then
+        launches nothing and returns the logits, and :meth:`discard` throws the step away
+        (it is a transaction like any other: what it wrote lies above the committed
+        lengths, its pages and state rows go back)."""
+
+        if prepared.launched:
+            raise RuntimeError("the step runs already.")
+        if tokens.dtype != torch.int32 or tokens.ndim != 1 or tokens.numel() < len(prepared.request_ids) or not tokens.is_cuda:
+            raise ValueError("a chained step takes the device's int32 tokens, one a request.")
+        metas = prepared.reservation.sequences
+        graph = self._decode_graphs[self._recorded_step_key(len(metas), max(meta.after for meta in metas))]
+        graph.launch_chained(prepared.buffer, tokens, len(metas))
+        prepared.launched = True
+        self.chained_steps += 1
+
     def discard(self, prepared: "PreparedDecode | PreparedStep") -> None:
         """Gives back what :meth:`prepare_decode` or :meth:`prepare_step` took."""
 
+        if getattr(prepared, "launched", False):
+            self.voided_chained_steps += 1
         self.cache.abort_step(prepared.reservation)
         for request_id in getattr(prepared, "admitted", ()):
             self.release(request_id)
@@ -491,6 +532,18 @@ class ModelRunner:
             self.prepared_steps += 1
         else:
             reservation = self._open_step(entries)
+        if prepared is not None and prepared.launched:
+            # the step runs already (launch_chained): its logits lie in its recording's output
+            metas = reservation.sequences
+            graph = self._decode_graphs[self._recorded_step_key(len(metas), max(meta.after for meta in metas))]
+            self.cache.commit_step(reservation)
+            self.steps_run += 1
+            self.tokens_run += len(entries)
+            self.graph_steps += 1
+            wanted = [index for index, entry in enumerate(entries) if entry.want]
+            if len(wanted) == len(entries):
+                return graph.logits[: len(entries)]
+            return graph.logits[torch.tensor(wanted, device=self.device)] if wanted else None
         if self.engine_config.decode_graphs and all(len(entry.token_ids) == 1 for entry in entries):
             try:
                 logits = self._decode_graph_step(entries, reservation, None if prepared is None else prepared.buffer)

@@ -92,6 +92,7 @@ def test_preempted_requests_under_recorded_steps_planned_ahead_match_the_plain_i
           f"{runner.prepared_steps} planned ahead ({runner.prepared_mixed_steps} with prompt portions)", flush=True)
     assert preempted >= 3 and engine.counters["preemptions"] == preempted
     assert runner.graph_steps > 0 and runner.prepared_steps > 0 and runner.prepared_mixed_steps > 0
+    assert runner.chained_steps > 0                 # steps launched before the host had read the tokens they ran
     assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (13,)
     worst = 0.0
     for index, (prompt, result) in enumerate(zip(prompts, results)):
@@ -111,6 +112,46 @@ def test_preempted_requests_under_recorded_steps_planned_ahead_match_the_plain_i
         # and the token is the largest of those logits
         assert [int(row.argmax()) for row in got] == list(result.token_ids)
     print(f"worst difference from the plain implementation {worst:.2e}", flush=True)
+
+
+def test_a_stop_token_throws_the_step_that_was_launched_ahead_away(model_folders):
+    """Decode steps are launched before the host has read the tokens they run.  When one
+    of those tokens turns out to be a request's stop token, the step that already runs is
+    thrown away and the others' tokens come out as if nothing had been launched: every
+    request's tokens are those of a run without stop tokens, cut behind the stop token."""
+
+    from miniserve_amd.config import EngineConfig
+    from miniserve_amd.engine import Engine, ModelRunner, SamplingParams
+
+    folder, block = model_folders["c"]
+    config = read_config(folder)
+    prompts = [random_tokens(n, config["vocab_size"], 950 + n) for n in (12, 30, 21, 44)]
+
+    def run(stops):
+        runner = ModelRunner.from_folder(folder, EngineConfig(dtype="float32", kv_block_size=block, num_kv_blocks=24, max_num_seqs=4))
+        engine = Engine(runner)
+        for index, prompt in enumerate(prompts):
+            engine.add_request(f"r{index}", prompt, SamplingParams(max_new_tokens=40, stop_token_ids=stops[index]), arrival_ns=index)
+        while engine.has_unfinished():
+            engine.step()
+            runner.cache.assert_invariants()
+        assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (24,)
+        return [engine.pop_result(f"r{index}") for index in range(len(prompts))], runner
+
+    free, runner = run([()] * 4)
+    assert runner.chained_steps > 20 and runner.voided_chained_steps == 0
+    # the first token that each of two requests produces for the first time at its 9th and 23rd place or later
+    stops, cut = [()] * 4, [40] * 4
+    for index, place in ((1, 8), (3, 22)):
+        tokens = free[index].token_ids
+        at = next(p for p in range(place, 40) if tokens[p] not in tokens[:p])
+        stops[index], cut[index] = (tokens[at],), at + 1
+    assert cut[1] < 40 and cut[3] < 40
+    stopped, runner = run(stops)
+    for index in range(4):
+        assert stopped[index].token_ids == free[index].token_ids[: cut[index]]
+        assert stopped[index].finish_reason == ("stop" if cut[index] < 40 else "length")
+    assert runner.voided_chained_steps == 2 and runner.chained_steps > 20
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
