@@ -36,6 +36,17 @@ class NonFiniteLogitsError(ValueError):
 class Sampler:
     def __init__(self) -> None:
         self._generators: dict[str, torch.Generator] = {}
+        # pinned host buffers that the chosen tokens are copied into, used in turn (a launch's
+        # tokens are read before the launch after the next one reuses its buffer)
+        self._token_buffers: list[torch.Tensor | None] = [None] * 4
+        self._token_turn = 0
+
+    def _token_buffer(self, rows: int) -> torch.Tensor:
+        index = self._token_turn = (self._token_turn + 1) % len(self._token_buffers)
+        buffer = self._token_buffers[index]
+        if buffer is None or buffer.numel() < rows:
+            buffer = self._token_buffers[index] = torch.empty(max(rows, 64), dtype=torch.int32, pin_memory=True)
+        return buffer[:rows]
 
     # ---- random streams ---------------------------------------------------------------
     @staticmethod
@@ -106,13 +117,26 @@ class Sampler:
                 logits, temperature=sent[0], top_p=sent[1], uniform=sent[2], top_k=sent[3].view(torch.int32),
                 top_p_alone=alone,
             )
-        return tokens, tuple(requests), states
+        # The copy to the host is asked for now, and an event marks its end: what the caller
+        # launches between here and finish() (the next step, fed from `tokens` on the device)
+        # lies behind the copy in the stream, and finish() does not wait for it.
+        arrived = None
+        if tokens.is_cuda:
+            on_host = self._token_buffer(tokens.numel())
+            on_host.copy_(tokens, non_blocking=True)
+            arrived = torch.cuda.Event()
+            arrived.record()
+        else:
+            on_host = tokens
+        return tokens, tuple(requests), states, on_host, arrived
 
     def finish(self, launched) -> tuple[StagedSample, ...]:
         """The second half of :meth:`stage`: waits for the tokens of :meth:`launch`."""
 
-        tokens, requests, states = launched
-        token_ids = tokens.tolist()
+        _, requests, states, on_host, arrived = launched
+        if arrived is not None:
+            arrived.synchronize()
+        token_ids = on_host.tolist()
         if any(token < 0 for token in token_ids):
             raise NonFiniteLogitsError("a row of logits holds a value that is not finite; no token can be chosen from it.")
         return tuple(
