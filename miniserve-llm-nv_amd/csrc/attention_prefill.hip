@@ -34,9 +34,7 @@ using ms::floatx16;
 using ms::kTileKeys;
 
 constexpr int kTileTokens = 64;       // query tokens of a workgroup at most
-constexpr int kComputeUnits = 256;
-constexpr int kXcds = 8;    // of the chip: a launch wants a workgroup for each
-constexpr int kPairedFrom = 2 * kComputeUnits - kComputeUnits / 4;   // workgroups from which they are handed out in pairs
+constexpr int kXcds = 8;    // dies of the chip, each with an L2 of its own (a wrong number costs speed only)
 constexpr int kWaveColumns = 32;      // columns (token, head) of one wave
 
 // Softmax arithmetic runs in base 2: the scale and log2(e) enter the exponent's
@@ -567,14 +565,15 @@ extern "C" int ms_attention_prefill(const void* q, const void* key_pool, const v
   // 512 tokens with histories lose, 37 -> 46 us: left as the rule has it.)
   const bool sorted = tile_order != 0;
   const int64_t with_two = static_cast<int64_t>(num_tiles) * num_kv_heads * ((group + 1) / 2);
-  const int hb = (group >= 2 && with_two >= kComputeUnits - kComputeUnits / 4) ? 2 : 1;
+  const int units = ms_compute_units();      // a launch wants a workgroup for each
+  const int hb = (group >= 2 && with_two >= units - units / 4) ? 2 : 1;
   const int64_t workgroups = static_cast<int64_t>(num_tiles) * num_kv_heads * ((group + hb - 1) / hb);
   // A long and a short tile to a workgroup where the pairs still fill the chip (256
   // compute units hold one workgroup each): then every workgroup walks about the same
   // number of keys (8,192 tokens of 16 heads: 396 -> 294 us).  A small launch keeps a tile
   // a workgroup: the longest tile sets its time either way, and a second tile costs a
   // workgroup a second start.
-  const int paired = sorted && workgroups >= kPairedFrom;
+  const int paired = sorted && workgroups >= 2 * units - units / 4;
   MS_REQUIRE(num_kv_heads * ((group + hb - 1) / hb) <= 65535, "attention_prefill: too many heads");
 #define MS_PREFILL_CASE(DIM)                                                                                       \
   case DIM:                                                                                                        \

@@ -124,6 +124,9 @@ enum MsDtype : int { MS_F32 = 0, MS_BF16 = 1 };
 // Records a message for ms_last_error() and returns a non-zero code.
 int ms_fail(const char* format, ...);
 
+// Compute units of the current device (256 on MI355X), asked once.
+int ms_compute_units();
+
 #define MS_REQUIRE(cond, ...)                \
   do {                                       \
     if (!(cond)) return ms_fail(__VA_ARGS__); \

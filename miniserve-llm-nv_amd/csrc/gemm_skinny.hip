@@ -221,19 +221,20 @@ void launch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, 
   const int out_rows = epilogue == kSiluMul ? n / 2 : n;
   const int blocks_per_group = epilogue == kSiluMul ? RB / 2 : RB;
   const int m_tiles = (m + 16 * MB - 1) / (16 * MB);
-  // How many of the 16 rows of a block a workgroup takes.  The chip has 256 compute
-  // units; the launch lasts as long as the unit with the most to stream, that is
-  // ceil(workgroups / 256) times a workgroup's rows: 6144 rows in blocks of 16 are 384
+  // How many of the 16 rows of a block a workgroup takes.  The chip has `units` compute
+  // units (256 on MI355X); the launch lasts as long as the unit with the most to stream, that is
+  // ceil(workgroups / units) times a workgroup's rows: 6144 rows in blocks of 16 are 384
   // workgroups, two for half of the units and one for the others; in blocks of 12 they are
   // 512, two for each, and a quarter less to stream for the busiest.  Fewest rows on the
   // busiest unit wins, more rows a workgroup among equals (fewer workgroups, less of x read).
   int rows = 16;
+  const int64_t units = ms_compute_units();
   if (RB <= 2) {
     int64_t best = INT64_MAX;
     for (int candidate = 16; candidate >= 4; --candidate) {
       const int64_t workgroups =
           static_cast<int64_t>((out_rows + candidate * blocks_per_group - 1) / (candidate * blocks_per_group)) * m_tiles;
-      const int64_t busiest = ((workgroups + 255) / 256) * candidate;
+      const int64_t busiest = ((workgroups + units - 1) / units) * candidate;
       if (busiest < best) {
         best = busiest;
         rows = candidate;

@@ -282,10 +282,17 @@ def _report_fallback(head_dim: int, block_size: int, reason: str) -> None:
         )
 
 
-# Workgroups that the key-split attention aims to launch: a few per compute unit
-# (the chip has 256), so that short batches still fill it.
-_DECODE_TARGET_WORKGROUPS = 512
+# Workgroups that the key-split attention aims to launch: two per compute unit, so that
+# short batches still fill the chip (256 units on MI355X: 512).
 _DECODE_MAX_SPLITS = 64
+_decode_target_workgroups: int | None = None
+
+
+def _decode_target() -> int:
+    global _decode_target_workgroups
+    if _decode_target_workgroups is None:
+        _decode_target_workgroups = 2 * int(load().ms_device_compute_units())
+    return _decode_target_workgroups
 
 
 def decode_splits(num_tokens: int, num_kv_heads: int, group: int, max_context: int) -> int:
@@ -295,7 +302,7 @@ def decode_splits(num_tokens: int, num_kv_heads: int, group: int, max_context: i
     of 2,100)."""
 
     rows = num_tokens * num_kv_heads * ((group + 15) // 16)
-    by_chip = -(-_DECODE_TARGET_WORKGROUPS // rows)
+    by_chip = -(-_decode_target() // rows)
     by_keys = max(1, max_context // 160)
     return max(1, min(by_chip, by_keys, _DECODE_MAX_SPLITS))
 

@@ -42,6 +42,7 @@ _SIGNATURES: dict[str, list] = {
     "ms_gemm_library_bucket": [_I],
     "ms_gemm_library_time": [_P, _P, _P, _I, _I, _I, _I, _P, c_size_t, _P, c_size_t, _P, _P, _I, _P, _P],
     "ms_silu_mul": [_P, _P, _I, _I, _I, _P],
+    "ms_device_compute_units": [],
     "ms_sample_rows": [_P, _P, _P, _P, _P, _P, _I, _I, _P],
     "ms_argmax_rows": [_P, _P, _P, _P, _I, _I, _I, _P],
     "ms_sample_rows_workspace_bytes": [_I, _I],
