@@ -330,7 +330,6 @@ class ModelRunner:
         )
         self.cache.allocate_storage(self.dtype, self.device)
         self._call_views = self.cache.call_views()
-        self.max_blocks_per_seq = tuple(-(-self.max_model_len // size) for size in self.cache.block_sizes)
         self._decode_graphs: dict[tuple[int, int], DecodeGraph] = {}     # by (rows, context bound)
         self._graph_pool = None
         self.steps_run = 0

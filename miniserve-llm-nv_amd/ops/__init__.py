@@ -20,12 +20,18 @@ from .library import KernelError, call, library_path, load
 
 __all__ = [
     "KernelError",
+    "LIBRARY_PRODUCTS_TABLE",
     "PREFILL_TILE_TOKENS",
     "QueryTiles",
     "attention",
     "attention_calls",
     "forced_product",
+    "hipblaslt_build",
+    "library_product_bucket",
+    "noting_library_products",
+    "open_gemm_library",
     "prefers_skinny",
+    "prepare_products",
     "product_calls",
     "query_tiles_host",
     "embedding_gather",
@@ -42,6 +48,7 @@ __all__ = [
     "rope_table",
     "sample_rows",
     "silu_mul",
+    "time_library_product",
 ]
 
 _DTYPE_CODES = {torch.float32: 0, torch.bfloat16: 1}
