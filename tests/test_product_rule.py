@@ -65,3 +65,25 @@ def test_a_forced_product_overrides_the_rule_and_is_undone():
     with pytest.raises(ValueError):
         with ops.forced_product("fastest"):
             pass
+
+
+def test_the_table_of_pinned_library_solutions_is_well_formed():
+    """``ops/library_products.json``: the library's build it was measured under and one pin
+    for a (matrix, output type, bucket of row counts), each once, all whole numbers; the
+    matrices of the three presets are there."""
+
+    import json
+
+    from miniserve_amd import ops
+
+    table = json.loads(ops.LIBRARY_PRODUCTS_TABLE.read_text())
+    assert isinstance(table["library"], str) and ":" in table["library"]
+    pins = table["pins"]
+    assert all(len(pin) == 5 and all(type(v) is int for v in pin) for pin in pins)
+    keys = [tuple(pin[:4]) for pin in pins]
+    assert len(keys) == len(set(keys)) and all(pin[2] in (0, 1) and pin[3] >= 0 and pin[4] > 0 for pin in pins)
+    matrices = {(n, k) for n, k, _, _, _ in pins}
+    # q/k/v, o, gate and up, down of the 0.6B, 8B and 32B sizes (o and down add into the 32-bit stream)
+    for shape in [(4096, 1024), (1024, 2048), (6144, 1024), (1024, 3072), (6144, 4096), (4096, 4096), (24576, 4096),
+                  (4096, 12288), (10240, 5120), (5120, 8192), (51200, 5120), (5120, 25600)]:
+        assert shape in matrices, shape
