@@ -480,3 +480,39 @@ def test_a_preempted_request_builds_its_state_again(toy):
     assert tight.generate(prompts, params) == expected
     assert tight.engine.counters["preemptions"] > 0
     tight.runner.cache.assert_invariants()
+
+
+def test_a_chained_step_that_is_thrown_away_puts_the_state_back(toy):
+    """Recorded steps are launched before the host has read the tokens they run.  When a
+    stop token ends a request, the step that runs already is thrown away, and with it what
+    its mixers wrote into the state rows of the OTHER requests: their tokens are those of
+    a run without stop tokens, which the plain form and the plain sampler confirm on the way
+    (temperature 1 from a seed a request, so that the tokens vary)."""
+
+    import plain_sampling
+
+    from miniserve_amd.engine import SamplingParams
+    from miniserve_amd.entrypoint import LLM
+    from miniserve_amd.sampling import Sampler
+
+    config, weights = read_config(toy), read_weights(toy)
+    prompts = [random_tokens(n, config["vocab_size"], 700 + n) for n in (9, 22, 15)]
+    options = dict(dtype="float32", kv_block_size=16, num_kv_blocks=24, max_num_seqs=4)
+    sampling = lambda index, **more: SamplingParams(max_new_tokens=30, temperature=1.0, seed=40 + index, **more)
+    free_engine = LLM(str(toy), **options)
+    free = free_engine.generate(prompts, [sampling(index) for index in range(3)])
+    assert free_engine.runner.chained_steps > 10 and free_engine.runner.voided_chained_steps == 0
+    for index, (prompt, tokens) in enumerate(zip(prompts, free)):         # against the plain form and the plain sampler
+        logits = toy_logits(weights, config, list(prompt) + tokens[:-1])[len(prompt) - 1 :].float()
+        stream = torch.Generator().manual_seed(40 + index)
+        for place, token in enumerate(tokens):
+            uniform = Sampler.draw_uniform(stream)
+            if plain_sampling.edge_distance(logits[place], 1.0, 0, 1.0, uniform) > 1e-4:      # a draw on an edge may fall either way
+                assert token == plain_sampling.sample_row(logits[place], 1.0, 0, 1.0, uniform), (index, place)
+    # request 1 stops at the first token that it produces for the first time at its 7th place or later
+    at = next(p for p in range(6, 30) if free[1][p] not in free[1][:p])
+    stopped_engine = LLM(str(toy), **options)
+    stopped = stopped_engine.generate(prompts, [sampling(0), sampling(1, stop_token_ids=(free[1][at],)), sampling(2)])
+    assert stopped == [free[0], free[1][: at + 1], free[2]]
+    assert stopped_engine.runner.voided_chained_steps == 1
+    stopped_engine.runner.cache.assert_invariants()
