@@ -23,6 +23,12 @@
 //   2  out_f32 += C                                    residual add (qwen3.py:367-368, 381-382)
 //   3  out = bf16(silu(C[gate row]) * C[up row])       gated activation (layers.py:86-87);
 //      the workgroup owns row n of the gate half and row n + N/2 of the up half
+//   4  as 2, and the RMSNorm that follows the residual add is prepared: beside the new
+//      residual value v the workgroup stores bf16(w_norm[n] * v), the operand of the product
+//      behind that norm, and the sum of v^2 over its own columns for every row, into a slot
+//      of its own (no atomics: the sums have a fixed order).  The product behind the norm
+//      (ms_gemm_skinny_scaled) adds the workgroups' sums in their order, and
+//      scales its own sums by 1 / rms: the norm is no kernel and no prologue of its own.
 #include "mfma.hpp"
 
 namespace {
@@ -34,7 +40,16 @@ using ms::floatx4;
 constexpr int kWavesPerGroup = 8;
 constexpr int kGroupThreads = kWavesPerGroup * ms::kWave;
 
-enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAddF32 = 2, kSiluMul = 3 };
+enum Epilogue : int { kStoreBf16 = 0, kStoreF32 = 1, kAddF32 = 2, kSiluMul = 3, kAddF32Ahead = 4 };
+
+// What the epilogue 4 leaves for the product behind the norm, and what that product reads.
+struct NormAhead {
+  const bf16* weight;   // of the norm, [n of the producer]
+  bf16* x;              // [m, n]: bf16(weight * residual)
+  float* squares;       // [groups, m]: every producer workgroup's sum of squares of its columns
+  int groups;           // of the producer (its gridDim.x); for the consumer: how many to add
+  float eps;
+};
 // rows of W from which two blocks of 10 rows and more a workgroup still make 256 workgroups
 constexpr int kTwoBlockRows = 5120;
 
@@ -47,17 +62,21 @@ constexpr int kTwoBlockRows = 5120;
 // normalised value before the multiply by the weight, as the reference does; here
 // the one rounding is of w_norm * h.  Both carry 8 significant bits.)
 // UNROLL: k-steps whose loads are issued together (more for long rows: more bytes in flight)
-template <int MB, int RB, bool NORM, int UNROLL>
+template <int MB, int RB, bool NORM, int UNROLL, bool SCALED>
 __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* __restrict__ x,
                                                                     const float* __restrict__ h,
                                                                     const bf16* __restrict__ norm_weight, float eps,
                                                                     const bf16* __restrict__ w, bf16* out_bf16,
                                                                     float* out_f32, int m, int n, int k,
-                                                                    int epilogue, int rows) {
+                                                                    int epilogue, int rows, NormAhead ahead) {
+  // ahead: epilogue 4 writes it.  SCALED: x is the `ahead.x` of a product before; the sums are
+  // scaled by 1 / sqrt(mean of squares + eps), the squares taken from ahead.squares.
   // rows: how many of the 16 rows of a block are this workgroup's (16, or 8 or 4 for a
   // matrix of few rows, so that there are workgroups enough to fill the chip)
   __shared__ float c_s[kWavesPerGroup][RB * MB][16][16];
   __shared__ float square_s[kWavesPerGroup][16];
+  __shared__ float tile_square_s[RB * MB][16];      // epilogue 4: a tile's sum of squares a row
+  __shared__ float inv_rms_s[MB * 16];              // SCALED: 1 / rms of the workgroup's rows of x
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -108,7 +127,8 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
   // will add to is asked for now, so that it has arrived when the sums are made (no
   // other thread writes it).
   float residual_ahead = 0.f;
-  if (epilogue == kAddF32 && threadIdx.x < RB * MB * 256) {
+  const bool adds = epilogue == kAddF32 || epilogue == kAddF32Ahead;
+  if (adds && threadIdx.x < RB * MB * 256) {
     const int n_local = threadIdx.x & 15, m_local = (threadIdx.x >> 4) & 15, tile = threadIdx.x >> 8;
     const int rb = tile / MB, mb = tile - rb * MB;
     const int row_m = m_base + 16 * mb + m_local, col_n = row_start[rb] + n_local;
@@ -118,6 +138,24 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
   // NORM: this lane makes column m = r of x from row r of h, and sums its squares
   const float* h_row = NORM ? h + static_cast<int64_t>(min(r, m - 1)) * k : nullptr;
   float square_sum = 0.f;
+
+  // SCALED: the threads are dealt to the workgroup's rows of x (32, 16 or 8 to a row); each
+  // asks now, ahead of the walk along K, for its share of the producer workgroups' sums of
+  // that row's squares (the loads go out before the first of W and have arrived when those
+  // have), and adds them up after the walk in their order, with what more there may be.
+  constexpr int kStatThreads = kGroupThreads / (16 * MB);
+  constexpr int kStatAhead = 8;
+  float group_square[kStatAhead];
+  const int stat_row = threadIdx.x / kStatThreads, stat_part = threadIdx.x % kStatThreads;
+  const bool stat_live = SCALED && m_base + stat_row < m;
+  const float* stat_from = ahead.squares + m_base + stat_row;
+  if (SCALED) {
+#pragma unroll
+    for (int j = 0; j < kStatAhead; ++j) {
+      const int group = stat_part + kStatThreads * j;
+      group_square[j] = (stat_live && group < ahead.groups) ? stat_from[static_cast<int64_t>(group) * m] : 0.f;
+    }
+  }
 
   const int steps = (k + 31) / 32;
   for (int base = wave; base < steps; base += kWavesPerGroup * UNROLL) {
@@ -172,6 +210,17 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     square_sum += __shfl_xor(square_sum, 32, ms::kWave);
     if (g == 0) square_s[wave][r] = square_sum;
   }
+  if (SCALED) {
+    float total = 0.f;
+#pragma unroll
+    for (int j = 0; j < kStatAhead; ++j) total += group_square[j];
+    if (stat_live)
+      for (int group = stat_part + kStatThreads * kStatAhead; group < ahead.groups; group += kStatThreads)
+        total += stat_from[static_cast<int64_t>(group) * m];
+#pragma unroll
+    for (int step = 1; step < kStatThreads; step *= 2) total += __shfl_xor(total, step, ms::kWave);
+    if (stat_part == 0) inv_rms_s[stat_row] = 1.0f / sqrtf(total / static_cast<float>(k) + ahead.eps);
+  }
   __syncthreads();
 
   // c_s[wave][tile][m_local][n_local]; consecutive threads take consecutive n
@@ -184,7 +233,8 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     const int rb = tile / MB, mb = tile - rb * MB;
     const int row_m = m_base + 16 * mb + m_local;
     const int col_n = row_start[rb] + n_local;
-    if (row_m >= m || col_n >= row_limit || n_local >= rows) continue;
+    const bool live = row_m < m && col_n < row_limit && n_local < rows;
+    if (epilogue != kAddF32Ahead && !live) continue;      // (epilogue 4: every lane of a row's sixteen takes part in its sum)
     float sum = 0.f;
 #pragma unroll
     for (int wv = 0; wv < kWavesPerGroup; ++wv) sum += c_s[wv][tile][m_local][n_local];
@@ -195,6 +245,9 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
       for (int wv = 0; wv < kWavesPerGroup; ++wv) squares += square_s[wv][m_local];
       inv_rms = 1.0f / sqrtf(squares / static_cast<float>(k) + eps);
       sum *= inv_rms;
+    } else if (SCALED) {
+      inv_rms = inv_rms_s[16 * mb + m_local];
+      sum *= inv_rms;
     }
     if (epilogue == kStoreBf16) {
       out_bf16[static_cast<int64_t>(row_m) * n + col_n] = ms::from_float<bf16>(sum);
@@ -203,6 +256,21 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
     } else if (epilogue == kAddF32) {
       float* place = out_f32 + static_cast<int64_t>(row_m) * n + col_n;
       *place = (index == static_cast<int>(threadIdx.x) ? residual_ahead : *place) + sum;
+    } else if (epilogue == kAddF32Ahead) {
+      float square = 0.f;
+      if (live) {
+        const int64_t at = static_cast<int64_t>(row_m) * n + col_n;
+        const float value = (index == static_cast<int>(threadIdx.x) ? residual_ahead : out_f32[at]) + sum;
+        out_f32[at] = value;
+        ahead.x[at] = ms::from_float<bf16>(ms::to_float(ahead.weight[col_n]) * value);
+        square = value * value;
+      }
+      // the sixteen columns of the tile's row: a fixed tree over the lanes
+      square += __shfl_xor(square, 1, ms::kWave);
+      square += __shfl_xor(square, 2, ms::kWave);
+      square += __shfl_xor(square, 4, ms::kWave);
+      square += __shfl_xor(square, 8, ms::kWave);
+      if (n_local == 0) tile_square_s[tile][m_local] = square;
     } else {
       float up = 0.f;
 #pragma unroll
@@ -213,46 +281,100 @@ __global__ __launch_bounds__(kGroupThreads) void gemm_skinny_kernel(const bf16* 
       out_bf16[static_cast<int64_t>(row_m) * half + col_n] = ms::from_float<bf16>(gate / (1.0f + __expf(-gate)) * up);
     }
   }
+  if (epilogue == kAddF32Ahead) {
+    // this workgroup's share of every row's squares: its tiles of that row, in their order
+    __syncthreads();
+    if (threadIdx.x < MB * 16) {
+      const int mb = threadIdx.x >> 4, m_local = threadIdx.x & 15;
+      const int row_m = m_base + 16 * mb + m_local;
+      float total = 0.f;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) total += tile_square_s[rb * MB + mb][m_local];
+      if (row_m < m) ahead.squares[static_cast<int64_t>(blockIdx.x) * m + row_m] = total;
+    }
+  }
 }
 
-template <int MB, int RB, bool NORM = false>
-void launch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, int n, int k, int epilogue,
-            hipStream_t stream, const void* h = nullptr, const void* norm_weight = nullptr, float eps = 0.f) {
+// How a product is cut into workgroups: `rows` of the 16 rows of a block to a workgroup (see
+// launch()), `groups` workgroups along N, `m_tiles` along M.
+struct Cut {
+  int rows, groups, m_tiles;
+};
+
+Cut cut_of(int mb_t, int rb_t, int m, int n, int epilogue) {
   const int out_rows = epilogue == kSiluMul ? n / 2 : n;
-  const int blocks_per_group = epilogue == kSiluMul ? RB / 2 : RB;
-  const int m_tiles = (m + 16 * MB - 1) / (16 * MB);
+  const int blocks_per_group = epilogue == kSiluMul ? rb_t / 2 : rb_t;
+  Cut cut;
+  cut.m_tiles = (m + 16 * mb_t - 1) / (16 * mb_t);
   // How many of the 16 rows of a block a workgroup takes.  The chip has `units` compute
   // units (256 on MI355X); the launch lasts as long as the unit with the most to stream, that is
   // ceil(workgroups / units) times a workgroup's rows: 6144 rows in blocks of 16 are 384
   // workgroups, two for half of the units and one for the others; in blocks of 12 they are
   // 512, two for each, and a quarter less to stream for the busiest.  Fewest rows on the
   // busiest unit wins, more rows a workgroup among equals (fewer workgroups, less of x read).
-  int rows = 16;
+  cut.rows = 16;
   const int64_t units = ms_compute_units();
-  if (RB <= 2) {
+  if (rb_t <= 2) {
     int64_t best = INT64_MAX;
     for (int candidate = 16; candidate >= 4; --candidate) {
       const int64_t workgroups =
-          static_cast<int64_t>((out_rows + candidate * blocks_per_group - 1) / (candidate * blocks_per_group)) * m_tiles;
+          static_cast<int64_t>((out_rows + candidate * blocks_per_group - 1) / (candidate * blocks_per_group)) * cut.m_tiles;
       const int64_t busiest = ((workgroups + units - 1) / units) * candidate;
       if (busiest < best) {
         best = busiest;
-        rows = candidate;
+        cut.rows = candidate;
       }
     }
   }
-  const int groups = (out_rows + rows * blocks_per_group - 1) / (rows * blocks_per_group);
+  cut.groups = (out_rows + cut.rows * blocks_per_group - 1) / (cut.rows * blocks_per_group);
+  return cut;
+}
+
+template <int MB, int RB, bool NORM = false, bool SCALED = false>
+void launch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, int n, int k, int epilogue,
+            hipStream_t stream, const void* h = nullptr, const void* norm_weight = nullptr, float eps = 0.f,
+            NormAhead ahead = NormAhead{nullptr, nullptr, nullptr, 0, 0.f}) {
+  const Cut cut = cut_of(MB, RB, m, n, epilogue);
   // rows of 2048 elements and more: eight k-steps in flight a wave (where the registers allow it)
-  if (k >= 2048 && MB * RB <= 2) {
-    hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 8>), dim3(groups, m_tiles), dim3(kGroupThreads), 0, stream,
-                       static_cast<const bf16*>(x), static_cast<const float*>(h),
-                       static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
-                       static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue, rows);
+  if constexpr (MB * RB <= 2) {
+    if (k >= 2048) {
+      hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 8, SCALED>), dim3(cut.groups, cut.m_tiles), dim3(kGroupThreads), 0,
+                         stream, static_cast<const bf16*>(x), static_cast<const float*>(h),
+                         static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
+                         static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue, cut.rows, ahead);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 4, SCALED>), dim3(cut.groups, cut.m_tiles), dim3(kGroupThreads), 0,
+                     stream, static_cast<const bf16*>(x), static_cast<const float*>(h),
+                     static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
+                     static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue, cut.rows, ahead);
+}
+
+// Which instantiation serves a product of `m` rows against `n` rows of W: (MB, RB) as the
+// entry point below chooses them.
+void shape_of(int m, int n, int epilogue, int* mb_t, int* rb_t) {
+  const int mb = (m + 15) / 16;
+  const int out_rows = epilogue == kSiluMul ? n / 2 : n;
+  const bool many_rows = out_rows >= 32768;   // the head: larger tiles, fewer workgroups
+  if (mb == 1) {
+    *mb_t = 1;
+    if (epilogue == kSiluMul) *rb_t = 2;
+    else if (many_rows) *rb_t = 4;
+    else if (out_rows >= kTwoBlockRows && m >= 4) *rb_t = 2;
+    else *rb_t = 1;
+  } else if (out_rows <= 2048 && epilogue != kSiluMul) {
+    *mb_t = 1;
+    *rb_t = 1;
+  } else if (epilogue == kSiluMul) {
+    *mb_t = mb == 2 ? 2 : 4;
+    *rb_t = 2;
+  } else if (mb == 2) {
+    *mb_t = 2;
+    *rb_t = many_rows ? 2 : 1;
   } else {
-    hipLaunchKernelGGL((gemm_skinny_kernel<MB, RB, NORM, 4>), dim3(groups, m_tiles), dim3(kGroupThreads), 0, stream,
-                       static_cast<const bf16*>(x), static_cast<const float*>(h),
-                       static_cast<const bf16*>(norm_weight), eps, static_cast<const bf16*>(w),
-                       static_cast<bf16*>(out_bf16), static_cast<float*>(out_f32), m, n, k, epilogue, rows);
+    *mb_t = 4;
+    *rb_t = 1;
   }
 }
 
@@ -264,6 +386,40 @@ extern "C" int ms_gemm_skinny_supported(int m, int n, int k, int epilogue) {
   return epilogue >= 0 && epilogue <= 3;
 }
 
+namespace {
+
+void dispatch(const void* x, const void* w, void* out_bf16, void* out_f32, int m, int n, int k, int epilogue,
+              hipStream_t stream, NormAhead ahead, bool scaled) {
+  int mb_t, rb_t;
+  shape_of(m, n, epilogue, &mb_t, &rb_t);
+  // One row block (m <= 16), by the rows of W:
+  //   Every workgroup reads all of x beside its rows of W, and the loads of x take the
+  //   places of loads of W among those in flight.  From kTwoBlockRows rows of W on, two
+  //   blocks a workgroup still give a workgroup to every compute unit, and half as many
+  //   workgroups read x (25600 x 5120 at 8 rows: 74 -> 63 us); one row of x costs little either way.
+  // More than 16 rows against a matrix of few rows: a workgroup that took all rows of x
+  //   would read far more of x than of W.  The launch is cut along M too: 16 rows of x
+  //   against 16 (or fewer) rows of W a workgroup.
+#define MS_SKINNY_CASE(MB, RB)                                                                                 \
+  if (mb_t == MB && rb_t == RB) {                                                                              \
+    if (scaled) launch<MB, RB, false, true>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream, nullptr, nullptr, 0.f, ahead); \
+    else launch<MB, RB>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream, nullptr, nullptr, 0.f, ahead);      \
+    return;                                                                                                    \
+  }
+  MS_SKINNY_CASE(1, 1);
+  MS_SKINNY_CASE(1, 2);
+  MS_SKINNY_CASE(1, 4);
+  MS_SKINNY_CASE(2, 1);
+  MS_SKINNY_CASE(2, 2);
+  MS_SKINNY_CASE(4, 1);
+  MS_SKINNY_CASE(4, 2);
+#undef MS_SKINNY_CASE
+}
+
+const NormAhead kNoNormAhead{nullptr, nullptr, nullptr, 0, 0.f};
+
+}  // namespace
+
 // x: bfloat16 [m, k]; w: bfloat16 [n, k]; the output by epilogue: 0 bfloat16 [m, n],
 // 1 and 2 float [m, n], 3 bfloat16 [m, n / 2].
 extern "C" int ms_gemm_skinny(const void* x, const void* w, void* out_bf16, void* out_f32, int m, int n, int k,
@@ -273,33 +429,52 @@ extern "C" int ms_gemm_skinny(const void* x, const void* w, void* out_bf16, void
              epilogue);
   MS_REQUIRE((epilogue == kStoreBf16 || epilogue == kSiluMul) ? out_bf16 != nullptr : out_f32 != nullptr,
              "gemm_skinny: the output of epilogue %d is null", epilogue);
-  const int mb = (m + 15) / 16;
-  const int out_rows = epilogue == kSiluMul ? n / 2 : n;
-  const bool many_rows = out_rows >= 32768;   // the head: larger tiles, fewer workgroups
-  if (mb == 1) {
-    if (epilogue == kSiluMul) launch<1, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-    else if (many_rows) launch<1, 4>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-    // Every workgroup reads all of x beside its rows of W, and the loads of x take the
-    // places of loads of W among those in flight.  From kTwoBlockRows rows of W on, two
-    // blocks a workgroup still give a workgroup to every compute unit, and half as many
-    // workgroups read x (25600 x 5120 at 8 rows: 74 -> 63 us); one row of x costs little either way.
-    else if (out_rows >= kTwoBlockRows && m >= 4) launch<1, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-    else launch<1, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-  } else if (out_rows <= 2048 && epilogue != kSiluMul) {
-    // More than 16 rows against a matrix of few rows: a workgroup that took all rows of x
-    // would read far more of x than of W.  The launch is cut along M too: 16 rows of x
-    // against 16 (or fewer) rows of W a workgroup.
-    launch<1, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-  } else if (epilogue == kSiluMul) {
-    if (mb == 2) launch<2, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-    else launch<4, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-  } else if (mb == 2) {
-    if (many_rows) launch<2, 2>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-    else launch<2, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-  } else {
-    launch<4, 1>(x, w, out_bf16, out_f32, m, n, k, epilogue, stream);
-  }
+  dispatch(x, w, out_bf16, out_f32, m, n, k, epilogue, stream, kNoNormAhead, false);
   MS_CHECK_LAUNCH("gemm_skinny");
+  return 0;
+}
+
+// How many workgroups along N the += product of [m, k] against W [n, k] is cut into: the
+// first size of the `squares` that ms_gemm_skinny_norm_ahead writes.
+extern "C" int ms_gemm_skinny_groups(int m, int n) {
+  int mb_t, rb_t;
+  shape_of(m, n, kAddF32, &mb_t, &rb_t);
+  return cut_of(mb_t, rb_t, m, n, kAddF32).groups;
+}
+
+// h[m, n] += x[m, k] . W[n, k]^T as epilogue 2, and for the RMSNorm (weight `norm_weight`
+// [n]) and the product that follow: ahead_x[m, n] = bf16(norm_weight * h) and
+// squares[group, m] = the sum of h^2 over the columns of workgroup `group`, for the
+// ms_gemm_skinny_groups(m, n) workgroups.
+extern "C" int ms_gemm_skinny_norm_ahead(const void* x, const void* w, void* h, int m, int n, int k,
+                                         const void* norm_weight, void* ahead_x, void* squares,
+                                         hipStream_t stream) {
+  MS_REQUIRE(ms_gemm_skinny_supported(m, n, k, kAddF32),
+             "gemm_skinny_norm_ahead: m %d (1..64), n %d or k %d (a multiple of 8) is not supported", m, n, k);
+  MS_REQUIRE(h != nullptr && norm_weight != nullptr && ahead_x != nullptr && squares != nullptr,
+             "gemm_skinny_norm_ahead: an output or the norm's weight is null");
+  const NormAhead ahead{static_cast<const bf16*>(norm_weight), static_cast<bf16*>(ahead_x),
+                        static_cast<float*>(squares), ms_gemm_skinny_groups(m, n), 0.f};
+  dispatch(x, w, nullptr, h, m, n, k, kAddF32Ahead, stream, ahead, false);
+  MS_CHECK_LAUNCH("gemm_skinny_norm_ahead");
+  return 0;
+}
+
+// ms_gemm_skinny of the RMSNorm that ms_gemm_skinny_norm_ahead prepared: x is its ahead_x
+// [m, k], squares [groups, m] its sums; every sum of the product is scaled by
+// 1 / sqrt(sum of the row's squares / k + eps) before the epilogue.
+extern "C" int ms_gemm_skinny_scaled(const void* x, const void* w, void* out_bf16, void* out_f32, int m, int n,
+                                     int k, int epilogue, const void* squares, int groups, float eps,
+                                     hipStream_t stream) {
+  MS_REQUIRE(ms_gemm_skinny_supported(m, n, k, epilogue) && epilogue != kAddF32Ahead,
+             "gemm_skinny_scaled: m %d (1..64), n %d, k %d (a multiple of 8) or epilogue %d is not supported", m, n,
+             k, epilogue);
+  MS_REQUIRE((epilogue == kStoreBf16 || epilogue == kSiluMul) ? out_bf16 != nullptr : out_f32 != nullptr,
+             "gemm_skinny_scaled: the output of epilogue %d is null", epilogue);
+  MS_REQUIRE(squares != nullptr && groups >= 1, "gemm_skinny_scaled: no sums of squares (%d groups)", groups);
+  const NormAhead ahead{nullptr, nullptr, const_cast<float*>(static_cast<const float*>(squares)), groups, eps};
+  dispatch(x, w, out_bf16, out_f32, m, n, k, epilogue, stream, ahead, true);
+  MS_CHECK_LAUNCH("gemm_skinny_scaled");
   return 0;
 }
 

@@ -40,6 +40,10 @@ __all__ = [
     "linear_normed",
     "linear_silu_mul",
     "can_fuse_norm",
+    "can_prepare_norm",
+    "can_use_prepared_norm",
+    "linear_norm_ahead",
+    "linear_prepared",
     "can_accumulate",
     "load",
     "qk_norm_rope_append",
@@ -704,6 +708,99 @@ def linear_normed(
     product_calls["skinny"] += 1
     call("ms_gemm_skinny_normed", _ptr(residual), _ptr(norm_weight), float(eps), _ptr(weight), _ptr(out), m, n, k,
          _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16, _stream())
+    return out
+
+
+def can_prepare_norm(rows: int, weight: torch.Tensor) -> bool:
+    """Whether :func:`linear_norm_ahead` serves ``rows`` rows against ``weight``: where
+    ``linear(..., accumulate_into=...)`` would run this library's product."""
+
+    n, k = weight.shape
+    return (
+        weight.dtype == torch.bfloat16
+        and rows <= SKINNY_KERNEL_ROWS
+        and bool(load().ms_gemm_skinny_supported(rows, n, k, _EPILOGUE_ADD_F32))
+        and prefers_skinny(rows, n, k)
+    )
+
+
+def can_use_prepared_norm(rows: int, weight: torch.Tensor, *, gated: bool = False) -> bool:
+    """Whether :func:`linear_prepared` is the form to take for ``rows`` rows against
+    ``weight``: where this library's product serves the shape and the norm would otherwise
+    be a kernel of its own.  Measured on MI355X, pairs of (+= product, norm, product) in
+    recorded graphs over matrices that no cache holds, in us, as (norm kernel | norm as
+    prologue | prepared): 1024 wide into 6144 rows, 8 rows 13.0 | 11.1 | 11.7, 64 rows
+    18.7 | - | 17.2; 4096 wide into 24576 rows, 8 rows 58.7 | 63.9 | 56.5, 16 rows
+    66.0 | 73.6 | 68.1.  A small matrix with few rows keeps the prologue; every workgroup
+    of the prepared form reads all rows' partial sums (as many as the product before had
+    workgroups), which costs a large matrix more than the norm kernel from 16 rows on."""
+
+    n, k = weight.shape
+    epilogue = _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16
+    if not (
+        weight.dtype == torch.bfloat16
+        and rows <= SKINNY_KERNEL_ROWS
+        and bool(load().ms_gemm_skinny_supported(rows, n, k, epilogue))
+        and prefers_skinny(rows, n, k, fused=True)
+    ):
+        return False
+    if _forced_product is not None:
+        return True
+    if can_fuse_norm(rows, weight, gated=gated):
+        return False
+    return rows <= 8 or 2 * n * k <= 16 * _MIB
+
+
+def linear_norm_ahead(
+    x: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """``residual += x @ weight^T`` as ``linear(..., accumulate_into=residual)``, and in the
+    same kernel what the RMSNorm of the new ``residual`` needs: returns ``(weighted,
+    squares)`` with ``weighted [M, N]`` = bfloat16(norm_weight * residual) and ``squares
+    [G, M]``, every workgroup's sum of ``residual^2`` over its columns.
+    :func:`linear_prepared` takes a product of that norm from the two."""
+
+    _check(x, "x", dtype=torch.bfloat16)
+    _check(weight, "weight", dtype=torch.bfloat16)
+    if x.ndim != 2 or weight.ndim != 2 or x.shape[1] != weight.shape[1] or x.shape[0] == 0:
+        raise KernelError(f"linear_norm_ahead: x {tuple(x.shape)} does not match weight {tuple(weight.shape)}.")
+    m, k = x.shape
+    n = weight.shape[0]
+    _check(residual, "residual", dtype=torch.float32, shape=(m, n))
+    _check(norm_weight, "norm_weight", dtype=torch.bfloat16, shape=(n,))
+    if not can_prepare_norm(m, weight):
+        raise KernelError("linear_norm_ahead: this shape is not served by this library's product.")
+    groups = int(load().ms_gemm_skinny_groups(m, n))
+    weighted = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    squares = torch.empty((groups, m), dtype=torch.float32, device=x.device)
+    product_calls["skinny"] += 1
+    call("ms_gemm_skinny_norm_ahead", _ptr(x), _ptr(weight), _ptr(residual), m, n, k, _ptr(norm_weight),
+         _ptr(weighted), _ptr(squares), _stream())
+    return weighted, squares
+
+
+def linear_prepared(
+    weighted: torch.Tensor, squares: torch.Tensor, eps: float, weight: torch.Tensor, *, gated: bool = False
+) -> torch.Tensor:
+    """``RMSNorm(residual) @ weight^T`` (``gated``: then SiLU(gate) * up of the two halves)
+    from what :func:`linear_norm_ahead` left: the product of ``weighted`` with every sum
+    scaled by ``1 / sqrt(sum of the row's squares / K + eps)``."""
+
+    _check(weighted, "weighted", dtype=torch.bfloat16)
+    _check(weight, "weight", dtype=torch.bfloat16)
+    if weighted.ndim != 2 or weight.ndim != 2 or weighted.shape[1] != weight.shape[1] or weighted.shape[0] == 0:
+        raise KernelError(f"linear_prepared: x {tuple(weighted.shape)} does not match weight {tuple(weight.shape)}.")
+    m, k = weighted.shape
+    n = weight.shape[0]
+    if squares.ndim != 2 or squares.shape[0] == 0:
+        raise KernelError(f"linear_prepared: squares {tuple(squares.shape)} are not [groups, {m}].")
+    _check(squares, "squares", dtype=torch.float32, shape=(squares.shape[0], m))
+    if not can_use_prepared_norm(m, weight, gated=gated):
+        raise KernelError("linear_prepared: this shape is not served by this library's product.")
+    out = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=weighted.device)
+    product_calls["skinny"] += 1
+    call("ms_gemm_skinny_scaled", _ptr(weighted), _ptr(weight), _ptr(out), None, m, n, k,
+         _EPILOGUE_SILU_MUL if gated else _EPILOGUE_BF16, _ptr(squares), int(squares.shape[0]), float(eps), _stream())
     return out
 
 

@@ -35,6 +35,9 @@ _SIGNATURES: dict[str, list] = {
     "ms_gemm_f32": [_P, _P, _P, _I, _I, _I, _I, _P],
     "ms_gemm_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
     "ms_gemm_skinny_supported": [_I, _I, _I, _I],
+    "ms_gemm_skinny_groups": [_I, _I],
+    "ms_gemm_skinny_norm_ahead": [_P, _P, _P, _I, _I, _I, _P, _P, _P, _P],
+    "ms_gemm_skinny_scaled": [_P, _P, _P, _P, _I, _I, _I, _I, _P, _I, _F, _P],
     "ms_gemm_skinny_normed": [_P, _P, _F, _P, _P, _I, _I, _I, _I, _P],
     "ms_gemm_library_open": [c_char_p],
     "ms_gemm_library": [_P, _P, _P, _I, _I, _I, _I, _I, _P, c_size_t, _P],

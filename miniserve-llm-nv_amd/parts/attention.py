@@ -22,6 +22,7 @@ from .base import (
     PendingNorm,
     StepContext,
     WeightSpec,
+    add_output,
     build_part,
     register_part,
     release_tensors,
@@ -34,6 +35,7 @@ from .rotary import RotaryHalf
 class Attention(Part):
     accepts_pending_norm = True
     accumulates_residual = True
+    prepares_norm = True
 
     def __init__(self, spec: PartSpec, dtype: torch.dtype) -> None:
         params = require_params(spec, "hidden_size", "num_heads", "num_kv_heads", "head_dim")
@@ -123,10 +125,16 @@ class Attention(Part):
         release_tensors(tensors, names)       # the stacked copy serves from here on
 
     # -- execution ------------------------------------------------------------------
-    def forward(self, x, ctx: StepContext, cache: KVCacheView, *, residual: torch.Tensor | None = None):
-        """``x``: the normed input ``[N, H]``, or a ``PendingNorm`` (then the norm becomes
-        the prologue of the q/k/v product where one kernel serves the shape).  With
-        ``residual`` the output may be added into it (the product's epilogue); None is returned then."""
+    def takes_prepared_norm(self, rows: int) -> bool:
+        return ops.can_use_prepared_norm(rows, self.w_qkv)
+
+    def forward(self, x, ctx: StepContext, cache: KVCacheView, *, residual: torch.Tensor | None = None, norm_after=None):
+        """``x``: the normed input ``[N, H]``, or a ``PendingNorm`` (then the norm becomes a
+        part of the q/k/v product where one kernel serves the shape: scales prepared by
+        the part before, or the product's prologue).  With ``residual`` the output may be
+        added into it (the product's epilogue); None is returned then, or, with
+        ``norm_after`` (the RMSNorm taken of the residual stream next), what that epilogue
+        prepared of it."""
 
         if not isinstance(cache, KVCacheView):
             raise TypeError("attention needs a paged key/value cache.")
@@ -135,7 +143,9 @@ class Attention(Part):
         kv_heads = self.num_kv_heads if cache.write else 0
         w_in = self.w_qkv if cache.write else self.w_q
         if isinstance(x, PendingNorm):
-            if x.fusable and ops.can_fuse_norm(n, w_in):
+            if x.prepared is not None and ops.can_use_prepared_norm(n, w_in):
+                packed = ops.linear_prepared(x.prepared.weighted, x.prepared.squares, x.norm.eps, w_in)
+            elif x.fusable and ops.can_fuse_norm(n, w_in):
                 packed = ops.linear_normed(x.residual, x.norm.weight, x.norm.eps, w_in)
             else:
                 packed = ops.linear(x.materialize(), w_in)
@@ -171,10 +181,7 @@ class Attention(Part):
             max_context=ctx.max_context_len,
         )
         attended = attended.reshape(n, self.num_heads * self.head_dim)
-        if residual is not None and ops.can_accumulate(n, self.w_o):
-            ops.linear(attended, self.w_o, accumulate_into=residual)
-            return None
-        return ops.linear(attended, self.w_o)
+        return add_output(attended, self.w_o, residual, norm_after)
 
     def _prepare_unfused(self, packed, ctx, cache, group, kv_heads) -> torch.Tensor:
         """Norms and position encoding through their own parts, then the cache write."""

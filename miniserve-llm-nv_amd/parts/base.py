@@ -226,16 +226,35 @@ class StepContext:
 
 # ---- a norm that is not yet taken ------------------------------------------------------
 
+class PreparedNorm:
+    """What a part that added its output into the residual stream left for the RMSNorm
+    behind it (``ops.linear_norm_ahead``): ``weighted`` = the norm's weight times the new
+    residual values, rounded to the model's dtype, and ``squares``, partial sums of their
+    squares.  ``ops.linear_prepared`` makes a product of the norm from the two; the norm
+    itself can always still be taken from the residual stream."""
+
+    def __init__(self, norm, weighted: torch.Tensor, squares: torch.Tensor) -> None:
+        self.norm = norm
+        self.weighted = weighted
+        self.squares = squares
+
+
 class PendingNorm:
     """``norm(residual + delta)``, not yet computed.  A block hands it to a mixer or a
     feed-forward that sets ``accepts_pending_norm = True``; such a part may fuse the
     norm into its first product (when ``fusable``: an RMSNorm whose input is the bare
-    residual stream) or call :meth:`materialize` for the normed tensor.  Every other
-    part receives the materialised tensor."""
+    residual stream; ``prepared``: what the part before left for exactly this norm, or
+    None) or call :meth:`materialize` for the normed tensor.  Every other part receives
+    the materialised tensor."""
 
-    def __init__(self, norm, residual: torch.Tensor, delta: torch.Tensor | None) -> None:
+    def __init__(self, norm, residual: torch.Tensor, delta: "torch.Tensor | PreparedNorm | None") -> None:
         self.norm = norm
         self.residual = residual
+        self.prepared: PreparedNorm | None = None
+        if isinstance(delta, PreparedNorm):
+            # made for another norm than this one: the residual stream holds the sum all the same
+            self.prepared = delta if delta.norm is norm else None
+            delta = None
         self.delta = delta
         self._value: torch.Tensor | None = None
 
@@ -252,6 +271,25 @@ class PendingNorm:
             self._value = self.norm.add_forward(self.residual, self.delta)
             self.delta = None       # the sum has been stored into the residual stream
         return self._value
+
+
+def add_output(hidden: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor | None, norm_after=None):
+    """The last product of a mixer or feed-forward, ``hidden @ weight^T``.  Without
+    ``residual`` it is returned.  With it, the product is added into the residual stream
+    by its own epilogue where a kernel does that, and None is returned, or, when
+    ``norm_after`` is an RMSNorm with a weight and the kernel serves the shape, the
+    ``PreparedNorm`` that the same epilogue made for it."""
+
+    from .. import ops
+
+    rows = hidden.shape[0]
+    if residual is None or not ops.can_accumulate(rows, weight):
+        return ops.linear(hidden, weight)
+    norm_weight = getattr(norm_after, "weight", None)
+    if norm_weight is not None and hasattr(norm_after, "eps") and ops.can_prepare_norm(rows, weight):
+        return PreparedNorm(norm_after, *ops.linear_norm_ahead(hidden, weight, residual, norm_weight))
+    ops.linear(hidden, weight, accumulate_into=residual)
+    return None
 
 
 # ---- registries -------------------------------------------------------------------

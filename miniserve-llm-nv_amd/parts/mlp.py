@@ -9,7 +9,7 @@ import torch
 
 from .. import ops
 from ..config.model_spec import PartSpec
-from .base import Part, PendingNorm, StepContext, WeightSpec, register_part, release_tensors, require_params
+from .base import Part, PendingNorm, StepContext, add_output, WeightSpec, register_part, release_tensors, require_params
 
 # activation name -> (gated activation of a packed [N, 2 I] row, the same fused with the product)
 _ACTIVATIONS = {"silu": (ops.silu_mul, ops.linear_silu_mul)}
@@ -18,6 +18,7 @@ _ACTIVATIONS = {"silu": (ops.silu_mul, ops.linear_silu_mul)}
 class GatedMLP(Part):
     accepts_pending_norm = True
     accumulates_residual = True
+    prepares_norm = True
 
     def __init__(self, spec: PartSpec, dtype: torch.dtype) -> None:
         params = require_params(spec, "hidden_size", "intermediate_size", "activation")
@@ -48,22 +49,27 @@ class GatedMLP(Part):
         self.w_down = tensors[self.prefix + "down_proj.weight"]
         release_tensors(tensors, names)       # the stacked copy serves from here on
 
-    def forward(self, x, ctx: StepContext | None = None, *, residual: torch.Tensor | None = None):
-        """``x``: the normed input, or a ``PendingNorm`` (then the norm becomes the
-        prologue of the gate/up product where one kernel serves the shape).  With
-        ``residual`` the output may be added into it (the product's epilogue); None is returned then."""
+    def takes_prepared_norm(self, rows: int) -> bool:
+        return self._fused_with_norm and ops.can_use_prepared_norm(rows, self.w_gate_up, gated=True)
+
+    def forward(self, x, ctx: StepContext | None = None, *, residual: torch.Tensor | None = None, norm_after=None):
+        """``x``: the normed input, or a ``PendingNorm`` (then the norm becomes a part of the
+        gate/up product where one kernel serves the shape: scales prepared by the part
+        before, or the product's prologue).  With ``residual`` the output may be added
+        into it (the product's epilogue); None is returned then, or, with ``norm_after``
+        (the RMSNorm taken of the residual stream next), what that epilogue prepared of it."""
 
         if isinstance(x, PendingNorm):
-            if x.fusable and self._fused_with_norm and ops.can_fuse_norm(x.shape[0], self.w_gate_up, gated=True):
+            rows = x.shape[0]
+            if x.prepared is not None and self.takes_prepared_norm(rows):
+                hidden = ops.linear_prepared(x.prepared.weighted, x.prepared.squares, x.norm.eps, self.w_gate_up, gated=True)
+            elif x.fusable and self._fused_with_norm and ops.can_fuse_norm(rows, self.w_gate_up, gated=True):
                 hidden = ops.linear_normed(x.residual, x.norm.weight, x.norm.eps, self.w_gate_up, gated=True)
             else:
                 hidden = self._gated_product(x.materialize(), self.w_gate_up)
         else:
             hidden = self._gated_product(x, self.w_gate_up)
-        if residual is not None and ops.can_accumulate(hidden.shape[0], self.w_down):
-            ops.linear(hidden, self.w_down, accumulate_into=residual)
-            return None
-        return ops.linear(hidden, self.w_down)
+        return add_output(hidden, self.w_down, residual, norm_after)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

@@ -13,6 +13,7 @@ from ..config.model_spec import ModelSpec
 from .base import (
     KVCacheNeed,
     Part,
+    PreparedNorm,
     StateNeed,
     StepContext,
     WeightSpec,
@@ -116,9 +117,23 @@ class DecoderModel:
 
         residual = self.embedding.forward(ctx.token_ids, ctx)
         delta = None
+        rows = residual.shape[0]
         for index, call in enumerate(self.order):
-            residual, delta = self.layers[call.layer].forward(residual, delta, ctx, caches[index])
+            block = self.layers[call.layer]
+            # the norm that the next block takes first: this block's last part may prepare it
+            norm_after = None
+            if index + 1 < len(self.order) and getattr(block, "accepts_norm_after", False):
+                following = self.layers[self.order[index + 1].layer]
+                takes = getattr(following, "takes_prepared_norm", None)
+                if takes is not None and takes(rows):
+                    norm_after = getattr(following, "first_norm", None)
+            if norm_after is not None:
+                residual, delta = block.forward(residual, delta, ctx, caches[index], norm_after=norm_after)
+            else:
+                residual, delta = block.forward(residual, delta, ctx, caches[index])
         if logit_rows is None or logit_rows.numel() == 0:
             return None
+        if isinstance(delta, PreparedNorm):
+            delta = None            # the residual stream holds the sum
         normed = self.final_norm.add_forward(residual, delta, rows=logit_rows, write_back=False)
         return self.head.forward(normed)

@@ -1029,6 +1029,53 @@ def test_product_with_the_norm_as_its_prologue(ops, m, n, k):
     assert not ops.can_fuse_norm(m, weight.float())
 
 
+@pytest.mark.parametrize("m", [1, 7, 16, 17, 40, 64])
+@pytest.mark.parametrize("width,before,after", [(1024, 3072, 4096), (200, 96, 72), (4096, 1024, 6144), (5120, 64, 512),
+                                                (72, 2056, 5128)])
+def test_product_that_prepares_the_norm_behind_it(ops, m, width, before, after):
+    """``h += x W1^T`` that leaves, for the RMSNorm of the new h, the weighted values and
+    every workgroup's sum of squares; and the product of that norm made from the two.
+    The first is the plain += to the bit, its by-products are what torch makes of the
+    new h; the second is held against the norm and the product in float64 with nothing
+    rounded (bound as in the test below), and the gated form is the activation of the
+    plain one to the bit.  Widths with 13 to 512 workgroups of sums; 1 to 64 rows."""
+
+    x = rand(m, before, seed=m + before, dtype=torch.bfloat16)
+    w1 = rand(width, before, seed=width, dtype=torch.bfloat16, scale=0.05)
+    w2 = rand(after, width, seed=after + 1, dtype=torch.bfloat16, scale=0.05)
+    norm_weight = (1 + 0.1 * rand(width, seed=5)).to(torch.bfloat16)
+    start = rand(m, width, seed=3, scale=2.0)
+    with ops.forced_product("skinny"):
+        assert ops.can_prepare_norm(m, w1) and ops.can_use_prepared_norm(m, w2) and ops.can_use_prepared_norm(m, w2, gated=True)
+        plain = start.clone()
+        ops.linear(x, w1, accumulate_into=plain)
+        h = start.clone()
+        weighted, squares = ops.linear_norm_ahead(x, w1, h, norm_weight)
+        assert torch.equal(h, plain)
+        assert torch.equal(weighted, (norm_weight.float() * h).to(torch.bfloat16))
+        assert squares.shape == (ops.load().ms_gemm_skinny_groups(m, width), m)
+        torch.testing.assert_close(squares.double().sum(0), h.double().pow(2).sum(-1), atol=0, rtol=1e-6)
+        out = ops.linear_prepared(weighted, squares, 1e-5, w2)
+        wide = h.cpu().double()
+        inputs = wide / (wide.pow(2).mean(-1, keepdim=True) + 1e-5).sqrt() * norm_weight.cpu().double()
+        exact = inputs @ w2.cpu().double().T
+        deviation = 2**-8 / 3**0.5 * (inputs.pow(2) @ w2.cpu().double().pow(2).T).sqrt()
+        bound = 6 * deviation + 2**-8 * exact.abs() + 1e-6
+        ratio = ((out.cpu().double() - exact).abs() / bound).max()
+        assert float(ratio) <= 1.0, f"error / bound = {float(ratio):.2f}"
+        assert torch.equal(ops.linear_prepared(weighted, squares, 1e-5, w2, gated=True), ops.silu_mul(out))
+        # again into the same tensors, as a recorded step does: nothing is kept between calls
+        again = start.clone()
+        weighted_again, squares_again = ops.linear_norm_ahead(x, w1, again, norm_weight)
+        assert torch.equal(weighted_again, weighted) and torch.equal(squares_again, squares)
+    from miniserve_amd.ops import KernelError
+
+    with pytest.raises(KernelError, match="squares"):
+        ops.linear_prepared(weighted, squares[:, : m - 1] if m > 1 else squares[:0], 1e-5, w2)
+    with ops.forced_product("library"):
+        assert not ops.can_prepare_norm(m, w1) and not ops.can_use_prepared_norm(m, w2)
+
+
 @pytest.mark.parametrize("m", [1, 7, 16])
 @pytest.mark.parametrize("n,k", [(5128, 64), (6144, 2048), (5120, 4104)])
 def test_product_with_the_norm_as_its_prologue_against_many_rows(ops, m, n, k):

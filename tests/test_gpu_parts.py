@@ -265,3 +265,62 @@ def test_block_embedding_and_head(model, dtype):
     torch.testing.assert_close(logits.cpu().double(), y.double() @ matrix.T, atol=TOL[dtype], rtol=TOL[dtype])
     if config["tie_word_embeddings"]:
         assert head.weight.data_ptr() == embedding.weight.data_ptr()                   # the very same tensor
+
+
+def test_blocks_that_prepare_the_norm_behind_a_product(model, monkeypatch):
+    """bfloat16 and 30 rows, where the norm would be a kernel of its own: each product that
+    adds into the residual stream leaves the next norm prepared (between the parts of a
+    block, and for the block that follows when it is named), the product behind the norm
+    is made from that, and two blocks give what the plain implementation gives.  What was
+    prepared for another norm than the one that is taken is left alone."""
+
+    from miniserve_amd import ops
+    from miniserve_amd.parts import KVCacheView, PreparedNorm, build_block, build_part
+    from miniserve_amd.parts.base import load_part_weights
+
+    config, block_size, spec = model["config"], model["block"], model["spec"]
+    dtype = torch.bfloat16
+    device_weights = to_device(model["weights"], dtype)
+    weights = oracle_weights(model["weights"], dtype)
+    rows = 30
+    h = rand(rows, config["hidden_size"], seed=12).to(DEVICE)
+    layers = [build_block(spec.layers[index], dtype) for index in (0, 1)]
+    for layer in layers:
+        load_part_weights(layer, device_weights)
+    heads, dim = config["num_key_value_heads"], config["head_dim"]
+    caches = [KVCacheView(0, torch.zeros((4, heads, block_size, dim), dtype=dtype, device=DEVICE),
+                          torch.zeros((4, heads, dim, block_size), dtype=dtype, device=DEVICE), block_size) for _ in layers]
+    ctx, _ = step_context([rows], [0], block_size)
+    calls = {"made": 0, "used": 0}
+    make, use = ops.linear_norm_ahead, ops.linear_prepared
+
+    def counted(function, key):
+        def wrapper(*args, **kwargs):
+            calls[key] += 1
+            return function(*args, **kwargs)
+        return wrapper
+
+    monkeypatch.setattr(ops, "linear_norm_ahead", counted(make, "made"))
+    monkeypatch.setattr(ops, "linear_prepared", counted(use, "used"))
+    assert layers[1].takes_prepared_norm(rows) and not layers[1].takes_prepared_norm(8)   # few rows: the norm as prologue
+    expected = h.cpu().double()
+    for index in (0, 1):
+        expected, _ = plain.decoder_layer(expected, weights, index, config, torch.arange(rows))
+
+    residual, delta = layers[0].forward(h.clone(), None, ctx, caches[0], norm_after=layers[1].first_norm)
+    assert isinstance(delta, PreparedNorm) and delta.norm is layers[1].first_norm and calls == {"made": 2, "used": 1}
+    residual, delta = layers[1].forward(residual, delta, ctx, caches[1])
+    assert delta is None and calls == {"made": 3, "used": 3}
+    torch.testing.assert_close(residual.cpu().double(), expected, atol=TOL["bfloat16"], rtol=TOL["bfloat16"])
+    prepared_way = residual.clone()
+
+    # prepared for a norm that is not the one taken next: not used, and nothing is lost
+    other = build_part("norm", spec.layers[1].norms["pre_mixer"], dtype)
+    other.load_weights(device_weights)
+    residual, delta = layers[0].forward(h.clone(), None, ctx, caches[0], norm_after=other)
+    assert isinstance(delta, PreparedNorm) and delta.norm is other
+    residual, delta = layers[1].forward(residual, delta, ctx, caches[1])
+    assert calls == {"made": 6, "used": 5}
+    torch.testing.assert_close(residual.cpu().double(), expected, atol=TOL["bfloat16"], rtol=TOL["bfloat16"])
+    # the norm as a kernel of its own and as prepared scales differ by roundings alone
+    torch.testing.assert_close(residual, prepared_way, atol=TOL["bfloat16"], rtol=TOL["bfloat16"])
