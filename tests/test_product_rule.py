@@ -52,6 +52,47 @@ def test_the_norm_is_a_prologue_only_of_small_and_middle_matrices(monkeypatch):
         assert ops.can_fuse_norm(8, weight(10240, 5120))                # tests may still ask for the fused kernel
 
 
+def test_where_a_product_takes_a_norm_that_the_product_before_prepared(monkeypatch):
+    """A norm prepared by the product before it is taken where the norm would otherwise
+    be a kernel of its own and this library's product serves both: never where the
+    prologue form runs (few rows, small matrix), up to 8 rows against a large matrix, up
+    to 64 rows against a small one."""
+
+    import torch
+
+    from miniserve_amd import ops
+
+    class Library:
+        @staticmethod
+        def ms_gemm_skinny_supported(m, n, k, epilogue):
+            return 1
+
+    monkeypatch.setattr(ops, "load", lambda: Library)
+
+    def weight(n, k, dtype=torch.bfloat16):
+        return torch.empty((n, k), dtype=dtype, device="meta")
+
+    qkv, gate_up = weight(4096, 1024), weight(6144, 1024)               # 0.6B
+    for rows in (1, 8, 16):
+        assert not ops.can_use_prepared_norm(rows, qkv) and not ops.can_use_prepared_norm(rows, gate_up, gated=True)
+    for rows in (17, 40, 64):
+        assert ops.can_use_prepared_norm(rows, qkv) and ops.can_use_prepared_norm(rows, gate_up, gated=True)
+        assert ops.can_prepare_norm(rows, weight(1024, 2048)) and ops.can_prepare_norm(rows, weight(1024, 3072))
+    assert not ops.can_use_prepared_norm(65, qkv) and not ops.can_prepare_norm(65, weight(1024, 2048))
+    big = weight(24576, 4096)                                           # 8B, gate and up: 192 MiB
+    assert ops.can_use_prepared_norm(1, big, gated=True) and ops.can_use_prepared_norm(8, big, gated=True)
+    assert not ops.can_use_prepared_norm(9, big, gated=True) and not ops.can_use_prepared_norm(16, big, gated=True)
+    assert ops.can_use_prepared_norm(8, big)                             # the saved norm kernel pays for this library's product
+    assert ops.can_prepare_norm(8, weight(4096, 4096))                   # 8B, o: 32 MiB, this library's product
+    assert not ops.can_prepare_norm(8, weight(4096, 12288))              # 8B, down: the library's
+    assert not ops.can_use_prepared_norm(8, weight(51200, 5120), gated=True)    # 32B: the library's
+    assert not ops.can_use_prepared_norm(40, qkv.to(torch.float32)) and not ops.can_prepare_norm(40, weight(1024, 2048, torch.float32))
+    with ops.forced_product("skinny"):
+        assert ops.can_use_prepared_norm(8, qkv) and ops.can_use_prepared_norm(16, big)      # tests may ask for the kernel itself
+    with ops.forced_product("library"):
+        assert not ops.can_use_prepared_norm(40, qkv) and not ops.can_prepare_norm(40, weight(1024, 2048))
+
+
 def test_a_forced_product_overrides_the_rule_and_is_undone():
     from miniserve_amd import ops
 
