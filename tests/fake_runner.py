@@ -34,7 +34,9 @@ class FakeRunner:
         self.steps: list[list[tuple[str, int, int]]] = []     # per step: (request, start, end)
         self.fail_on_step = fail_on_step
         self.prepare_ahead = False          # tests switch it on
+        self.chain = False                  # tests switch it on: steps of single tokens are launched ahead
         self.prepared_ahead = self.used_ahead = self.discarded_ahead = self.prepared_mixed = 0
+        self.chained = self.voided_chained = 0
 
     def admit(self, request_id):
         self.tokens[request_id] = []
@@ -54,7 +56,19 @@ class FakeRunner:
             start = self.cache.committed_tokens(request_id)
             items.append(StepItem(request_id, start, start + 1))
         self.prepared_ahead += 1
-        return SimpleNamespace(request_ids=tuple(request_ids), reservation=self.cache.prepare_step(items))
+        prepared = SimpleNamespace(request_ids=tuple(request_ids), reservation=self.cache.prepare_step(items))
+        if self.chain:
+            prepared.launched = False
+        return prepared
+
+    def launch_chained(self, prepared, tokens):
+        """As the real runner's: the prepared step of single tokens runs now, on the tokens
+        that the "device" holds (``tokens.values``, which the host has not read yet)."""
+
+        assert not prepared.launched and tokens.is_cuda and len(tokens.values) >= len(prepared.request_ids)
+        prepared.launched = True
+        prepared.ran = tuple(int(token) for token in tokens.values[: len(prepared.request_ids)])
+        self.chained += 1
 
     def prepare_step(self, entries, admit=()):
         """As the real runner's: any other step's cache transaction, opened ahead; the
@@ -86,6 +100,7 @@ class FakeRunner:
 
     def discard(self, prepared):
         self.discarded_ahead += 1
+        self.voided_chained += bool(getattr(prepared, "launched", False))
         self.cache.abort_step(prepared.reservation)
         for request_id in getattr(prepared, "admitted", ()):
             self.release(request_id)
@@ -103,6 +118,9 @@ class FakeRunner:
                 assert all(entry.token_ids == prepared.known[entry.request_id] for entry in entries if len(entry.token_ids) > 1)
             else:
                 assert all(len(entry.token_ids) == 1 for entry in entries)
+            if getattr(prepared, "launched", False):
+                # what ran is what the engine now says the step is
+                assert tuple(entry.token_ids[0] for entry in entries) == prepared.ran
             reservation = prepared.reservation
             self.used_ahead += 1
         else:
@@ -126,20 +144,37 @@ class FakeRunner:
         return torch.stack(rows) if rows else None
 
 
+class DeviceTokens:
+    """Stands for the sampling kernel's output on the device: the engine may hand it to a
+    chained launch but reads token values only from what ``finish`` returns."""
+
+    is_cuda = True
+
+    def __init__(self, values):
+        self.values = values
+
+
 class ArgmaxSampler:
-    """Greedy on the host; the engine's sampler interface."""
+    """Greedy on the host; the engine's sampler interface.  ``on_device``: ``launch`` returns
+    its tokens as the real sampler does, as a tensor on the device, first."""
+
+    def __init__(self, on_device: bool = False) -> None:
+        self.on_device = on_device
 
     def stage(self, logits, requests):
         return self.finish(self.launch(logits, requests))
 
     def launch(self, logits, requests):
+        if self.on_device:
+            return DeviceTokens([int(torch.argmax(row)) for row in logits]), tuple(requests)
         return logits, tuple(requests)
 
     def finish(self, launched):
         from miniserve_amd.sampling import StagedSample
 
-        logits, requests = launched
-        return tuple(StagedSample(rid, int(torch.argmax(row)), None) for (rid, _), row in zip(requests, logits))
+        first, requests = launched
+        tokens = first.values if isinstance(first, DeviceTokens) else [int(torch.argmax(row)) for row in first]
+        return tuple(StagedSample(rid, token, None) for (rid, _), token in zip(requests, tokens))
 
     def commit(self, samples):
         pass

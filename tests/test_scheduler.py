@@ -413,6 +413,78 @@ def test_steps_planned_ahead_change_no_token():
     runner.cache.assert_invariants()
 
 
+def test_steps_launched_ahead_change_no_token():
+    """A step of single tokens that was planned ahead is launched before the host has read
+    the tokens it runs (they go from the sampling kernel to the step on the device).  The
+    requests generate what they generate without that, whatever voids such a step: a stop
+    token, a new request, a cancelled one, too few pages; and the tokens a launched step
+    ran are the tokens the engine later says it ran (the stand-in runner checks that)."""
+
+    def chained_engine(**options):
+        engine, runner = make_engine(**options)
+        engine.sampler = ArgmaxSampler(on_device=True)
+        runner.prepare_ahead = runner.chain = True
+        return engine, runner
+
+    params = SamplingParams(max_new_tokens=12)
+    expected = [expected_generation(p, 12, 97) for p in PROMPTS]
+    engine, runner = chained_engine()
+    assert engine.generate(PROMPTS, params) == expected
+    # (the step behind the prompts' step is planned ahead but not launched: its rows, longest context first,
+    # are not in the order in which that step sampled them)
+    assert runner.chained >= 8 and runner.chained == runner.used_ahead - 1 and runner.voided_chained == 0
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
+
+    # requests that end by length: the step after is planned, and launched, without them
+    lengths = (5, 12, 8, 10)
+    engine, runner = chained_engine()
+    got = engine.generate(PROMPTS, [SamplingParams(max_new_tokens=n) for n in lengths])
+    assert got == [tokens[:n] for tokens, n in zip(expected, lengths)]
+    # (the step behind one in which a request ends has other rows than that one sampled: planned, not launched)
+    assert runner.chained >= 6 and runner.voided_chained == 0 and runner.discarded_ahead == 0
+
+    # a stop token ends a request whose next token already runs: that step is thrown away
+    stop = expected[0][4]
+    engine, runner = chained_engine()
+    got = engine.generate(PROMPTS, [SamplingParams(max_new_tokens=12, stop_token_ids=(stop,))] + [params] * 3)
+    assert got[0] == expected[0][: expected[0].index(stop) + 1] and got[1:] == expected[1:]
+    assert runner.voided_chained >= 1 and runner.chained > runner.voided_chained
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
+    runner.cache.assert_invariants()
+
+    # a request that arrives, and one that is cancelled, while a launched step runs
+    engine, runner = chained_engine()
+    engine.add_request("a", PROMPTS[0], params, arrival_ns=0)
+    engine.add_request("b", PROMPTS[1], params, arrival_ns=1)
+    for _ in range(4):
+        engine.step()
+    assert runner.prepared_ahead == runner.used_ahead + 1 and runner.chained == 3     # one runs and has not been taken yet
+    engine.add_request("c", PROMPTS[3], params, arrival_ns=2)
+    engine.step()                                                      # the launched step did not know "c"
+    assert runner.voided_chained == 1
+    for _ in range(3):
+        engine.step()
+    engine.cancel("b")                                                 # its pages go back: the running step first
+    assert runner.voided_chained == 2
+    runner.cache.assert_invariants()
+    while engine.has_unfinished():
+        engine.step()
+    assert list(engine.pop_result("a").token_ids) == expected[0] and list(engine.pop_result("c").token_ids) == expected[3]
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
+
+    # so few pages that decoding requests are preempted
+    tight, runner = chained_engine(num_kv_blocks=14, enable_chunked_prefill=True, max_num_batched_tokens=64)
+    assert tight.generate(PROMPTS, params) == expected
+    assert tight.counters["preemptions"] > 0 and runner.chained > 0
+    assert runner.cache.capacity().free_blocks == (14,)
+    runner.cache.assert_invariants()
+
+    # tokens that the host holds (a sampler that returns them at once) are never chained
+    engine, runner = make_engine()
+    runner.prepare_ahead = runner.chain = True
+    assert engine.generate(PROMPTS, params) == expected and runner.chained == 0 and runner.used_ahead >= 8
+
+
 def test_steps_with_prompt_portions_are_planned_ahead_too():
     """Portions of prompts beside decode tokens: the step after is foreseen as well (a
     request that is admitted in it is admitted ahead), and the steps that run are the
