@@ -552,6 +552,69 @@ def test_steps_with_prompt_portions_are_planned_ahead_too():
         assert runner.cache.live_requests() == () and runner.used_ahead > 0
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_serving_never_changes_a_token(seed):
+    """Requests of random lengths arrive at random steps, some with stop tokens, some
+    cancelled on the way, on pools from roomy to so tight that requests are preempted,
+    with prompts whole or in portions, steps planned ahead or not and launched ahead or
+    not: every request that ends has generated exactly what its tokens determine, a
+    cancelled one a prefix of it; no page or slot is lost at any step or at the end."""
+
+    rng = random.Random(1000 + seed)
+    vocab = 97
+    blocks = rng.choice([12, 16, 24, 64])
+    options = dict(num_kv_blocks=blocks, max_num_seqs=rng.choice([2, 3, 4]))
+    if rng.random() < 0.6:
+        options.update(enable_chunked_prefill=True, prefill_chunk_size=rng.choice([3, 7, 16]),
+                       max_num_batched_tokens=rng.choice([8, 16, 48]))
+    engine, runner = make_engine(**options)
+    runner.prepare_ahead = rng.random() < 0.7
+    if runner.prepare_ahead and rng.random() < 0.7:
+        runner.chain = True
+        engine.sampler = ArgmaxSampler(on_device=True)
+    requests = {}
+    for index in range(rng.randrange(3, 9)):
+        # (a request never needs more pages than the pool has: 4 tokens a page)
+        prompt = [rng.randrange(vocab) for _ in range(rng.randrange(1, min(40, 4 * blocks - 24)))]
+        new_tokens = rng.randrange(1, 21)
+        whole = expected_generation(prompt, new_tokens, vocab)
+        stops = (whole[rng.randrange(len(whole))],) if rng.random() < 0.3 else ()
+        requests[f"r{index}"] = dict(
+            prompt=prompt, params=SamplingParams(max_new_tokens=new_tokens, stop_token_ids=stops),
+            expected=expected_generation(prompt, new_tokens, vocab, stop=stops), due=rng.randrange(0, 25),
+            cancel_at=rng.randrange(1, 40) if rng.random() < 0.2 else None)
+    pending = dict(requests)
+    cancelled = set()
+    step = 0
+    while pending or engine.has_unfinished():
+        for name, request in list(pending.items()):
+            if request["due"] <= step:
+                engine.add_request(name, request["prompt"], request["params"], arrival_ns=step * 100 + int(name[1:]))
+                del pending[name]
+        for name, request in requests.items():
+            if request["cancel_at"] == step and name in engine._sequences:
+                engine.cancel(name)
+                cancelled.add(name)
+        if engine.has_unfinished():
+            engine.step()
+        runner.cache.assert_invariants()
+        step += 1
+        assert step < 2000
+    for name, request in requests.items():
+        result = engine.pop_result(name)
+        got = list(result.token_ids)
+        if name in cancelled:
+            assert got == request["expected"][: len(got)] and len(got) < len(request["expected"])
+        else:
+            assert got == request["expected"], (name, result.finish_reason)
+            assert result.finish_reason == ("stop" if got[-1] in request["params"].stop_token_ids else "length")
+    capacity = runner.cache.capacity()
+    assert runner.cache.live_requests() == () and capacity.free_blocks == (blocks,)
+    assert capacity.free_slots == options["max_num_seqs"]
+    if runner.chain:
+        assert runner.chained >= runner.voided_chained
+
+
 def test_stop_tokens_and_per_request_parameters():
     engine, _ = make_engine()
     first = expected_generation(PROMPTS[0], 12, 97)
