@@ -136,3 +136,33 @@ def test_a_preempted_request_builds_its_state_again(toy, on_the_cpu):  # noqa: F
             row = toy_tests.toy_logits(weights, config, list(prompt) + wanted[:place])[-1]
             assert abs(float(row[tokens[place]] - row[wanted[place]])) < 1e-4
     tight.runner.cache.assert_invariants()
+
+
+# ---- the toy of test_gpu_toy_cache.py: planes of a mixer's own, pages and a state row at once, an embedding
+# ---- that reads the step's context, tables that a part asks for ------------------------------------------
+
+import test_gpu_toy_cache as latent_tests  # noqa: E402
+
+latent_toy = latent_tests.toy
+
+
+@pytest.fixture
+def gpu_names_mean_the_cpu(monkeypatch, on_the_cpu):
+    """The GPU tests name their device; here the name is taken to mean the CPU."""
+
+    from miniserve_amd.cache import CacheManager
+    from miniserve_amd.engine import ModelRunner
+
+    from_folder = ModelRunner.from_folder.__func__
+    monkeypatch.setattr(ModelRunner, "from_folder", classmethod(
+        lambda cls, folder, config, device="cpu": from_folder(cls, folder, config, device="cpu")))
+    allocate = CacheManager.allocate_storage
+    monkeypatch.setattr(CacheManager, "allocate_storage", lambda self, dtype, device: allocate(self, dtype, "cpu"))
+
+
+def test_the_latent_cache_is_laid_out_as_the_mixers_say(latent_toy, gpu_names_mean_the_cpu):
+    latent_tests.test_the_cache_is_laid_out_as_the_mixers_say(latent_toy)
+
+
+def test_the_latent_toy_steps_like_its_plain_form(latent_toy, gpu_names_mean_the_cpu):
+    latent_tests.test_the_toy_model_steps_like_its_plain_form(latent_toy, False)
