@@ -20,11 +20,11 @@ TOLERANCE = 2e-5
 LENGTHS = {"a": (45, 70, 33, 18, 64), "b": (41, 64, 57, 9), "c": (70, 37, 66, 40)}
 
 
-def make_runner(folder, block_size, num_blocks, **options):
+def make_runner(folder, block_size, num_blocks, dtype="float32", **options):
     from miniserve_amd.config import EngineConfig
     from miniserve_amd.engine import ModelRunner
 
-    config = EngineConfig(dtype="float32", kv_block_size=block_size, num_kv_blocks=num_blocks, max_num_seqs=8,
+    config = EngineConfig(dtype=dtype, kv_block_size=block_size, num_kv_blocks=num_blocks, max_num_seqs=8,
                           enable_chunked_prefill=True, decode_graphs=False, **options)
     runner = ModelRunner.from_folder(folder, config, device="cpu")
     for pool in (*runner.cache.key_pools, *runner.cache.value_pools):
@@ -79,6 +79,34 @@ def test_replay_shapes_on_the_cpu(name, fused, model_folders, monkeypatch, tmp_p
         # every norm but the first of a step (behind the embedding) and the final one is prepared
         assert taken["linear_norm_ahead"] > 0 and taken["linear_prepared"] == taken["linear_norm_ahead"]
         assert taken["linear_normed"] == 0 and taken["linear_prepared"] % (2 * layers - 1) == 0
+
+
+@pytest.mark.parametrize("name", ["a", "c"])
+def test_bfloat16_replay_on_the_cpu(name, model_folders, monkeypatch, tmp_path):
+    """The same in bfloat16 (weights, cache and the values between kernels; the residual
+    stream stays 32-bit): within three times what the reference's own rounding does to
+    these logits, as the GPU tests hold the kernels."""
+
+    from miniserve_amd.engine.replay import replay
+
+    torch_kernels.install(monkeypatch)
+    folder, block_size = model_folders[name]
+    config = read_config(folder)
+    weights = {key: tensor.to(torch.bfloat16).float() for key, tensor in read_weights(folder).items()}
+    requests = {f"r{i}": random_tokens(n, config["vocab_size"], 50 + i) for i, n in enumerate(LENGTHS[name][:3])}
+    exact = {rid: plain.forward_logits(weights, config, tokens).float() for rid, tokens in requests.items()}
+    yardstick = max(float((plain.forward_logits(weights, config, tokens, rd=torch.bfloat16).float() - exact[rid]).abs().max())
+                    for rid, tokens in requests.items())
+    for shape, steps in (("portions", shapes.portions(requests)), ("mixed", shapes.mixed(requests, seed=3))):
+        pages = -(-shapes.max_live_tokens(steps) // block_size)
+        runner = make_runner(folder, block_size, pages, dtype="bfloat16")
+        assert runner.cache.key_pools[0].dtype == torch.bfloat16
+        out = tmp_path / shape
+        replay(runner, shapes.to_lines(steps), out, report=io.StringIO())
+        got = shapes.collect(steps, out, config["vocab_size"])
+        worst = max(float((row - exact[rid][position]).abs().max()) for (rid, position), row in got.items())
+        assert worst <= 3 * yardstick, f"{shape}: {worst:.3e} > 3 x {yardstick:.3e}"
+        runner.cache.assert_invariants()
 
 
 def test_the_engine_generates_the_plain_implementations_tokens_on_a_tight_pool(model_folders, monkeypatch):
