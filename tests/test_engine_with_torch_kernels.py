@@ -141,3 +141,49 @@ def test_the_engine_generates_the_plain_implementations_tokens_on_a_tight_pool(m
             # the engine's token is the plain implementation's, or lies within rounding of it
             assert token == wanted or float(logits[place, wanted] - logits[place, token]) <= 2 * TOLERANCE
     assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (9,)
+
+
+def test_sampled_generation_through_the_entry_point(model_folders, monkeypatch):
+    """Temperature, top-k and top-p with a seed a request, through ``LLM.generate``: every
+    token is the plain sampler's for the plain implementation's logits and the request's
+    own stream of uniform numbers; a pool so tight that requests are preempted and run
+    again changes no token (a stream advances only with tokens that are kept)."""
+
+    import plain_sampling
+
+    from miniserve_amd.engine import SamplingParams
+    from miniserve_amd.entrypoint import LLM
+    from miniserve_amd.sampling import Sampler
+
+    torch_kernels.install(monkeypatch)
+    folder, block_size = model_folders["b"]
+    config, weights = read_config(folder), read_weights(folder)
+    prompts = [random_tokens(n, config["vocab_size"], 900 + n) for n in (14, 31, 22, 9)]
+    params = [SamplingParams(max_new_tokens=16, temperature=0.9, top_k=(0, 12, 0, 40)[i], top_p=(1.0, 0.9, 0.7, 1.0)[i], seed=70 + i)
+              for i in range(4)]
+    options = dict(dtype="float32", kv_block_size=block_size, max_num_seqs=4, decode_graphs=False, device="cpu")
+    roomy = LLM(str(folder), num_kv_blocks=40, **options)
+    tokens = roomy.generate(prompts, params)
+    for index, (prompt, generated) in enumerate(zip(prompts, tokens)):
+        logits = plain.forward_logits(weights, config, list(prompt) + generated[:-1]).float()[len(prompt) - 1 :]
+        stream = torch.Generator().manual_seed(70 + index)
+        for place, token in enumerate(generated):
+            uniform = Sampler.draw_uniform(stream)
+            p = params[index]
+            if plain_sampling.edge_distance(logits[place], p.temperature, p.top_k, p.top_p, uniform) > 1e-4:
+                assert token == plain_sampling.sample_row(logits[place], p.temperature, p.top_k, p.top_p, uniform), (index, place)
+    tight = LLM(str(folder), num_kv_blocks=-(-(31 + 16) // block_size) + 3, enable_chunked_prefill=True, **options)
+    again = tight.generate(prompts, params)
+    assert tight.engine.counters["preemptions"] > 0
+    for index, (first, second) in enumerate(zip(tokens, again)):
+        if first != second:
+            # torch's products on the CPU depend on the rows beside a row in the last bit: only a draw on an edge may differ
+            place = next(i for i, (a, b) in enumerate(zip(first, second)) if a != b)
+            logits = plain.forward_logits(weights, config, list(prompts[index]) + first[:place]).float()[-1]
+            stream = torch.Generator().manual_seed(70 + index)
+            for _ in range(place + 1):
+                uniform = Sampler.draw_uniform(stream)
+            p = params[index]
+            assert plain_sampling.edge_distance(logits, p.temperature, p.top_k, p.top_p, uniform) <= 1e-4
+    assert tight.runner.cache.live_requests() == ()
+    tight.runner.cache.assert_invariants()
