@@ -187,3 +187,32 @@ def test_sampled_generation_through_the_entry_point(model_folders, monkeypatch):
             assert plain_sampling.edge_distance(logits, p.temperature, p.top_k, p.top_p, uniform) <= 1e-4
     assert tight.runner.cache.live_requests() == ()
     tight.runner.cache.assert_invariants()
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_mixed_traces_on_the_cpu(seed, model_folders, monkeypatch, tmp_path):
+    """Ten more ways of mixing requests (who joins when, who sits a step out, portions of 2
+    to 21 tokens beside single tokens, two to four live at a time), each on a pool that
+    only just holds the live requests, alternating the tiny configurations and the way
+    the norms are taken: every position's logits are the plain implementation's."""
+
+    from miniserve_amd.engine.replay import replay
+
+    name = "abc"[seed % 3]
+    torch_kernels.install(monkeypatch, fused=(None, "prologue", "prepared")[(seed // 3) % 3])
+    folder, block_size = model_folders[name]
+    config, weights = read_config(folder), read_weights(folder)
+    lengths = [torch.randint(5, 90, (), generator=torch.Generator().manual_seed(seed * 31 + i)).item() for i in range(6)]
+    requests = {f"r{i}": random_tokens(n, config["vocab_size"], 200 + 10 * seed + i) for i, n in enumerate(lengths)}
+    exact = {rid: plain.forward_logits(weights, config, tokens).float() for rid, tokens in requests.items()}
+    steps = shapes.mixed(requests, seed=100 + seed, live_limit=2 + seed % 3, tail=3 + seed)
+    pages = -(-shapes.max_live_tokens(steps, block=block_size) // block_size)
+    runner = make_runner(folder, block_size, pages)
+    replay(runner, shapes.to_lines(steps), tmp_path, report=io.StringIO())
+    got = shapes.collect(steps, tmp_path, config["vocab_size"])
+    assert len(got) == sum(lengths)
+    for (rid, position), row in got.items():
+        error = float((row - exact[rid][position]).abs().max())
+        assert error <= TOLERANCE, f"seed {seed}: {rid} at {position}: {error:.3e}"
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (pages,)
+    runner.cache.assert_invariants()
