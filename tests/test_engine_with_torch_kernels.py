@@ -133,6 +133,7 @@ def test_the_engine_generates_the_plain_implementations_tokens_on_a_tight_pool(m
         assert steps < 1000
     results = [engine.pop_result(f"r{index}") for index in range(len(prompts))]
     assert sum(result.num_preemptions for result in results) >= 1
+    assert runner.prepared_mixed_steps > 0          # steps with prompt portions were planned, and their tensors built, a step ahead
     for prompt, result in zip(prompts, results):
         tokens = list(prompt) + list(result.token_ids)
         logits = plain.forward_logits(weights, config, tokens[:-1]).float()[len(prompt) - 1 :]
