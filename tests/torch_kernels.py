@@ -142,11 +142,61 @@ def sample_rows(logits, *, temperature=None, top_k=None, top_p=None, uniform=Non
     return torch.tensor(tokens, dtype=torch.int32)
 
 
-def install(monkeypatch, *, fused: str | None = None):
+class OnDevice(torch.Tensor):
+    """A CPU tensor that says it lives on the device: what the sampling stand-in returns
+    where recorded steps are played, so that the engine feeds it to the next step "on the
+    device" as it does with the kernel's output."""
+
+    @property
+    def is_cuda(self):
+        return True
+
+
+class Recording:
+    """Stands for ``torch.cuda.graph(graph, pool=...)``: while it is open, a model's forward
+    pass is not run but noted in ``graph``, with an output tensor of its own."""
+
+    current = None
+
+    def __init__(self, graph, pool=None):
+        self.graph = graph
+
+    def __enter__(self):
+        Recording.current = self.graph
+
+    def __exit__(self, *exc):
+        Recording.current = None
+
+
+class RecordedGraph:
+    """Stands for ``torch.cuda.CUDAGraph``: ``replay`` runs what was noted, on what the
+    step's tensors hold at that moment, into the same output tensors."""
+
+    def __init__(self):
+        self.calls = []
+
+    def replay(self):
+        for call in self.calls:
+            call()
+
+
+class PassedEvent:
+    def record(self):
+        pass
+
+    def synchronize(self):
+        pass
+
+
+def install(monkeypatch, *, fused: str | None = None, recordings: bool = False):
     """Puts the stand-ins in the kernels' places for one test and lets a runner stand on
     the CPU.  ``fused``: None, the parts take the plain calls; ``"prologue"``, every norm
     before a product is that product's prologue; ``"prepared"``, every norm behind a
-    product that adds into the residual stream is prepared by it."""
+    product that adds into the residual stream is prepared by it.  ``recordings``: the
+    runner may record decode steps; a recording is a note of the model's forward pass that
+    ``replay`` runs again (so everything around the recordings is the product's own: the
+    numbers of a step, block tables at their fixed widths, spare rows, the two host
+    buffers, steps launched behind the sampling "on the device")."""
 
     import miniserve_amd.engine.runner as runner_module
     import miniserve_amd.parts.mlp as mlp_module
@@ -166,3 +216,32 @@ def install(monkeypatch, *, fused: str | None = None):
     monkeypatch.setattr(runner_module, "_require_gpu", lambda device: None)
     # (the feed-forward keeps its activation's two kernels by name)
     monkeypatch.setitem(mlp_module._ACTIVATIONS, "silu", (silu_mul, linear_silu_mul))
+    if not recordings:
+        return
+    from miniserve_amd.parts import DecoderModel
+    from miniserve_amd.sampling import Sampler
+
+    forward = DecoderModel.forward
+
+    def noted_forward(self, ctx, caches, logit_rows):
+        graph = Recording.current
+        if graph is None:
+            return forward(self, ctx, caches, logit_rows)
+        output = torch.zeros((logit_rows.numel(), self.spec.vocab_size), dtype=torch.float32)
+
+        def again():
+            ctx.scratch.clear()             # what a step shares between layers is made again in every replay
+            output.copy_(forward(self, ctx, caches, logit_rows))
+
+        graph.calls.append(again)
+        return output
+
+    monkeypatch.setattr(DecoderModel, "forward", noted_forward)
+    monkeypatch.setattr(torch.cuda, "CUDAGraph", RecordedGraph)
+    monkeypatch.setattr(torch.cuda, "graph", Recording)
+    monkeypatch.setattr(torch.cuda, "graph_pool_handle", lambda: None)
+    monkeypatch.setattr(torch.cuda, "synchronize", lambda device=None: None)
+    monkeypatch.setattr(torch.cuda, "Event", PassedEvent)
+    monkeypatch.setattr(torch.Tensor, "pin_memory", lambda self: self)
+    monkeypatch.setattr(Sampler, "_token_buffer", lambda self, rows: torch.empty(rows, dtype=torch.int32))
+    monkeypatch.setattr(ops, "sample_rows", lambda *args, **kwargs: sample_rows(*args, **kwargs).as_subclass(OnDevice))
