@@ -315,21 +315,28 @@ class Engine:
 
     def _launch_chained(self, ahead: "_StepAhead | None", sampled: Sequence[SequenceState], launched) -> None:
         """A recorded step of single tokens that was planned ahead is launched at once,
-        behind the running step, when its rows are the requests that the running step
-        samples, in that order: the sampling kernel's tokens go into its token ids on the
-        device, and the GPU does not wait while the host reads them and advances the
-        requests.  Should a request of it turn out to have ended (a stop token), or the set
-        of requests change before the next call, the step is thrown away like any step
-        planned ahead; it has then run for nothing."""
+        behind the running step, when each of its rows is a request that the running step
+        samples: the sampling kernel's tokens go into its token ids on the device (row by
+        row, or through a map of rows when a request of the running step ends by length
+        now or the order differs), and the GPU does not wait while the host reads them and
+        advances the requests.  Should a request of it turn out to have ended (a stop
+        token), or the set of requests change before the next call, the step is thrown
+        away like any step planned ahead; it has then run for nothing."""
 
         launch = getattr(self.runner, "launch_chained", None)
         if ahead is None or launch is None or ahead.plan.prefill_items or not hasattr(ahead.prepared, "launched"):
             return
         tokens = launched[0]
-        rows = tuple(item.request_id for item in _longest_first(ahead.plan.decode_items))
-        if rows != tuple(state.request_id for state in sampled) or not getattr(tokens, "is_cuda", False):
+        if not getattr(tokens, "is_cuda", False):
             return
-        launch(ahead.prepared, tokens)
+        rows = [item.request_id for item in _longest_first(ahead.plan.decode_items)]
+        sampled_ids = [state.request_id for state in sampled]
+        if rows == sampled_ids:
+            launch(ahead.prepared, tokens)
+            return
+        place = {request_id: row for row, request_id in enumerate(sampled_ids)}
+        if all(request_id in place for request_id in rows):
+            launch(ahead.prepared, tokens, [place[request_id] for request_id in rows])
 
     def _finalize(self, state: SequenceState) -> None:
         """A request that ended gives back its pages, its state slot and its random stream."""

@@ -95,6 +95,8 @@ class DecodeGraph:
         sizes += [(f"part:{name}", values.size) for name, values in part_tables.items()]
         for group in range(groups):
             sizes += [(f"slots{group}", batch), (f"table{group}", batch * widths[group])]
+        # for a step launched behind the sampling of the step before: which of that step's rows each row continues
+        sizes += [("token_rows", batch)]
         self.offsets: dict[str, tuple[int, int]] = {}
         total = 0
         for name, size in sizes:
@@ -247,18 +249,27 @@ class DecodeGraph:
         self.replays += 1
         return self.logits[: len(entries)]
 
-    def launch_chained(self, which: int, tokens: torch.Tensor, count: int) -> None:
+    def launch_chained(self, which: int, tokens: torch.Tensor, count: int, source_rows: Sequence[int] | None = None) -> None:
         """Replays the step whose numbers :meth:`prepare` wrote into host buffer ``which``
         with the token ids of its first ``count`` rows taken from ``tokens`` (int32, on
-        the device: what the sampling kernel of the step before chose, in row order)
-        instead of from the host, which has not read them yet.  Rows that only fill the
-        step up keep the ids they had (any id inside the vocabulary serves them)."""
+        the device: what the sampling kernel of the step before chose) instead of from the
+        host, which has not read them yet: row ``i`` runs ``tokens[i]``, or
+        ``tokens[source_rows[i]]`` when the step before had other rows or another order
+        (a request of it has ended, say).  Rows that only fill the step up keep the ids
+        they had (any id inside the vocabulary serves them)."""
 
         start, size = self.offsets["token_ids"]
         if start != 0 or self.graph is None:
             raise RuntimeError("a chained step needs its recording, and the token ids at the front of its numbers.")
+        if source_rows is not None:
+            # the map goes to the device with the step's other numbers, in the same copy
+            map_start, _ = self.offsets["token_rows"]
+            self.hosts_np[which][map_start : map_start + count] = source_rows
         self.meta[size:].copy_(self.hosts[which][size:], non_blocking=True)
-        self.meta[:count].copy_(tokens[:count])
+        if source_rows is None:
+            self.meta[:count].copy_(tokens[:count])
+        else:
+            self.meta[:count].copy_(torch.index_select(tokens, 0, self.meta[map_start : map_start + count]))
         self.graph.replay()
         self.replays += 1
 
@@ -339,6 +350,7 @@ class ModelRunner:
         self.prepared_mixed_steps = 0  # those of them that are not recorded steps
         self.chained_steps = 0         # recorded steps launched before the host had read the tokens they run
         self.voided_chained_steps = 0  # those of them that were thrown away (a request of theirs had ended)
+        self.mapped_chained_steps = 0  # those of them whose tokens were taken through a map of rows
 
     # ---- construction -----------------------------------------------------------------
     @classmethod
@@ -473,24 +485,32 @@ class ModelRunner:
         return PreparedStep(tuple(entry.request_id for entry in entries), reservation, built, tuple(admitted))
 
     @torch.inference_mode()
-    def launch_chained(self, prepared: "PreparedDecode", tokens: torch.Tensor) -> None:
+    def launch_chained(self, prepared: "PreparedDecode", tokens: torch.Tensor, source_rows: Sequence[int] | None = None) -> None:
         """Launches the prepared step of single tokens now, behind the step that is still
         running: row ``i`` runs ``tokens[i]`` (int32 on the device, the sampling kernel's
-        output of the running step, whose rows are this step's requests in this order).
-        The host reads those tokens afterwards; :meth:`step` with this ``prepared`` then
-        launches nothing and returns the logits, and :meth:`discard` throws the step away
-        (it is a transaction like any other: what it wrote lies above the committed
-        lengths, its pages and state rows go back)."""
+        output of the running step), or ``tokens[source_rows[i]]`` when the running step's
+        rows are not this step's requests in this order.  The host reads those tokens
+        afterwards; :meth:`step` with this ``prepared`` then launches nothing and returns
+        the logits, and :meth:`discard` throws the step away (it is a transaction like any
+        other: what it wrote lies above the committed lengths, its pages and state rows go
+        back)."""
 
         if prepared.launched:
             raise RuntimeError("the step runs already.")
-        if tokens.dtype != torch.int32 or tokens.ndim != 1 or tokens.numel() < len(prepared.request_ids) or not tokens.is_cuda:
+        rows = len(prepared.request_ids)
+        if tokens.dtype != torch.int32 or tokens.ndim != 1 or not tokens.is_cuda:
             raise ValueError("a chained step takes the device's int32 tokens, one a request.")
+        if source_rows is None:
+            if tokens.numel() < rows:
+                raise ValueError("a chained step takes the device's int32 tokens, one a request.")
+        elif len(source_rows) != rows or any(not 0 <= row < tokens.numel() for row in source_rows):
+            raise ValueError("a chained step's row map names one row of the tokens for each of its requests.")
         metas = prepared.reservation.sequences
         graph = self._decode_graphs[self._recorded_step_key(len(metas), max(meta.after for meta in metas))]
-        graph.launch_chained(prepared.buffer, tokens, len(metas))
+        graph.launch_chained(prepared.buffer, tokens, len(metas), source_rows)
         prepared.launched = True
         self.chained_steps += 1
+        self.mapped_chained_steps += source_rows is not None
 
     def discard(self, prepared: "PreparedDecode | PreparedStep") -> None:
         """Gives back what :meth:`prepare_decode` or :meth:`prepare_step` took."""

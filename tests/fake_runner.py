@@ -36,7 +36,7 @@ class FakeRunner:
         self.prepare_ahead = False          # tests switch it on
         self.chain = False                  # tests switch it on: steps of single tokens are launched ahead
         self.prepared_ahead = self.used_ahead = self.discarded_ahead = self.prepared_mixed = 0
-        self.chained = self.voided_chained = 0
+        self.chained = self.voided_chained = self.mapped = 0
 
     def admit(self, request_id):
         self.tokens[request_id] = []
@@ -61,13 +61,21 @@ class FakeRunner:
             prepared.launched = False
         return prepared
 
-    def launch_chained(self, prepared, tokens):
+    def launch_chained(self, prepared, tokens, source_rows=None):
         """As the real runner's: the prepared step of single tokens runs now, on the tokens
-        that the "device" holds (``tokens.values``, which the host has not read yet)."""
+        that the "device" holds (``tokens.values``, which the host has not read yet), row
+        by row or through the map of rows."""
 
-        assert not prepared.launched and tokens.is_cuda and len(tokens.values) >= len(prepared.request_ids)
+        assert not prepared.launched and tokens.is_cuda
+        rows = len(prepared.request_ids)
+        if source_rows is None:
+            assert len(tokens.values) >= rows
+            source_rows = range(rows)
+        else:
+            assert len(source_rows) == rows and list(source_rows) != list(range(rows)) or len(tokens.values) != rows
+            self.mapped += 1
         prepared.launched = True
-        prepared.ran = tuple(int(token) for token in tokens.values[: len(prepared.request_ids)])
+        prepared.ran = tuple(int(tokens.values[row]) for row in source_rows)
         self.chained += 1
 
     def prepare_step(self, entries, admit=()):

@@ -88,6 +88,45 @@ def test_preempted_requests_under_recorded_steps_planned_and_launched_ahead(mode
         assert [int(row.argmax()) for row in got] == list(result.token_ids)
 
 
+def test_requests_that_end_by_length_do_not_break_the_chain(model_folders, recordings):
+    """Eight requests on a roomy pool, three of which end early by length: the step behind
+    one in which a request ends has fewer rows than that one sampled, and is still
+    launched ahead, its tokens taken through a map of rows (eight, seven, six and five
+    rows share the recording of eight).  Every token was chosen from the plain
+    implementation's logits for the tokens before it."""
+
+    from miniserve_amd.config import EngineConfig
+    from miniserve_amd.engine import Engine, ModelRunner, SamplingParams
+
+    folder, block = model_folders["c"]
+    config, weights = read_config(folder), read_weights(folder)
+    prompts = [random_tokens(n, config["vocab_size"], 800 + n) for n in (12, 30, 21, 44, 9, 17, 26, 35)]
+    lengths = (6, 20, 9, 20, 13, 20, 20, 20)
+    runner = ModelRunner.from_folder(folder, EngineConfig(dtype="float32", kv_block_size=block, num_kv_blocks=40, max_num_seqs=8),
+                                     device="cpu")
+    sampler = keeping_sampler()
+    engine = Engine(runner, sampler=sampler)
+    for index, prompt in enumerate(prompts):
+        engine.add_request(f"r{index}", prompt, SamplingParams(max_new_tokens=lengths[index]), arrival_ns=index)
+    while engine.has_unfinished():
+        engine.step()
+        runner.cache.assert_invariants()
+    # 19 decode steps behind the prompts' step; the first makes the recording, the others are launched ahead,
+    # three of them (behind the steps in which r0, r2 and r4 end) through a map of rows
+    assert sorted(runner._decode_graphs) == [(8, 256)]
+    assert runner.graph_steps == 19 and runner.chained_steps == 18 and runner.mapped_chained_steps == 3
+    assert runner.voided_chained_steps == 0
+    for index, prompt in enumerate(prompts):
+        result = engine.pop_result(f"r{index}")
+        assert result.finish_reason == "length" and len(result.token_ids) == lengths[index]
+        tokens = list(prompt) + list(result.token_ids[:-1])
+        exact = plain.forward_logits(weights, config, tokens).float()[len(prompt) - 1 :]
+        got = torch.stack(sampler.kept[f"r{index}"])
+        assert float((got - exact).abs().max()) <= TOLERANCE
+        assert [int(row.argmax()) for row in got] == list(result.token_ids)
+    assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (40,)
+
+
 def test_a_stop_token_throws_the_step_that_was_launched_ahead_away(model_folders, recordings):
     from miniserve_amd.config import EngineConfig
     from miniserve_amd.engine import Engine, ModelRunner, SamplingParams

@@ -430,9 +430,9 @@ def test_steps_launched_ahead_change_no_token():
     expected = [expected_generation(p, 12, 97) for p in PROMPTS]
     engine, runner = chained_engine()
     assert engine.generate(PROMPTS, params) == expected
-    # (the step behind the prompts' step is planned ahead but not launched: its rows, longest context first,
-    # are not in the order in which that step sampled them)
-    assert runner.chained >= 8 and runner.chained == runner.used_ahead - 1 and runner.voided_chained == 0
+    # (the step behind the prompts' step runs its rows longest context first, not in the order in which that step
+    # sampled them: its tokens are taken through a map of rows)
+    assert runner.chained >= 8 and runner.chained == runner.used_ahead and runner.voided_chained == 0 and runner.mapped == 1
     assert runner.cache.live_requests() == () and runner.cache.capacity().free_blocks == (64,)
 
     # requests that end by length: the step after is planned, and launched, without them
@@ -440,8 +440,9 @@ def test_steps_launched_ahead_change_no_token():
     engine, runner = chained_engine()
     got = engine.generate(PROMPTS, [SamplingParams(max_new_tokens=n) for n in lengths])
     assert got == [tokens[:n] for tokens, n in zip(expected, lengths)]
-    # (the step behind one in which a request ends has other rows than that one sampled: planned, not launched)
-    assert runner.chained >= 6 and runner.voided_chained == 0 and runner.discarded_ahead == 0
+    # (the step behind one in which a request ends by length has fewer rows than that one sampled: a map of rows again)
+    assert runner.chained == runner.used_ahead >= 9 and runner.mapped == 4
+    assert runner.voided_chained == 0 and runner.discarded_ahead == 0
 
     # a stop token ends a request whose next token already runs: that step is thrown away
     stop = expected[0][4]
@@ -458,7 +459,7 @@ def test_steps_launched_ahead_change_no_token():
     engine.add_request("b", PROMPTS[1], params, arrival_ns=1)
     for _ in range(4):
         engine.step()
-    assert runner.prepared_ahead == runner.used_ahead + 1 and runner.chained == 3     # one runs and has not been taken yet
+    assert runner.prepared_ahead == runner.used_ahead + 1 and runner.chained == 4     # one runs and has not been taken yet
     engine.add_request("c", PROMPTS[3], params, arrival_ns=2)
     engine.step()                                                      # the launched step did not know "c"
     assert runner.voided_chained == 1
