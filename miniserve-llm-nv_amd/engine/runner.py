@@ -269,7 +269,7 @@ class DecodeGraph:
         if source_rows is None:
             self.meta[:count].copy_(tokens[:count])
         else:
-            self.meta[:count].copy_(torch.index_select(tokens, 0, self.meta[map_start : map_start + count]))
+            self.meta[:count].copy_(torch.index_select(tokens, 0, self.meta[map_start : map_start + count].long()))
         self.graph.replay()
         self.replays += 1
 
