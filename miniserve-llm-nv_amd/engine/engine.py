@@ -331,8 +331,8 @@ class Engine:
             return
         rows = [item.request_id for item in _longest_first(ahead.plan.decode_items)]
         sampled_ids = [state.request_id for state in sampled]
-        if rows == sampled_ids:
-            launch(ahead.prepared, tokens)
+        if rows == sampled_ids[: len(rows)]:
+            launch(ahead.prepared, tokens)          # the same rows, or the first of them (the last ones end now)
             return
         place = {request_id: row for row, request_id in enumerate(sampled_ids)}
         if all(request_id in place for request_id in rows):

@@ -73,8 +73,8 @@ class FakeRunner:
             source_rows = range(rows)
         else:
             assert len(source_rows) == rows and all(0 <= row < len(tokens.values) for row in source_rows)
-            # (a map comes only when it is needed: other rows than the sampled ones, or another order)
-            assert list(source_rows) != list(range(rows)) or len(tokens.values) != rows
+            # (a map comes only when it is needed: the rows are not the first of the sampled ones in their order)
+            assert list(source_rows) != list(range(rows))
             self.mapped += 1
         prepared.launched = True
         prepared.ran = tuple(int(tokens.values[row]) for row in source_rows)

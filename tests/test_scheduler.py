@@ -440,8 +440,9 @@ def test_steps_launched_ahead_change_no_token():
     engine, runner = chained_engine()
     got = engine.generate(PROMPTS, [SamplingParams(max_new_tokens=n) for n in lengths])
     assert got == [tokens[:n] for tokens, n in zip(expected, lengths)]
-    # (the step behind one in which a request ends by length has fewer rows than that one sampled: a map of rows again)
-    assert runner.chained == runner.used_ahead >= 9 and runner.mapped == 4
+    # (the step behind one in which a request ends by length has fewer rows than that one sampled: a map of rows again,
+    # unless the request that ends held the last row)
+    assert runner.chained == runner.used_ahead >= 9 and runner.mapped == 3
     assert runner.voided_chained == 0 and runner.discarded_ahead == 0
 
     # a stop token ends a request whose next token already runs: that step is thrown away
