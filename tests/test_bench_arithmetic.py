@@ -71,3 +71,36 @@ def test_the_numbers_of_the_headline_configuration():
 def test_more_than_one_gpu_is_refused_with_one_line_and_code_2():
     done = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert done.returncode == 2 and len(done.stdout.strip().splitlines()) == 1 and "--gpus 2" in done.stdout
+
+
+def test_a_kernel_trace_is_accounted_step_by_step(tmp_path, capsys):
+    """``--account-trace`` on a made-up trace: a step begins with the embedding kernel, decode steps are those
+    of the most frequent kernel count without the first four, medians a kernel."""
+
+    import bench
+
+    rows, clock = ["Kernel_Name,Start_Timestamp,End_Timestamp"], 0
+
+    def kernel(name, us):
+        nonlocal clock
+        rows.append(f'"{name}",{clock},{clock + int(us * 1000)}')
+        clock += int(us * 1000) + 2000
+
+    for step in range(10):                                           # ten decode steps of 1 + 2 * 3 kernels
+        kernel("void (anonymous namespace)::embedding_gather_kernel<ms::bf16>(int const*)", 3)
+        for _ in range(2):
+            kernel("void (anonymous namespace)::gemm_skinny_kernel<1, 1, false, 8, false>(ms::bf16 const*)", 5)
+            kernel("void (anonymous namespace)::attention_decode_kernel<128>(ms::bf16 const*)", 17 if step != 7 else 40)
+            kernel("Cijk_Alik_Bljk_BBS_BH_MT16x16x512_MI16x16x1_SN_K1", 21)
+    for _ in range(3):                                               # three prefill steps
+        kernel("void (anonymous namespace)::embedding_gather_kernel<ms::bf16>(int const*)", 9)
+        kernel("void (anonymous namespace)::attention_prefill_kernel<128, 2, 2>(ms::bf16 const*)", 43)
+    path = tmp_path / "p_kernel_trace.csv"
+    path.write_text("\n".join(rows) + "\n")
+    bench.account_trace(str(path))
+    out = capsys.readouterr().out
+    assert "decode step: 6 steps, 7 kernels a step; kernel time 89.0 us" in out
+    assert "attention_decode_kernel<128>" in out and "hipBLASLt MT16x16x512" in out and "gemm_skinny_kernel<1, 1, false, 8, false>" in out
+    line = next(text for text in out.splitlines() if text.startswith("attention_decode_kernel<128>"))
+    assert line.split()[-4:] == ["2", "34.0", "17.00", "6"]          # calls, us a step (median: the slow step does not move it), average, steps
+    assert "prefill step: 3 steps, 2 kernels a step; kernel time 52.0 us" in out
