@@ -16,7 +16,7 @@ from .batch import StepEntry
 from .plan import ExecutionPlan
 from .request import Request, SamplingParams
 from .scheduler import Scheduler
-from .sequence import TERMINAL, RequestStatus, SequenceState, SequenceView
+from .sequence import TERMINAL, RequestStatus, SequenceState
 
 
 @dataclass(frozen=True)

@@ -4,7 +4,6 @@ weights in a temporary place, and replay shapes."""
 from __future__ import annotations
 
 import json
-import os
 import sys
 from pathlib import Path
 

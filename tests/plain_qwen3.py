@@ -9,7 +9,6 @@ so that differences to an engine in float32 are the engine's rounding alone).
 
 from __future__ import annotations
 
-import math
 
 import torch
 

@@ -6,7 +6,6 @@ again - in 32-bit and in bfloat16, for every tiny configuration."""
 from __future__ import annotations
 
 import io
-import os
 import subprocess
 import sys
 from pathlib import Path
