@@ -33,7 +33,6 @@ using ms::bf16x8;
 using ms::floatx16;
 using ms::kTileKeys;
 
-constexpr int kTileTokens = 64;       // query tokens of a workgroup at most
 constexpr int kXcds = 8;    // dies of the chip, each with an L2 of its own (a wrong number costs speed only)
 constexpr int kWaveColumns = 32;      // columns (token, head) of one wave
 

@@ -165,10 +165,6 @@ __device__ __forceinline__ void unpack8(const uint4& raw, float out[8]) {
   }
 }
 
-__device__ __forceinline__ void load8(const ms::bf16* src, float out[8]) {
-  unpack8(*reinterpret_cast<const uint4*>(src), out);
-}
-
 __device__ __forceinline__ void load8(const float* src, float out[8]) {
   const float4 a = *reinterpret_cast<const float4*>(src);
   const float4 b = *reinterpret_cast<const float4*>(src + 4);
